@@ -1,0 +1,229 @@
+"""Bookkeeping of everything a request keeps between steps: pages of keys and values,
+one block table per request and cache group, and a slot for state of fixed size.
+
+Host-side only (no tensors), so it is tested without a GPU; `storage.py` holds the device
+memory the ids refer to.
+
+Layers with the same needs (same KV heads, head size and window) form a *group*: one page
+pool, one allocator, one block table per request.  Position p of a request lives in page
+`table[p // block_size]` at offset `p % block_size` (src/llmserve/kvcache/paged.py:196-197).
+Pages come back when the request ends, or, in a windowed group, as soon as every later
+query is out of their reach; a returned entry of the table becomes -1.
+
+`append` is atomic like the reference's `build_batch` (src/llmserve/kvcache/paged.py:174-200):
+it first sums what the whole step needs over all groups and raises `OutOfBlocks` before
+changing anything; on success the lengths advance at once.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+from ..parts.spec import PagedCacheSpec, StateCacheSpec
+from .allocator import BlockAllocator, OutOfBlocks
+
+
+@dataclass(frozen=True)
+class CacheGroup:
+    group_id: int
+    spec: PagedCacheSpec | StateCacheSpec
+    layers: tuple[int, ...]  # layers that own storage in this group, in order
+
+    @property
+    def paged(self) -> bool:
+        return isinstance(self.spec, PagedCacheSpec)
+
+
+def group_layers(cache_specs: list[PagedCacheSpec | StateCacheSpec | None]) -> list[CacheGroup]:
+    """Groups for a list of per-layer needs (None: the layer keeps nothing of its own)."""
+    by_spec: dict = {}
+    for layer, spec in enumerate(cache_specs):
+        if spec is not None:
+            by_spec.setdefault(spec, []).append(layer)
+    return [CacheGroup(g, spec, tuple(layers)) for g, (spec, layers) in enumerate(by_spec.items())]
+
+
+@dataclass
+class StepLayout:
+    """What `append` decided for one step (host lists, in the order of the step's requests)."""
+
+    seq_ids: list
+    counts: list[int]
+    starts: list[int]  # length of each request before the step
+    state_slots: list[int]
+    fresh_slots: list[int]  # slots whose state must be cleared before this step runs
+    slots: dict[int, list[int]] = field(default_factory=dict)  # group -> cache slot of every new token
+    tables: dict[int, list[list[int]]] = field(default_factory=dict)  # group -> block table per request
+
+
+class CacheManager:
+    def __init__(self, groups: list[CacheGroup], num_blocks: int, block_size: int, max_seqs: int):
+        if block_size < 1 or max_seqs < 1:
+            raise ValueError("block_size and max_seqs must be >= 1")
+        self.groups = list(groups)
+        self.paged_groups = [g for g in self.groups if g.paged]
+        self.num_blocks = num_blocks
+        self.block_size = block_size
+        self.max_seqs = max_seqs
+        self.allocators = {g.group_id: BlockAllocator(num_blocks) for g in self.paged_groups}
+        self.tables: dict[int, dict] = {g.group_id: {} for g in self.paged_groups}
+        self.lengths: dict = {}
+        self.slot_of: dict = {}
+        self._slot_alloc = BlockAllocator(max_seqs)
+        self._fresh: set[int] = set()
+
+    # ---- sizes ------------------------------------------------------------------------
+    def blocks_for(self, n_tokens: int) -> int:
+        return -(-n_tokens // self.block_size)
+
+    @property
+    def num_free_blocks(self) -> int:
+        """Free pages of the tightest group (every group must fit a request)."""
+        if not self.allocators:
+            return self.num_blocks
+        return min(a.num_free for a in self.allocators.values())
+
+    @property
+    def num_free_slots(self) -> int:
+        return self._slot_alloc.num_free
+
+    def utilization(self) -> float:
+        """Fraction of pages in use (src/llmserve/kvcache/paged.py:145-147), fullest group."""
+        if not self.allocators:
+            return 0.0
+        return max(a.num_used for a in self.allocators.values()) / self.num_blocks
+
+    def internal_fragmentation(self) -> float:
+        """Fraction of slots in held pages that hold no token (src/llmserve/kvcache/paged.py:149-153);
+        first paged group."""
+        if not self.paged_groups:
+            return 0.0
+        g = self.paged_groups[0]
+        held = self.allocators[g.group_id].num_used * self.block_size
+        if held == 0:
+            return 0.0
+        live = 0
+        for seq, table in self.tables[g.group_id].items():
+            first = next((i for i, b in enumerate(table) if b >= 0), len(table))
+            live += self.lengths[seq] - first * self.block_size
+        return 1.0 - live / held
+
+    # ---- requests -----------------------------------------------------------------------
+    def has_sequence(self, seq_id) -> bool:
+        return seq_id in self.lengths
+
+    def add_sequence(self, seq_id) -> int:
+        """Register a request: empty tables, length 0, a state slot of its own."""
+        if seq_id in self.lengths:
+            raise ValueError(f"sequence {seq_id!r} already exists")
+        try:
+            slot = self._slot_alloc.allocate()
+        except OutOfBlocks:
+            raise OutOfBlocks(f"all {self.max_seqs} state slots are taken") from None
+        self.lengths[seq_id] = 0
+        self.slot_of[seq_id] = slot
+        self._fresh.add(slot)
+        for g in self.paged_groups:
+            self.tables[g.group_id][seq_id] = []
+        return slot
+
+    def free_sequence(self, seq_id) -> None:
+        """Give back everything the request holds."""
+        if seq_id not in self.lengths:
+            raise KeyError(f"unknown sequence {seq_id!r}")
+        for g in self.paged_groups:
+            table = self.tables[g.group_id].pop(seq_id)
+            self.allocators[g.group_id].free([b for b in table if b >= 0])
+        slot = self.slot_of.pop(seq_id)
+        self._fresh.discard(slot)
+        self._slot_alloc.free([slot])
+        del self.lengths[seq_id]
+
+    def extra_blocks_needed(self, seq_id, new_tokens: int) -> int:
+        """Pages one group must add for `new_tokens` more tokens (the same for every group)."""
+        if not self.paged_groups:
+            return 0
+        table = self.tables[self.paged_groups[0].group_id][seq_id]
+        return max(0, self.blocks_for(self.lengths[seq_id] + new_tokens) - len(table))
+
+    def can_append(self, seq_ids, counts) -> bool:
+        need = sum(self.extra_blocks_needed(s, n) for s, n in zip(seq_ids, counts))
+        return need <= self.num_free_blocks
+
+    # ---- one step ---------------------------------------------------------------------------
+    def append(self, seq_ids: list, counts: list[int]) -> StepLayout:
+        if len(set(seq_ids)) != len(seq_ids):
+            raise ValueError("a request may appear once in a step")
+        for s, n in zip(seq_ids, counts):
+            if s not in self.lengths:
+                raise KeyError(f"unknown sequence {s!r}")
+            if n < 1:
+                raise ValueError("every request of a step brings at least one token")
+        need = sum(self.extra_blocks_needed(s, n) for s, n in zip(seq_ids, counts))
+        if need > self.num_free_blocks:
+            raise OutOfBlocks(f"step needs {need} pages, {self.num_free_blocks} free")
+
+        bs = self.block_size
+        layout = StepLayout(seq_ids=list(seq_ids), counts=list(counts),
+                            starts=[self.lengths[s] for s in seq_ids],
+                            state_slots=[self.slot_of[s] for s in seq_ids], fresh_slots=[])
+        for s in seq_ids:
+            slot = self.slot_of[s]
+            if slot in self._fresh:
+                self._fresh.discard(slot)
+                layout.fresh_slots.append(slot)
+        for g in self.paged_groups:
+            alloc, tables = self.allocators[g.group_id], self.tables[g.group_id]
+            token_slots: list[int] = []
+            for s, n, start in zip(seq_ids, counts, layout.starts):
+                table = tables[s]
+                while len(table) < self.blocks_for(start + n):
+                    table.append(alloc.allocate())
+                for p in range(start, start + n):
+                    token_slots.append(table[p // bs] * bs + p % bs)
+            layout.slots[g.group_id] = token_slots
+            layout.tables[g.group_id] = [list(tables[s]) for s in seq_ids]
+        for s, n in zip(seq_ids, counts):
+            self.lengths[s] += n
+        return layout
+
+    def release_passed(self, seq_ids) -> int:
+        """After a step: return the pages of windowed groups that no later query can reach.
+
+        The next query of a request of length `len` sits at position >= len and sees the keys
+        j > position - window, so a page is dead when its last key is <= len - window.
+        Returns the number of pages given back.
+        """
+        bs, freed = self.block_size, 0
+        for g in self.paged_groups:
+            window = g.spec.window
+            if window is None:
+                continue
+            for s in seq_ids:
+                if s not in self.lengths:
+                    continue
+                table = self.tables[g.group_id][s]
+                dead_upto = (self.lengths[s] - window + 1) // bs  # pages [0, dead_upto) are out of reach
+                back = []
+                for i in range(min(max(dead_upto, 0), len(table))):
+                    if table[i] >= 0:
+                        back.append(table[i])
+                        table[i] = -1
+                self.allocators[g.group_id].free(back)
+                freed += len(back)
+        return freed
+
+    # ---- checks used by tests and by `snapshot` ---------------------------------------------
+    def check_invariants(self) -> None:
+        for g in self.paged_groups:
+            alloc = self.allocators[g.group_id]
+            held = [b for t in self.tables[g.group_id].values() for b in t if b >= 0]
+            if len(held) != len(set(held)):
+                raise AssertionError(f"group {g.group_id}: a page is held twice")
+            if set(held) != alloc._used:
+                raise AssertionError(f"group {g.group_id}: tables and allocator disagree")
+            if alloc.num_free + alloc.num_used != alloc.num_blocks:
+                raise AssertionError(f"group {g.group_id}: pages lost")
+        slots = list(self.slot_of.values())
+        if len(slots) != len(set(slots)) or set(slots) != self._slot_alloc._used:
+            raise AssertionError("state slots are not unique among live requests")

@@ -1,0 +1,102 @@
+// Shared helpers of the gfx950 kernels: element types, conversions, wave64 reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#define LLMS_WAVE 64
+
+// Error codes returned by the extern "C" launchers (0 = launched).
+#define LLMS_OK 0
+#define LLMS_ERR_ARG 1     // an argument the kernel cannot take (message printed to stderr)
+#define LLMS_ERR_LAUNCH 2  // the HIP runtime refused the launch
+
+#define LLMS_REQUIRE(cond, msg)                                        \
+    do {                                                               \
+        if (!(cond)) {                                                 \
+            fprintf(stderr, "llmserve kernel argument error: %s\n", msg); \
+            return LLMS_ERR_ARG;                                       \
+        }                                                              \
+    } while (0)
+
+#define LLMS_LAUNCH_CHECK()                                            \
+    do {                                                               \
+        hipError_t e_ = hipGetLastError();                             \
+        if (e_ != hipSuccess) {                                        \
+            fprintf(stderr, "llmserve kernel launch failed: %s\n", hipGetErrorString(e_)); \
+            return LLMS_ERR_LAUNCH;                                    \
+        }                                                              \
+        return LLMS_OK;                                                \
+    } while (0)
+
+// bfloat16 is carried as its 16 raw bits.
+struct bf16 {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+// Round to nearest even; NaN stays NaN.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16 v) { return bf16_bits_to_f32(v.bits); }
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ bf16 from_f32<bf16>(float v) {
+    bf16 r;
+    r.bits = f32_to_bf16_bits(v);
+    return r;
+}
+
+// Value of v after one rounding to T (what a store followed by a load would give).
+template <typename T>
+__device__ __forceinline__ float round_to(float v) { return to_f32(from_f32<T>(v)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = LLMS_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, LLMS_WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = LLMS_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, LLMS_WAVE));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads, same value returned to every thread.  The order
+// of additions depends only on the block size, never on the data or the grid.
+__device__ __forceinline__ float block_sum(float v, float* lds /* >= 16 floats */) {
+    const int lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
+    const int nwaves = (blockDim.x + LLMS_WAVE - 1) / LLMS_WAVE;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) lds[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nwaves; ++i) t += lds[i];
+    return t;
+}
+
+__device__ __forceinline__ float block_max(float v, float* lds) {
+    const int lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
+    const int nwaves = (blockDim.x + LLMS_WAVE - 1) / LLMS_WAVE;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) lds[wave] = v;
+    __syncthreads();
+    float t = lds[0];
+    for (int i = 1; i < nwaves; ++i) t = fmaxf(t, lds[i]);
+    return t;
+}

@@ -1,0 +1,187 @@
+// Row-wise kernels of the decoder: embedding gather, (residual add +) RMSNorm,
+// rotary position encoding fused with the paged key/value store, SiLU(gate)*up.
+// Every kernel exists for float and for bfloat16 storage; statistics, angles and the
+// residual sum are always computed in 32-bit.
+#include "common.h"
+
+// ------------------------------------------------------------------ embedding gather
+// out[n, :] = table[ids[n], :].  An id outside [0, vocab) yields a row of NaN, so a bad
+// token shows in the logits and never reads outside the table.
+template <typename T>
+__global__ void embed_gather_kernel(T* __restrict__ out, const T* __restrict__ table,
+                                    const int* __restrict__ ids, int hidden, int vocab) {
+    const int n = blockIdx.x;
+    const int id = ids[n];
+    T* o = out + (size_t)n * hidden;
+    if ((unsigned)id >= (unsigned)vocab) {
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_f32<T>(__uint_as_float(0x7fc00000u));
+        return;
+    }
+    const T* src = table + (size_t)id * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = src[i];
+}
+
+// ------------------------------------------------------------------ RMSNorm
+// For output row r (source row s = rows ? rows[r] : r):
+//   v = x[s] (+ delta[s], summed in 32-bit and rounded once to T)
+//   if resid_out: resid_out[s] = v                    (may alias x)
+//   out[r] = weight * T(v * rsqrt(mean(v^2) + eps))   (cast before the weight, as the
+//            reference does: src/llmserve/model/llama.py:24-28)
+template <typename T>
+__global__ void rmsnorm_kernel(T* __restrict__ out, const T* x, const T* __restrict__ delta, T* resid_out,
+                               const T* __restrict__ weight, const int* __restrict__ rows, float eps,
+                               int hidden) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const int s = rows ? rows[r] : r;
+    const T* xs = x + (size_t)s * hidden;
+    const T* ds = delta ? delta + (size_t)s * hidden : nullptr;
+    T* rs = resid_out ? resid_out + (size_t)s * hidden : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = to_f32(xs[i]);
+        if (ds) v = round_to<T>(v + to_f32(ds[i]));
+        if (rs) rs[i] = from_f32<T>(v);
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float inv = rsqrtf(ss / (float)hidden + eps);
+    T* o = out + (size_t)r * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v;
+        if (rs) {
+            v = to_f32(rs[i]);  // written by this same thread above
+        } else {
+            v = to_f32(xs[i]);
+            if (ds) v = round_to<T>(v + to_f32(ds[i]));
+        }
+        o[i] = from_f32<T>(to_f32(weight[i]) * round_to<T>(v * inv));
+    }
+}
+
+// ------------------------------------------------------------------ rotary encoding + cache store
+// qkv row n = [q heads | k heads | v heads], head_dim wide each.
+//   q, k: x' = x*cos + rotate_half(x)*sin with pairs (i, i + D/2) and angle
+//         float(position) * inv_freq[i]  (src/llmserve/model/llama.py:31-54), computed in
+//         32-bit and rounded once.  q is rotated in place.  inv_freq == nullptr: no rotation.
+//   k' goes to k_pool[page, kv_head, offset, :], v to v_pool[page, kv_head, :, offset]
+//   (values transposed inside a page so that attention reads keys of one dimension
+//   contiguously), page = slot / block_size, offset = slot % block_size.  slot < 0: no store.
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ qkv, const float* __restrict__ inv_freq,
+                                  const int* __restrict__ positions, const int* __restrict__ slots,
+                                  T* __restrict__ k_pool, T* __restrict__ v_pool, int n_heads,
+                                  int n_kv_heads, int head_dim, int block_size) {
+    const int n = blockIdx.x;
+    const int half = head_dim / 2;
+    const int row_width = (n_heads + 2 * n_kv_heads) * head_dim;
+    T* row = qkv + (size_t)n * row_width;
+    const float pos = (float)positions[n];
+    const int slot = slots ? slots[n] : -1;
+    const int page = slot >= 0 ? slot / block_size : 0;
+    const int off = slot >= 0 ? slot % block_size : 0;
+
+    // rotate q heads in place and k heads into the pool: one thread per (head, pair)
+    const int rot_heads = n_heads + n_kv_heads;
+    for (int t = threadIdx.x; t < rot_heads * half; t += blockDim.x) {
+        const int h = t / half, i = t % half;
+        T* x = row + (size_t)h * head_dim;
+        float a = to_f32(x[i]), b = to_f32(x[i + half]);
+        float ra = a, rb = b;
+        if (inv_freq) {
+            float sn, cs;
+            sincosf(pos * inv_freq[i], &sn, &cs);
+            ra = a * cs - b * sn;
+            rb = b * cs + a * sn;
+        }
+        if (h < n_heads) {
+            x[i] = from_f32<T>(ra);
+            x[i + half] = from_f32<T>(rb);
+        } else if (slot >= 0) {
+            const int kvh = h - n_heads;
+            T* dst = k_pool + (((size_t)page * n_kv_heads + kvh) * block_size + off) * head_dim;
+            dst[i] = from_f32<T>(ra);
+            dst[i + half] = from_f32<T>(rb);
+        }
+    }
+    if (slot >= 0) {
+        const T* v = row + (size_t)(n_heads + n_kv_heads) * head_dim;
+        for (int t = threadIdx.x; t < n_kv_heads * head_dim; t += blockDim.x) {
+            const int kvh = t / head_dim, d = t % head_dim;
+            v_pool[(((size_t)page * n_kv_heads + kvh) * head_dim + d) * block_size + off] = v[t];
+        }
+    }
+}
+
+// ------------------------------------------------------------------ SiLU(gate) * up
+// gate_up row = [gate (inter) | up (inter)]; out = T(T(silu(gate)) * up), the reference's
+// rounding points (src/llmserve/model/llama.py:120).
+template <typename T>
+__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gate_up, int inter, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const size_t n = idx / inter;
+    const int i = (int)(idx % inter);
+    const T* row = gate_up + n * 2 * (size_t)inter;
+    const float g = to_f32(row[i]);
+    const float u = to_f32(row[inter + i]);
+    const float s = round_to<T>(g / (1.f + expf(-g)));
+    out[idx] = from_f32<T>(s * u);
+}
+
+// ------------------------------------------------------------------ launchers
+#define DISPATCH_DTYPE(dtype, ...)                 \
+    if ((dtype) == 0) {                            \
+        typedef float T;                           \
+        __VA_ARGS__                                \
+    } else if ((dtype) == 1) {                     \
+        typedef bf16 T;                            \
+        __VA_ARGS__                                \
+    } else {                                       \
+        LLMS_REQUIRE(false, "dtype must be 0 (float32) or 1 (bfloat16)"); \
+    }
+
+extern "C" {
+
+int llms_embed_gather(int dtype, void* out, const void* table, const int* ids, int n_tokens, int hidden,
+                      int vocab, hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && hidden > 0 && vocab > 0, "embed_gather: sizes must be positive");
+    DISPATCH_DTYPE(dtype, embed_gather_kernel<T><<<n_tokens, 256, 0, stream>>>((T*)out, (const T*)table, ids,
+                                                                                hidden, vocab);)
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_rmsnorm(int dtype, void* out, const void* x, const void* delta, void* resid_out, const void* weight,
+                 const int* rows, float eps, int n_rows, int hidden, hipStream_t stream) {
+    LLMS_REQUIRE(n_rows > 0 && hidden > 0, "rmsnorm: sizes must be positive");
+    LLMS_REQUIRE(!(rows && resid_out), "rmsnorm: a row gather cannot also write the residual back");
+    const int threads = hidden >= 2048 ? 512 : 256;
+    DISPATCH_DTYPE(dtype, rmsnorm_kernel<T><<<n_rows, threads, 0, stream>>>(
+                              (T*)out, (const T*)x, (const T*)delta, (T*)resid_out, (const T*)weight, rows,
+                              eps, hidden);)
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_rope_store(int dtype, void* qkv, const float* inv_freq, const int* positions, const int* slots,
+                    void* k_pool, void* v_pool, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                    int block_size, hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0, "rope_store: sizes must be positive");
+    LLMS_REQUIRE(head_dim > 0 && head_dim % 2 == 0, "rope_store: head_dim must be even");
+    LLMS_REQUIRE(block_size > 0, "rope_store: block_size must be positive");
+    LLMS_REQUIRE(slots == nullptr || (k_pool && v_pool), "rope_store: slots given without pools");
+    DISPATCH_DTYPE(dtype, rope_store_kernel<T><<<n_tokens, 256, 0, stream>>>(
+                              (T*)qkv, inv_freq, positions, slots, (T*)k_pool, (T*)v_pool, n_heads,
+                              n_kv_heads, head_dim, block_size);)
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_silu_mul(int dtype, void* out, const void* gate_up, int n_rows, int inter, hipStream_t stream) {
+    LLMS_REQUIRE(n_rows > 0 && inter > 0, "silu_mul: sizes must be positive");
+    const size_t total = (size_t)n_rows * inter;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    DISPATCH_DTYPE(dtype, silu_mul_kernel<T><<<blocks, 256, 0, stream>>>((T*)out, (const T*)gate_up, inter,
+                                                                          total);)
+    LLMS_LAUNCH_CHECK();
+}
+
+}  // extern "C"

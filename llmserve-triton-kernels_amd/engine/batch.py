@@ -1,0 +1,129 @@
+"""One step's batch as the kernels see it: a flat run of new tokens, no padding.
+
+The reference describes a step by `PagedBatch` (src/llmserve/kvcache/paged.py:65-79):
+positions and a validity mask over a right-padded [B, T] grid, write blocks and offsets,
+block tables, context lengths, last indices.  Here the new tokens of all requests lie end
+to end (request b owns rows cu_seqlens[b] .. cu_seqlens[b+1]), any mixture of portions of
+prompts and single decoded tokens; requests that bring one token come first.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from ..cache.manager import StepLayout
+
+
+@dataclass
+class GroupView:
+    """One cache group's part of a step."""
+
+    block_tables: torch.Tensor  # int32 [B, M]; entries of returned pages are 0 and never read
+    slots: torch.Tensor  # int32 [N]: page * block_size + offset of every new token
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_seqs: int
+    token_ids: torch.Tensor  # int32 [N]
+    positions: torch.Tensor  # int32 [N] absolute position of each new token
+    token_seq: torch.Tensor  # int32 [N] index (0..B-1) of the request a token belongs to
+    cu_seqlens: torch.Tensor  # int32 [B+1]
+    context_lens: torch.Tensor  # int32 [B] keys present after this step's store
+    state_slots: torch.Tensor  # int32 [B] state slot of each request
+    logit_rows: torch.Tensor  # int32 [R] rows whose logits are wanted
+    groups: dict[int, GroupView]
+    # host copies, for choosing kernels without a read-back
+    counts: list[int] = field(default_factory=list)
+    starts: list[int] = field(default_factory=list)
+    num_decode: int = 0  # leading requests that bring exactly one token
+    max_count: int = 0
+    max_context: int = 0
+
+
+class BatchUploader:
+    """Packs a step's integer arrays into one pinned buffer and sends them with one copy.
+
+    A small ring of pinned buffers, each guarded by an event, lets a caller issue steps
+    back to back without waiting for the device."""
+
+    def __init__(self, device: torch.device, ring: int = 4):
+        self.device = device
+        self._ring = [None] * ring
+        self._events = [None] * ring
+        self._next = 0
+
+    def upload(self, flat: list[int]) -> torch.Tensor:
+        n = len(flat)
+        i = self._next
+        self._next = (i + 1) % len(self._ring)
+        if self._events[i] is not None:
+            self._events[i].synchronize()
+        buf = self._ring[i]
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 4096), dtype=torch.int32, pin_memory=True)
+            self._ring[i] = buf
+        buf[:n] = torch.tensor(flat, dtype=torch.int32)
+        dev = torch.empty(n, dtype=torch.int32, device=self.device)
+        dev.copy_(buf[:n], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(self.device))
+        self._events[i] = ev
+        return dev
+
+
+def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[int],
+                uploader: BatchUploader) -> StepBatch:
+    """Device tensors for a step whose pages `layout` has already fixed."""
+    counts, starts = layout.counts, layout.starts
+    n_seqs = len(counts)
+    flat_tokens = [t for row in tokens for t in row]
+    n_tokens = len(flat_tokens)
+    positions, token_seq, cu = [], [], [0]
+    for b, (start, n) in enumerate(zip(starts, counts)):
+        positions.extend(range(start, start + n))
+        token_seq.extend([b] * n)
+        cu.append(cu[-1] + n)
+    context = [s + n for s, n in zip(starts, counts)]
+
+    sections: list[list[int]] = [flat_tokens, positions, token_seq, cu, context, layout.state_slots,
+                                 list(logit_rows)]
+    group_ids = sorted(layout.tables)
+    widths = {}
+    for g in group_ids:
+        width = max(1, max(len(t) for t in layout.tables[g]))
+        widths[g] = width
+        table_flat: list[int] = []
+        for t in layout.tables[g]:
+            table_flat.extend(b if b >= 0 else 0 for b in t)
+            table_flat.extend([0] * (width - len(t)))
+        sections.append(layout.slots[g])
+        sections.append(table_flat)
+    flat: list[int] = []
+    offsets = []
+    for sec in sections:
+        offsets.append(len(flat))
+        flat.extend(sec)
+        flat.extend([0] * (-len(flat) % 4))  # keep every section 16-byte aligned
+    dev = uploader.upload(flat)
+
+    def view(i: int, n: int) -> torch.Tensor:
+        return dev[offsets[i]: offsets[i] + n]
+
+    groups = {}
+    for j, g in enumerate(group_ids):
+        slots = view(7 + 2 * j, n_tokens)
+        tables = view(8 + 2 * j, n_seqs * widths[g]).view(n_seqs, widths[g])
+        groups[g] = GroupView(tables, slots)
+    num_decode = 0
+    while num_decode < n_seqs and counts[num_decode] == 1:
+        num_decode += 1
+    return StepBatch(
+        num_tokens=n_tokens, num_seqs=n_seqs, token_ids=view(0, n_tokens), positions=view(1, n_tokens),
+        token_seq=view(2, n_tokens), cu_seqlens=view(3, n_seqs + 1), context_lens=view(4, n_seqs),
+        state_slots=view(5, n_seqs), logit_rows=view(6, len(logit_rows)), groups=groups,
+        counts=list(counts), starts=list(starts), num_decode=num_decode, max_count=max(counts),
+        max_context=max(context))

@@ -1,0 +1,153 @@
+"""The step function: runs a batch of (request, its next tokens) through the model, from
+the cache that earlier steps left, and returns the logits at the wanted places.
+
+The reference has no single step function: its scheduler runs one padded forward for new
+prompts and one for decoding requests (src/llmserve/scheduler/engine.py:186-193,236-246).
+Here one call runs everything a step holds as one flat batch: portions of prompts beside
+single decoded tokens, cut anywhere.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from pathlib import Path
+
+import torch
+
+from ..cache.manager import CacheManager, group_layers
+from ..cache.storage import CacheStorage, num_blocks_for_budget
+from ..config.engine_config import EngineConfig
+from ..config.registry import architecture_of, read_config
+from ..ops import library as ops
+from ..parts.model import Model
+from ..parts.registry import BuildContext
+from ..weights.loader import load_tensors
+from ..weights.random import random_tensors
+from .batch import BatchUploader, build_batch
+
+_TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its next tokens, and the places among them (0-based
+    within `tokens`) whose logits are wanted."""
+
+    seq_id: object
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)
+
+
+class ModelRunner:
+    def __init__(self, model: Model, config, engine_config: EngineConfig, device: torch.device):
+        self.model = model
+        self.config = config
+        self.engine_config = engine_config
+        self.device = device
+        self.dtype = model.ctx.dtype
+        self.vocab_size = model.spec.vocab_size
+        self.max_model_len = engine_config.max_model_len or model.spec.max_positions
+        self.block_size = engine_config.block_size
+        groups = group_layers(model.cache_specs())
+        elem = torch.empty(0, dtype=self.dtype).element_size()
+        if engine_config.num_blocks is not None:
+            num_blocks = engine_config.num_blocks
+        else:
+            budget = engine_config.kv_bytes
+            if budget is None:
+                free, _total = torch.cuda.mem_get_info(device)
+                budget = int(free * engine_config.gpu_memory_fraction)
+            num_blocks = num_blocks_for_budget(groups, self.block_size, elem, budget)
+            # more pages than every slot could ever fill are of no use
+            most = engine_config.max_num_seqs * -(-self.max_model_len // self.block_size)
+            num_blocks = min(num_blocks, most)
+        self.manager = CacheManager(groups, num_blocks, self.block_size, engine_config.max_num_seqs)
+        self.storage = CacheStorage(groups, num_blocks, self.block_size, engine_config.max_num_seqs,
+                                    self.dtype, device)
+        self._uploader = BatchUploader(device)
+
+    # ---- construction ---------------------------------------------------------------------
+    @staticmethod
+    def _device(device=None) -> torch.device:
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible; this engine runs on gfx950 only and has no CPU path")
+        return torch.device(device or "cuda:0")
+
+    @classmethod
+    def from_folder(cls, model_dir: str | Path, engine_config: EngineConfig | None = None, device=None):
+        """Model chosen by the folder's config.json, weights from its safetensors files."""
+        engine_config = engine_config or EngineConfig()
+        engine_config.validate()
+        device = cls._device(device)
+        ops.ensure_built(engine_config.dtype)
+        arch, config, _raw = read_config(model_dir)
+        dtype = _TORCH_DTYPES[engine_config.dtype]
+        model = Model(arch.build_spec(config), BuildContext(dtype, device))
+        infos = model.param_infos()
+        ignore = {model.spec.weights["head"] + "weight"} if getattr(model.head, "tied", False) else set()
+        model.load(load_tensors(model_dir, infos, dtype, device, ignore))
+        return cls(model, config, engine_config, device)
+
+    @classmethod
+    def from_random(cls, config_dict: dict, seed: int = 0, engine_config: EngineConfig | None = None,
+                    device=None, on_device: bool = True):
+        """Seeded random weights made in memory (no folder).  `on_device` draws them on the GPU,
+        which is fast for large models; a folder written by `write_random_model` uses the CPU
+        streams instead, so the two do not hold the same numbers."""
+        engine_config = engine_config or EngineConfig()
+        engine_config.validate()
+        device = cls._device(device)
+        ops.ensure_built(engine_config.dtype)
+        arch = architecture_of(config_dict)
+        config = arch.config_class.from_dict(config_dict)
+        dtype = _TORCH_DTYPES[engine_config.dtype]
+        model = Model(arch.build_spec(config), BuildContext(dtype, device))
+        tensors = random_tensors(model.param_infos(), seed, dtype, device if on_device else "cpu")
+        model.load({k: v.to(device) for k, v in tensors.items()})
+        return cls(model, config, engine_config, device)
+
+    # ---- requests -------------------------------------------------------------------------
+    def add_sequence(self, seq_id) -> None:
+        self.manager.add_sequence(seq_id)
+
+    def free_sequence(self, seq_id) -> None:
+        self.manager.free_sequence(seq_id)
+
+    # ---- the step ---------------------------------------------------------------------------
+    @torch.inference_mode()
+    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+        """Run the entries' tokens as one batch; float32 logits [sum(len(want)), vocab] in the
+        order of the entries and of their `want`.  Raises `OutOfBlocks` (nothing changed) when
+        the pages do not suffice."""
+        if not entries:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        for e in entries:
+            if not e.tokens:
+                raise ValueError(f"request {e.seq_id!r} brings no tokens")
+            bad = [t for t in e.tokens if not 0 <= t < self.vocab_size]
+            if bad:
+                raise ValueError(f"request {e.seq_id!r}: token ids {bad[:5]} are outside the vocabulary "
+                                 f"[0, {self.vocab_size})")
+            if any(not 0 <= w < len(e.tokens) for w in e.want):
+                raise ValueError(f"request {e.seq_id!r}: wanted places {e.want} are outside its {len(e.tokens)} tokens")
+            length = self.manager.lengths.get(e.seq_id)
+            if length is None:
+                raise KeyError(f"unknown sequence {e.seq_id!r}")
+            if length + len(e.tokens) > self.max_model_len:
+                raise ValueError(f"request {e.seq_id!r} would reach {length + len(e.tokens)} tokens; "
+                                 f"the limit is {self.max_model_len}")
+        # requests that bring a single token go first (kernels for decoding take the leading rows)
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) != 1)
+        ordered = [entries[i] for i in order]
+        layout = self.manager.append([e.seq_id for e in ordered], [len(e.tokens) for e in ordered])
+        first_row = {}
+        row = 0
+        for e in ordered:
+            first_row[id(e)] = row
+            row += len(e.tokens)
+        logit_rows = [first_row[id(e)] + w for e in entries for w in e.want]
+        self.storage.clear_state(layout.fresh_slots)
+        batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader)
+        logits = self.model.forward(batch, self.storage)
+        self.manager.release_passed(layout.seq_ids)
+        return logits

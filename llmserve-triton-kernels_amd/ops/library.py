@@ -1,0 +1,324 @@
+"""Python face of the HIP kernels: loads the compiled libraries with ctypes and checks,
+on the host, every shape and dtype a kernel relies on before launching it.
+
+There is no fallback: a call fails with `KernelLibraryError` when its library cannot be
+built or loaded, and with `ValueError` when the arguments are not what the kernel takes.
+Kernels run on the current torch stream of the tensors' device.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+import threading
+
+import torch
+
+from . import build as _build
+
+c_void_p, c_int, c_float = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+_libs: dict[str, ctypes.CDLL] = {}
+_lock = threading.Lock()
+
+
+def load(name: str) -> ctypes.CDLL:
+    """The compiled library of ``csrc/<name>.hip`` (built at the first call if need be)."""
+    lib = _libs.get(name)
+    if lib is not None:
+        return lib
+    with _lock:
+        if name in _libs:
+            return _libs[name]
+        try:
+            path = _build.build([name])[name]
+            lib = ctypes.CDLL(str(path))
+        except (OSError, _build.BuildError) as e:
+            raise KernelLibraryError(f"HIP kernel library '{name}' is not available: {e}") from e
+        _libs[name] = lib
+        return lib
+
+
+def ensure_built(dtype_name: str, verbose: bool = True) -> None:
+    """Compile (if missing) and load every library a model of this dtype uses."""
+    names = _build.GROUPS[dtype_name]
+    _build.build(names, verbose=verbose)
+    for n in names:
+        load(n)
+
+
+def has_mfma() -> bool:
+    """Whether the matrix-core kernels for bfloat16 are part of this build."""
+    return "gemm_mfma" in _build.all_sources()
+
+
+def loaded_libraries() -> dict[str, str]:
+    return {k: v._name for k, v in _libs.items()}
+
+
+# ------------------------------------------------------------------------------ checks
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise ValueError(f"kernels take float32 or bfloat16 tensors, not {t.dtype}") from None
+
+
+def _dev(*tensors: torch.Tensor | None) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("kernels take GPU tensors only (there is no CPU path)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def _ptr(t: torch.Tensor | None) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream(dev: torch.device) -> c_void_p:
+    return c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _i32(t: torch.Tensor, name: str, numel: int | None = None) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous int32 tensor")
+    if numel is not None and t.numel() != numel:
+        raise ValueError(f"{name} has {t.numel()} elements, expected {numel}")
+
+
+def _f32(t: torch.Tensor, name: str, numel: int | None = None) -> None:
+    if t.dtype != torch.float32 or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous float32 tensor")
+    if numel is not None and t.numel() != numel:
+        raise ValueError(f"{name} has {t.numel()} elements, expected {numel}")
+
+
+def _rows(t: torch.Tensor, name: str, cols: int | None = None) -> None:
+    if t.dim() != 2 or t.stride(1) != 1 or not t.is_contiguous():
+        raise ValueError(f"{name} must be a contiguous 2-d tensor, got shape {tuple(t.shape)} stride {t.stride()}")
+    if cols is not None and t.shape[1] != cols:
+        raise ValueError(f"{name} has {t.shape[1]} columns, expected {cols}")
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        raise KernelLibraryError(f"{what}: kernel launcher returned {status} (see stderr)")
+
+
+# ------------------------------------------------------------------------------ elementwise
+
+
+def embed_gather(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """out[n] = table[ids[n]]; out [N,H], table [V,H], ids int32 [N]."""
+    dev = _dev(out, table, ids)
+    _rows(out, "out")
+    _rows(table, "table", out.shape[1])
+    _i32(ids, "ids", out.shape[0])
+    if out.dtype != table.dtype:
+        raise ValueError("out and table differ in dtype")
+    if out.shape[0] == 0:
+        return out
+    _check(load("elementwise").llms_embed_gather(
+        c_int(_code(out)), _ptr(out), _ptr(table), _ptr(ids), c_int(out.shape[0]), c_int(out.shape[1]),
+        c_int(table.shape[0]), _stream(dev)), "embed_gather")
+    return out
+
+
+def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, *,
+            delta: torch.Tensor | None = None, resid_out: torch.Tensor | None = None,
+            rows: torch.Tensor | None = None) -> torch.Tensor:
+    """out[r] = weight * norm(x[s] + delta[s]), s = rows[r] or r; resid_out[s] = x[s] + delta[s]."""
+    dev = _dev(out, x, weight, delta, resid_out, rows)
+    _rows(x, "x")
+    hidden = x.shape[1]
+    _rows(out, "out", hidden)
+    n_out = out.shape[0]
+    if weight.dim() != 1 or weight.numel() != hidden or not weight.is_contiguous():
+        raise ValueError(f"weight must have {hidden} elements")
+    for name, t in (("delta", delta), ("resid_out", resid_out)):
+        if t is not None:
+            _rows(t, name, hidden)
+            if t.shape != x.shape or t.dtype != x.dtype:
+                raise ValueError(f"{name} must match x in shape and dtype")
+    if out.dtype != x.dtype or weight.dtype != x.dtype:
+        raise ValueError("out, x and weight must share one dtype")
+    if rows is not None:
+        _i32(rows, "rows", n_out)
+        if resid_out is not None:
+            raise ValueError("a row gather cannot also write the residual back")
+    elif n_out != x.shape[0]:
+        raise ValueError("out and x differ in rows")
+    if n_out == 0:
+        return out
+    _check(load("elementwise").llms_rmsnorm(
+        c_int(_code(x)), _ptr(out), _ptr(x), _ptr(delta), _ptr(resid_out), _ptr(weight), _ptr(rows),
+        c_float(eps), c_int(n_out), c_int(hidden), _stream(dev)), "rmsnorm")
+    return out
+
+
+def rope_store(qkv: torch.Tensor, inv_freq: torch.Tensor | None, positions: torch.Tensor,
+               slots: torch.Tensor | None, k_pool: torch.Tensor | None, v_pool: torch.Tensor | None,
+               n_heads: int, n_kv_heads: int, head_dim: int, block_size: int) -> None:
+    """Rotate q (in place) and k, store k and v of each token at its cache slot.
+
+    qkv [N, (n_heads + 2 n_kv_heads) * head_dim]; k_pool [pages, n_kv_heads, block_size, head_dim];
+    v_pool [pages, n_kv_heads, head_dim, block_size]; slots int32 [N] (page * block_size + offset, or -1).
+    """
+    dev = _dev(qkv, inv_freq, positions, slots, k_pool, v_pool)
+    _rows(qkv, "qkv", (n_heads + 2 * n_kv_heads) * head_dim)
+    n = qkv.shape[0]
+    _i32(positions, "positions", n)
+    if inv_freq is not None:
+        _f32(inv_freq, "inv_freq", head_dim // 2)
+    if slots is not None:
+        _i32(slots, "slots", n)
+        if k_pool is None or v_pool is None:
+            raise ValueError("slots given without pools")
+        pages = k_pool.shape[0]
+        if tuple(k_pool.shape) != (pages, n_kv_heads, block_size, head_dim) or not k_pool.is_contiguous():
+            raise ValueError(f"k_pool shape {tuple(k_pool.shape)} is not [pages,{n_kv_heads},{block_size},{head_dim}]")
+        if tuple(v_pool.shape) != (pages, n_kv_heads, head_dim, block_size) or not v_pool.is_contiguous():
+            raise ValueError(f"v_pool shape {tuple(v_pool.shape)} is not [pages,{n_kv_heads},{head_dim},{block_size}]")
+        if k_pool.dtype != qkv.dtype or v_pool.dtype != qkv.dtype:
+            raise ValueError("pools and qkv differ in dtype")
+    if n == 0:
+        return
+    _check(load("elementwise").llms_rope_store(
+        c_int(_code(qkv)), _ptr(qkv), _ptr(inv_freq), _ptr(positions), _ptr(slots), _ptr(k_pool), _ptr(v_pool),
+        c_int(n), c_int(n_heads), c_int(n_kv_heads), c_int(head_dim), c_int(block_size), _stream(dev)),
+        "rope_store")
+
+
+def silu_mul(out: torch.Tensor, gate_up: torch.Tensor) -> torch.Tensor:
+    """out = silu(gate_up[:, :I]) * gate_up[:, I:]."""
+    dev = _dev(out, gate_up)
+    _rows(out, "out")
+    _rows(gate_up, "gate_up", 2 * out.shape[1])
+    if out.shape[0] != gate_up.shape[0] or out.dtype != gate_up.dtype:
+        raise ValueError("out and gate_up disagree")
+    if out.shape[0] == 0:
+        return out
+    _check(load("elementwise").llms_silu_mul(
+        c_int(_code(out)), _ptr(out), _ptr(gate_up), c_int(out.shape[0]), c_int(out.shape[1]), _stream(dev)),
+        "silu_mul")
+    return out
+
+
+# ------------------------------------------------------------------------------ matrix products
+
+
+def gemm_fma(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """out[M,N] = a[M,K] w[N,K]^T (+ bias): 32-bit multiply-add on the vector units."""
+    dev = _dev(out, a, w, bias)
+    if a.dim() != 2 or a.stride(1) != 1 or out.dim() != 2 or out.stride(1) != 1:
+        raise ValueError("a and out must be 2-d with unit inner stride")
+    _rows(w, "w", a.shape[1])
+    m, k = a.shape
+    n = w.shape[0]
+    if tuple(out.shape) != (m, n):
+        raise ValueError(f"out shape {tuple(out.shape)} is not {(m, n)}")
+    if a.dtype != w.dtype or (bias is not None and (bias.dtype != w.dtype or bias.numel() != n)):
+        raise ValueError("a, w and bias must share one dtype; bias has N elements")
+    if (a.dtype, out.dtype) not in ((torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                    (torch.bfloat16, torch.float32)):
+        raise ValueError(f"gemm_fma does not take {a.dtype} -> {out.dtype}")
+    if m == 0:
+        return out
+    _check(load("gemm").llms_gemm_fma(
+        c_int(_code(a)), c_int(_code(out)), _ptr(out), _ptr(a), _ptr(w), _ptr(bias), c_int(m), c_int(n), c_int(k),
+        c_int(a.stride(0)), c_int(out.stride(0)), _stream(dev)), "gemm_fma")
+    return out
+
+
+# ------------------------------------------------------------------------------ attention
+
+
+def _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size):
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < n_heads * head_dim:
+        raise ValueError("q must be [N, >= n_heads*head_dim] with unit inner stride")
+    _rows(out, "out", n_heads * head_dim)
+    if out.shape[0] != q.shape[0] or out.dtype != q.dtype:
+        raise ValueError("out and q disagree")
+    pages = k_pool.shape[0]
+    if tuple(k_pool.shape) != (pages, n_kv_heads, block_size, head_dim) or not k_pool.is_contiguous():
+        raise ValueError(f"k_pool shape {tuple(k_pool.shape)} is not [pages,{n_kv_heads},{block_size},{head_dim}]")
+    if tuple(v_pool.shape) != (pages, n_kv_heads, head_dim, block_size) or not v_pool.is_contiguous():
+        raise ValueError(f"v_pool shape {tuple(v_pool.shape)} is not [pages,{n_kv_heads},{head_dim},{block_size}]")
+    if k_pool.dtype != q.dtype or v_pool.dtype != q.dtype:
+        raise ValueError("pools and q differ in dtype")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise ValueError("block_tables must be a contiguous int32 [B, M] tensor")
+    if n_heads % n_kv_heads:
+        raise ValueError("n_heads must be a multiple of n_kv_heads")
+
+
+def attention_wave(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                   block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
+                   n_heads: int, n_kv_heads: int, head_dim: int, block_size: int, window: int = 0,
+                   scale: float | None = None) -> torch.Tensor:
+    """Causal attention of N new tokens over the paged cache (one wave per token and head).
+
+    q: rows of width >= n_heads*head_dim (the q part of a qkv buffer is fine); out [N, n_heads*head_dim];
+    token_seq[n] = row of block_tables for token n; positions[n] = its absolute position.
+    """
+    dev = _dev(out, q, k_pool, v_pool, block_tables, token_seq, positions)
+    _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
+    n = q.shape[0]
+    _i32(token_seq, "token_seq", n)
+    _i32(positions, "positions", n)
+    if not 0 < head_dim <= 256:
+        raise ValueError(f"head_dim={head_dim} is outside 1..256")
+    if n == 0:
+        return out
+    scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
+    _check(load("attention").llms_attention_wave(
+        c_int(_code(q)), _ptr(out), c_int(out.stride(0)), _ptr(q), c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool),
+        _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(token_seq), _ptr(positions), c_int(n),
+        c_int(n_heads), c_int(n_kv_heads), c_int(head_dim), c_int(block_size), c_int(window), c_float(scale),
+        _stream(dev)), "attention_wave")
+    return out
+
+
+# ------------------------------------------------------------------------------ sampling
+
+
+def sample_rows(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor | None = None,
+                top_k: torch.Tensor | None = None, top_p: torch.Tensor | None = None,
+                uniform: torch.Tensor | None = None) -> torch.Tensor:
+    """out[r] = chosen token of logits[r] (float32 [R,V]); all-None options mean greedy."""
+    dev = _dev(out, logits, temperature, top_k, top_p, uniform)
+    if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise ValueError("logits must be float32 [R, V] with unit inner stride")
+    r, v = logits.shape
+    _i32(out, "out", r)
+    if temperature is not None:
+        _f32(temperature, "temperature", r)
+        if uniform is None:
+            raise ValueError("temperature sampling needs uniform numbers")
+    if top_k is not None:
+        _i32(top_k, "top_k", r)
+    if top_p is not None:
+        _f32(top_p, "top_p", r)
+    if uniform is not None:
+        _f32(uniform, "uniform", r)
+    if r == 0:
+        return out
+    _check(load("sampling").llms_sample_rows(
+        _ptr(out), _ptr(logits), c_int(logits.stride(0)), c_int(r), c_int(v), _ptr(temperature), _ptr(top_k),
+        _ptr(top_p), _ptr(uniform), _stream(dev)), "sample_rows")
+    return out

@@ -1,0 +1,13 @@
+"""Parts of a decoder layer, their interfaces and registries, and the generic model."""
+
+from .registry import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS, Block,
+                       BuildContext, FeedForward, Mixer, Norm, Part, PositionEncoding, register_block,
+                       register_feed_forward, register_mixer, register_norm, register_position_encoding)
+from .spec import LayerSpec, ModelSpec, PagedCacheSpec, ParamInfo, PartSpec, StateCacheSpec
+
+__all__ = [
+    "BLOCKS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "Block",
+    "BuildContext", "FeedForward", "Mixer", "Norm", "Part", "PositionEncoding", "register_block",
+    "register_feed_forward", "register_mixer", "register_norm", "register_position_encoding", "LayerSpec",
+    "ModelSpec", "PagedCacheSpec", "ParamInfo", "PartSpec", "StateCacheSpec",
+]

@@ -1,0 +1,88 @@
+"""Grouped-query causal attention over the paged cache
+(src/llmserve/model/llama.py:57-109; mask and cache as src/llmserve/kvcache/paged.py:81-110).
+
+Parameters: hidden, num_heads, num_kv_heads, head_dim, bias (q/k/v only; o_proj never has
+one: src/llmserve/model/llama.py:67), window (None = all keys), position (a PartSpec).
+
+q, k and v projections are stacked into one [(nh + 2 nkv) D, H] matrix at load.  One step:
+project, rotate q and k and store k, v at the new tokens' cache slots, attend over the
+request's pages (the new tokens included), project back.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..ops import library as ops
+from .linear import linear
+from .registry import POSITION_ENCODINGS, Mixer, register_mixer
+from .spec import PagedCacheSpec, ParamInfo
+
+
+@register_mixer("attention")
+class Attention(Mixer):
+    def __init__(self, spec, ctx):
+        super().__init__(spec, ctx)
+        self.hidden = int(spec["hidden"])
+        self.num_heads = int(spec["num_heads"])
+        self.num_kv_heads = int(spec["num_kv_heads"])
+        self.head_dim = int(spec["head_dim"])
+        self.bias = bool(spec.get("bias", False))
+        self.window = spec.get("window")
+        if self.num_heads % self.num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        if not 0 < self.head_dim <= 256:
+            raise ValueError(f"head_dim={self.head_dim} is outside what the attention kernels take (1..256)")
+        if self.window is not None and self.window < 1:
+            raise ValueError("window must be >= 1")
+        self.scale = 1.0 / math.sqrt(self.head_dim)  # SDPA's default scale
+        self.position = POSITION_ENCODINGS.build(spec["position"], ctx)
+        self.qkv_weight = self.qkv_bias = self.o_weight = None
+
+    def cache_spec(self):
+        return PagedCacheSpec(self.num_kv_heads, self.head_dim, self.window)
+
+    def param_infos(self):
+        h, d = self.hidden, self.head_dim
+        infos = {"q_proj.weight": ParamInfo((self.num_heads * d, h)),
+                 "k_proj.weight": ParamInfo((self.num_kv_heads * d, h)),
+                 "v_proj.weight": ParamInfo((self.num_kv_heads * d, h)),
+                 "o_proj.weight": ParamInfo((h, self.num_heads * d))}
+        if self.bias:
+            infos.update({"q_proj.bias": ParamInfo((self.num_heads * d,), "zeros"),
+                          "k_proj.bias": ParamInfo((self.num_kv_heads * d,), "zeros"),
+                          "v_proj.bias": ParamInfo((self.num_kv_heads * d,), "zeros")})
+        return infos
+
+    def load(self, tensors):
+        self.qkv_weight = torch.cat([tensors[f"{n}_proj.weight"] for n in "qkv"], dim=0).contiguous()
+        if self.bias:
+            self.qkv_bias = torch.cat([tensors[f"{n}_proj.bias"] for n in "qkv"], dim=0).contiguous()
+        self.o_weight = tensors["o_proj.weight"].contiguous()
+        self.position.load({})
+
+    def forward(self, x, batch, cache):
+        nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        view = batch.groups[cache.group_id]
+        qkv = linear(x, self.qkv_weight, self.qkv_bias)
+        slots = view.slots if cache.store else None
+        fused = getattr(self.position, "rotate_and_store", None)
+        if fused is not None:
+            fused(qkv, batch.positions, slots, cache.k_pool, cache.v_pool, nh, nkv, d, cache.block_size)
+        else:
+            self.position.rotate(qkv, batch.positions, nh, nkv, d)
+            if slots is not None:
+                ops.rope_store(qkv, None, batch.positions, slots, cache.k_pool, cache.v_pool, nh, nkv, d,
+                               cache.block_size)
+        out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
+        self.attend(out, qkv, cache, view, batch)
+        return linear(out, self.o_weight)
+
+    def attend(self, out, qkv, cache, view, batch):
+        """out[n] = attention of token n's query heads (the first nh*D columns of qkv) over its
+        request's pages.  Picks the kernel by dtype and by what the step holds."""
+        ops.attention_wave(out, qkv, cache.k_pool, cache.v_pool, view.block_tables, batch.token_seq,
+                           batch.positions, self.num_heads, self.num_kv_heads, self.head_dim,
+                           cache.block_size, self.window or 0, self.scale)

@@ -1,0 +1,53 @@
+"""Token embedding (row gather, no scaling: src/llmserve/model/llama.py:141,171) and the
+output head (logits = h W^T in 32-bit, W being the embedding table itself when tied:
+src/llmserve/model/llama.py:151-153,185)."""
+
+from __future__ import annotations
+
+import torch
+
+from ..ops import library as ops
+from .linear import linear
+from .registry import EMBEDDINGS, HEADS, Part
+from .spec import ParamInfo
+
+
+@EMBEDDINGS.register("embedding")
+class TokenEmbedding(Part):
+    def __init__(self, spec, ctx):
+        super().__init__(spec, ctx)
+        self.vocab = int(spec["vocab"])
+        self.hidden = int(spec["hidden"])
+        self.weight: torch.Tensor | None = None
+
+    def param_infos(self):
+        return {"weight": ParamInfo((self.vocab, self.hidden))}
+
+    def load(self, tensors):
+        self.weight = tensors["weight"].contiguous()
+
+    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+        out = torch.empty((token_ids.numel(), self.hidden), dtype=self.weight.dtype, device=self.weight.device)
+        return ops.embed_gather(out, self.weight, token_ids)
+
+
+@HEADS.register("lm_head")
+class LMHead(Part):
+    """Parameters: vocab, hidden, tied.  A tied head has no tensor of its own: the model
+    hands it the embedding table."""
+
+    def __init__(self, spec, ctx):
+        super().__init__(spec, ctx)
+        self.vocab = int(spec["vocab"])
+        self.hidden = int(spec["hidden"])
+        self.tied = bool(spec.get("tied", False))
+        self.weight: torch.Tensor | None = None
+
+    def param_infos(self):
+        return {} if self.tied else {"weight": ParamInfo((self.vocab, self.hidden))}
+
+    def load(self, tensors):
+        self.weight = tensors["weight"].contiguous()
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return linear(h, self.weight, out_dtype=torch.float32)

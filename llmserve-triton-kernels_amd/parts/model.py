@@ -1,0 +1,78 @@
+"""The generic decoder: builds the parts a `ModelSpec` names and runs them in the spec's
+order.  It knows no architecture; an architecture is a function from its configuration to
+a `ModelSpec` (see `models/`).
+
+Forward of one step (src/llmserve/model/llama.py:171-185, restated for a flat batch):
+embed the new tokens, run the scheduled layers over the whole batch, then norm and
+project only the rows whose logits are wanted.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import attention, block, embedding, rmsnorm, rope, swiglu  # noqa: F401  (register the built-in parts)
+from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, BuildContext, Part
+from .spec import ModelSpec, ParamInfo
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, ctx: BuildContext):
+        spec.validate()
+        self.spec = spec
+        self.ctx = ctx
+        self.embedding = EMBEDDINGS.build(spec.embedding, ctx)
+        self.final_norm = NORMS.build(spec.final_norm, ctx)
+        self.head = HEADS.build(spec.head, ctx)
+        self.blocks = []
+        for layer in spec.layers:
+            self.blocks.append(BLOCKS.get(layer.block)(
+                MIXERS.build(layer.mixer, ctx), FEED_FORWARDS.build(layer.feed_forward, ctx),
+                NORMS.build(layer.mixer_norm, ctx), NORMS.build(layer.feed_forward_norm, ctx)))
+
+    # ---- tensors -------------------------------------------------------------------------
+    def _parts(self) -> list[tuple[str, Part]]:
+        """(checkpoint prefix, part) of every part that may hold tensors."""
+        w = self.spec.weights
+        out = [(w["embedding"], self.embedding), (w["final_norm"], self.final_norm), (w["head"], self.head)]
+        for layer, blk in zip(self.spec.layers, self.blocks):
+            out += [(layer.weights["mixer_norm"], blk.mixer_norm), (layer.weights["mixer"], blk.mixer),
+                    (layer.weights["feed_forward_norm"], blk.feed_forward_norm),
+                    (layer.weights["feed_forward"], blk.feed_forward)]
+        return out
+
+    def param_infos(self) -> dict[str, ParamInfo]:
+        """Every tensor of the checkpoint by its name."""
+        infos: dict[str, ParamInfo] = {}
+        for prefix, part in self._parts():
+            for local, info in part.param_infos().items():
+                infos[prefix + local] = info
+        return infos
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        """Hand every part its tensors (device tensors keyed by checkpoint name)."""
+        for prefix, part in self._parts():
+            if part is self.head and getattr(self.head, "tied", False):
+                continue
+            part.load({local: tensors[prefix + local] for local in part.param_infos()})
+        if getattr(self.head, "tied", False):
+            self.head.load({"weight": self.embedding.weight})
+
+    def cache_specs(self) -> list:
+        """Per layer what its mixer keeps between steps (None when it borrows another layer's)."""
+        return [None if layer.cache_from is not None else blk.mixer.cache_spec()
+                for layer, blk in zip(self.spec.layers, self.blocks)]
+
+    # ---- one step ----------------------------------------------------------------------------
+    def forward(self, batch, storage) -> torch.Tensor:
+        """Logits [R, vocab] in 32-bit at `batch.logit_rows` (empty tensor when R = 0)."""
+        x = self.embedding.forward(batch.token_ids)
+        delta = None
+        for index in self.spec.schedule:
+            cache = storage.layer_cache(index, self.spec.layers[index].cache_from)
+            x, delta = self.blocks[index].forward(x, delta, batch, cache)
+        rows = batch.logit_rows
+        if rows.numel() == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
+        h = self.final_norm.norm_rows(x, delta, rows)
+        return self.head.forward(h)

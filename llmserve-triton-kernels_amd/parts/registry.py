@@ -1,0 +1,136 @@
+"""Interfaces of the parts a layer is made of, and the registries that name them.
+
+A part is built from a `PartSpec` (its sizes and constants) and a `BuildContext`
+(dtype and device); it never sees the model it belongs to.  Constructing a part touches
+no device, so the list of a model's tensors can be derived on a machine without a GPU;
+device memory is taken in `load`.
+
+Interfaces (x is always the flat batch of new tokens, [N, hidden], in the model dtype):
+
+  Norm              forward(x) -> y
+                    add_norm(residual, delta) -> y     residual += delta in place (32-bit sum)
+                    norm_rows(x, delta, rows) -> y     only the given rows of x + delta
+  PositionEncoding  rotate(qkv, positions, n_heads, n_kv_heads, head_dim)   in place on q and k
+                    (optional) rotate_and_store(qkv, batch, cache, ...)     fused with the cache store
+  Mixer             cache_spec() -> PagedCacheSpec | StateCacheSpec | None
+                    forward(x, batch, cache) -> y
+  FeedForward       forward(x) -> y
+  Block             forward(x, delta, batch, cache) -> (x, delta)   hidden state is x + delta
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable
+
+import torch
+
+from .spec import PagedCacheSpec, ParamInfo, PartSpec, StateCacheSpec
+
+
+@dataclass(frozen=True)
+class BuildContext:
+    dtype: torch.dtype
+    device: torch.device
+
+
+class Part:
+    """Base of every part.  `param_infos` lists its tensors under their own (local) names."""
+
+    def __init__(self, spec: PartSpec, ctx: BuildContext):
+        self.spec = spec
+        self.ctx = ctx
+
+    def param_infos(self) -> dict[str, ParamInfo]:
+        return {}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        """Take the part's tensors (already on the device, in their stored dtype) and set up
+        device constants.  Called once, also for parts without tensors."""
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def add_norm(self, residual: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
+        if delta is not None:
+            residual.copy_((residual.float() + delta.float()).to(residual.dtype))
+        return self.forward(residual)
+
+    def norm_rows(self, x: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
+        picked = x[rows.long()]
+        if delta is not None:
+            picked = (picked.float() + delta[rows.long()].float()).to(x.dtype)
+        return self.forward(picked)
+
+
+class PositionEncoding(Part):
+    def rotate(self, qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv_heads: int,
+               head_dim: int) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self) -> PagedCacheSpec | StateCacheSpec | None:
+        return None
+
+    def forward(self, x: torch.Tensor, batch, cache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block:
+    """Arrangement of one layer's parts."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.feed_forward_norm = feed_forward_norm
+
+    def forward(self, x, delta, batch, cache):
+        raise NotImplementedError
+
+
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._items: dict[str, Callable] = {}
+
+    def register(self, kind: str, item: Callable | None = None):
+        def put(obj):
+            self._items[kind] = obj
+            return obj
+
+        return put if item is None else put(item)
+
+    def get(self, kind: str) -> Callable:
+        if kind not in self._items:
+            raise KeyError(f"unknown {self.what} kind {kind!r}; registered: {sorted(self._items)}")
+        return self._items[kind]
+
+    def names(self) -> list[str]:
+        return sorted(self._items)
+
+    def build(self, spec: PartSpec, ctx: BuildContext):
+        return self.get(spec.kind)(spec, ctx)
+
+
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+BLOCKS = Registry("block")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("output head")
+
+register_norm = NORMS.register
+register_position_encoding = POSITION_ENCODINGS.register
+register_mixer = MIXERS.register
+register_feed_forward = FEED_FORWARDS.register
+register_block = BLOCKS.register

@@ -1,0 +1,48 @@
+"""Rotary position encoding with half-split pairing (dimension i pairs with i + D/2):
+inv_freq_i = theta^(-2i/D), angle = position * inv_freq_i, x' = x cos + rotate_half(x) sin
+(src/llmserve/model/llama.py:31-54).  Parameters: head_dim, theta.
+
+The frequencies are computed once, in 32-bit, by the reference's formula; the kernel
+multiplies them by the position and rotates in 32-bit.  The rotation is fused with the
+store of the new keys and values into the paged cache.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..ops import library as ops
+from .registry import PositionEncoding, register_position_encoding
+
+
+@register_position_encoding("rope")
+class RotaryEncoding(PositionEncoding):
+    def __init__(self, spec, ctx):
+        super().__init__(spec, ctx)
+        self.head_dim = int(spec["head_dim"])
+        self.theta = float(spec["theta"])
+        if self.head_dim % 2:
+            raise ValueError(f"rotary encoding needs an even head_dim, got {self.head_dim}")
+        self.inv_freq: torch.Tensor | None = None
+
+    def frequencies(self) -> torch.Tensor:
+        exponent = torch.arange(0, self.head_dim, 2, dtype=torch.float32) / self.head_dim
+        return 1.0 / (self.theta ** exponent)
+
+    def load(self, tensors):
+        self.inv_freq = self.frequencies().to(self.ctx.device)
+
+    def rotate(self, qkv, positions, n_heads, n_kv_heads, head_dim):
+        ops.rope_store(qkv, self.inv_freq, positions, None, None, None, n_heads, n_kv_heads, head_dim, 1)
+
+    def rotate_and_store(self, qkv, positions, slots, k_pool, v_pool, n_heads, n_kv_heads, head_dim, block_size):
+        ops.rope_store(qkv, self.inv_freq, positions, slots, k_pool, v_pool, n_heads, n_kv_heads, head_dim,
+                       block_size)
+
+
+@register_position_encoding("none")
+class NoPositionEncoding(PositionEncoding):
+    """Keys and queries are used as projected."""
+
+    def rotate(self, qkv, positions, n_heads, n_kv_heads, head_dim):
+        return None
