@@ -1,0 +1,148 @@
+"""Decode and prefill throughput of the engine on one MI355X, TinyLlama-1.1B shape, random
+weights, bfloat16.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 512] [--layers L]
+
+Prints one JSON line.  `value` is decoded tokens per second at the default batch: K timed
+scheduler steps (step function + sampling + the read-back of the token ids) after W untimed
+ones, with synchronisation on both sides.  `prefill` is one request of 2,048 tokens in one
+step; `roofline` prices the decode step against HBM bandwidth (every weight it uses read
+once, plus the keys and values of the live requests); `points` holds decode at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}  # dense matrix-core peaks, MI355X
+PREFILL_TOKENS = 2048
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=512)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--model", default="tinyllama-1.1b")
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
+        return 2
+
+    import torch
+
+    from llmserve import EngineConfig, SamplingParams
+    from llmserve.config import preset
+    from llmserve.engine.runner import ModelRunner
+    from llmserve.engine.scheduler import ContinuousBatchingEngine
+    from llmserve.sampling import Sampler
+
+    cfg = preset(args.model)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    layers = cfg["num_hidden_layers"]
+    h, inter, vocab = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    nh, nkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    d = h // nh
+    elem = 2 if args.dtype == "bfloat16" else 4
+    block_size = 16
+    max_batch = 64 if not args.no_points else args.batch
+    decode_len = args.context + args.warmup + args.steps + 2
+    cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], PREFILL_TOKENS + 8, decode_len)
+    pages = max(max_batch * -(-decode_len // block_size), -(-(PREFILL_TOKENS + 8) // block_size)) + 16
+    engine_cfg = EngineConfig(dtype=args.dtype, block_size=block_size, num_blocks=pages, max_num_seqs=max_batch,
+                              max_num_batched_tokens=max(PREFILL_TOKENS, max_batch), seed=0)
+    runner = ModelRunner.from_random(cfg, seed=0, engine_config=engine_cfg)
+    sampler = Sampler(runner.device)
+    gen = torch.Generator().manual_seed(0)
+
+    def prompts(n, length):
+        lo = min(100, vocab // 4)
+        return [torch.randint(lo, vocab, (length,), generator=gen).tolist() for _ in range(n)]
+
+    def decode_rate(batch):
+        eng = ContinuousBatchingEngine(runner, sampler, max_num_seqs=batch,
+                                       max_num_batched_tokens=engine_cfg.max_num_batched_tokens)
+        for p in prompts(batch, args.context):
+            eng.add_request(p, SamplingParams(max_new_tokens=args.warmup + args.steps + 1))
+        while eng.waiting or any(len(r.all_ids) - r.num_computed_tokens > 1 for r in eng.running):
+            eng.step()  # prompts in
+        for _ in range(args.warmup):
+            eng.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            eng.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert len(eng.running) == batch and eng.stats.preemptions == 0
+        eng.run_until_complete()
+        return batch * args.steps / dt, dt / args.steps
+
+    def prefill_time():
+        eng = ContinuousBatchingEngine(runner, sampler, max_num_seqs=1, max_num_batched_tokens=PREFILL_TOKENS)
+        times = []
+        for i in range(4):
+            eng.add_request(prompts(1, PREFILL_TOKENS)[0], SamplingParams(max_new_tokens=1))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            eng.step()  # the whole prompt in one step, first token sampled and read back
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            assert not eng.has_unfinished()
+        return sorted(times[1:])[len(times[1:]) // 2]
+
+    value, step_s = decode_rate(args.batch)
+    points = {}
+    if not args.no_points:
+        points = {"decode_b1": round(decode_rate(1)[0], 1), "decode_b64": round(decode_rate(64)[0], 1)}
+    pre_s = prefill_time()
+
+    # bytes a decode step must read: every matrix and norm once, the rows of the embedding it
+    # gathers, and the keys and values of the live requests at their mean length in the timed steps
+    per_layer = ((nh + 2 * nkv) * d * h + h * nh * d + 3 * h * inter + 2 * h) * elem
+    weight_bytes = layers * per_layer + (vocab * h + h) * elem + args.batch * h * elem
+    mean_ctx = args.context + args.warmup + args.steps / 2
+    kv_bytes = args.batch * mean_ctx * 2 * layers * nkv * d * elem
+    achieved = (weight_bytes + kv_bytes) / step_s
+    # flops of the prefill step: the linear layers on every token, causal attention, one row of logits
+    t = PREFILL_TOKENS
+    linear = 2 * t * layers * ((nh + 2 * nkv) * d * h + h * nh * d + 3 * h * inter)
+    attention = layers * 4 * nh * d * t * (t + 1) / 2
+    flops = linear + attention + 2 * vocab * h
+    line = {
+        "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (TinyLlama 1.1B)",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": args.model, "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single-gpu", "layers": layers, "layers_full": full_layers, "hidden": h,
+                   "heads": nh, "kv_heads": nkv, "head_dim": d, "intermediate": inter, "vocab": vocab,
+                   "block_size": block_size, "weights": "random", "prefill_tokens": PREFILL_TOKENS},
+        "prefill": {"value": round(t / pre_s, 1), "tokens": t, "ms": round(pre_s * 1e3, 3),
+                    "frac": round(flops / pre_s / PEAK_FLOPS[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

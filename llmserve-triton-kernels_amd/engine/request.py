@@ -1,0 +1,73 @@
+"""Records of a request's life, with the reference's names: `Request`, `Status`,
+`TokenEvent`, `EngineStats` (src/llmserve/scheduler/engine.py:36-80) and `GenerationResult`
+(src/llmserve/datatypes.py:16-27)."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from enum import Enum
+
+from ..sampling.params import SamplingParams
+
+
+class Status(Enum):
+    WAITING = "waiting"
+    RUNNING = "running"
+    FINISHED = "finished"
+
+
+@dataclass
+class Request:
+    req_id: int
+    prompt_ids: list[int]
+    params: SamplingParams
+    arrival_time: float
+    seed: int = 0
+    generated: list[int] = field(default_factory=list)
+    status: Status = Status.WAITING
+    num_computed_tokens: int = 0  # tokens of prompt + generated already in the cache
+    token_times: list[float] = field(default_factory=list)
+    finish_time: float | None = None
+    finish_reason: str | None = None  # "stop" | "length" | "abort"
+    num_preemptions: int = 0
+
+    @property
+    def all_ids(self) -> list[int]:
+        return self.prompt_ids + self.generated
+
+    @property
+    def first_token_time(self) -> float | None:
+        return self.token_times[0] if self.token_times else None
+
+
+@dataclass
+class TokenEvent:
+    req_id: int
+    token: int | None
+    finished: bool
+    finish_reason: str | None = None
+    error: str | None = None
+
+
+@dataclass
+class EngineStats:
+    steps: int = 0
+    prefill_tokens: int = 0
+    decode_tokens: int = 0
+    tokens_generated: int = 0
+    preemptions: int = 0
+
+
+@dataclass
+class GenerationResult:
+    tokens: list[int]
+    ttft_s: float  # time to first token
+    step_latencies_s: list[float] = field(default_factory=list)  # gaps between later tokens
+    total_s: float = 0.0
+    peak_memory_bytes: int = 0
+    finish_reason: str | None = None
+
+    @property
+    def decode_tokens_per_s(self) -> float:
+        total = sum(self.step_latencies_s)
+        return len(self.step_latencies_s) / total if total > 0 else 0.0

@@ -1,0 +1,6 @@
+"""Sampling: request options and the device sampler."""
+
+from .params import SamplingParams
+from .sampler import Sampler, request_seed, uniform
+
+__all__ = ["SamplingParams", "Sampler", "request_seed", "uniform"]

@@ -1,0 +1,115 @@
+"""Generation through the Python entry point and the command line, on the GPU."""
+
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_llama
+import traces
+from conftest import ROOT, TINY
+
+pytestmark = pytest.mark.gpu
+
+
+def _llm(model_dir, name, dtype, **kw):
+    from llmserve import LLM, EngineConfig
+
+    opts = dict(block_size=TINY[name][1], num_blocks=64, max_num_seqs=4, max_num_batched_tokens=24)
+    opts.update(kw)
+    return LLM(model_dir, dtype=dtype, engine=EngineConfig(**opts))
+
+
+@pytest.mark.parametrize("name,lengths,new", [("a", [5, 17, 33], 16), ("b", [1, 7, 40, 64, 100], 24)])
+def test_greedy_generation_matches_plain(model_dirs, name, lengths, new):
+    from llmserve import SamplingParams
+
+    vocab = TINY[name][0]["vocab_size"]
+    prompts = [traces.random_ids(vocab, n, 300 + i) for i, n in enumerate(lengths)]
+    cfg, w = plain_llama.read_model_dir(model_dirs[name], torch.float32)
+    want = [plain_llama.generate(cfg, w, p, new, torch.float32) for p in prompts]
+    llm = _llm(model_dirs[name], name, "float32")
+    results = llm.generate(prompts, SamplingParams(max_new_tokens=new))
+    assert [r.tokens for r in results] == want
+    assert all(r.finish_reason == "length" and len(r.step_latencies_s) == new - 1 and r.ttft_s > 0 for r in results)
+    assert llm.engine.manager.num_free_blocks == 64
+    # the baseline without a cache between tokens gives the same tokens
+    assert llm.generate_naive(prompts[1], SamplingParams(max_new_tokens=6)).tokens == want[1][:6]
+    # preemption by recompute: so few pages that requests are thrown out and come back
+    tight = _llm(model_dirs[name], name, "float32", num_blocks=max(-(-(n + new) // TINY[name][1]) for n in lengths) + 3)
+    assert [r.tokens for r in tight.generate(prompts, SamplingParams(max_new_tokens=new))] == want
+    assert tight.engine.stats.preemptions > 0
+
+
+def test_bfloat16_generation_follows_plain_logits(model_dirs):
+    """In bfloat16 greedy ties can fall either way, so the check is on the logits: every token the
+    engine picks must be (nearly) the best one under the plain bfloat16 implementation."""
+    from llmserve import SamplingParams
+
+    name = "b"
+    vocab = TINY[name][0]["vocab_size"]
+    prompt = traces.random_ids(vocab, 40, 77)
+    llm = _llm(model_dirs[name], name, "bfloat16")
+    tokens = llm.generate([prompt], SamplingParams(max_new_tokens=12))[0].tokens
+    ref = traces.plain_logits(model_dirs[name], prompt + tokens, torch.bfloat16)
+    max_tol, _ = traces.tolerance(torch.bfloat16, ref)
+    for i, tok in enumerate(tokens):
+        row = ref[len(prompt) - 1 + i]
+        assert row.max() - row[tok] <= 2 * max_tol, f"token {i} = {tok} is not near the top of the plain logits"
+
+
+def test_temperature_sampling_is_seeded_and_matches_plain_sampler(model_dirs):
+    from llmserve import SamplingParams
+    from llmserve.sampling import uniform
+
+    name = "b"
+    vocab = TINY[name][0]["vocab_size"]
+    prompts = [traces.random_ids(vocab, n, 500 + i) for i, n in enumerate([1, 7, 40, 64, 100])]
+    params = [SamplingParams(temperature=0.8, seed=40 + i, max_new_tokens=24) for i in range(5)]
+    llm = _llm(model_dirs[name], name, "float32")
+    first = [r.tokens for r in llm.generate(prompts, params)]
+    assert first == [r.tokens for r in _llm(model_dirs[name], name, "float32", max_num_batched_tokens=64)
+                     .generate(prompts, params)]
+    assert len({tuple(t) for t in first}) == 5
+    # each sampled token is what the plain sampler picks from the plain logits with the same uniform number
+    cfg, w = plain_llama.read_model_dir(model_dirs[name], torch.float32)
+    for p, sp, toks in list(zip(prompts, params, first))[:3]:
+        logits = plain_llama.forward(cfg, w, p + toks, torch.float32)
+        for i, tok in enumerate(toks):
+            row = logits[len(p) - 1 + i]
+            u = uniform(sp.seed, i)
+            cdf = plain_llama.filtered_probs(row, 0.8, 0, 1.0).cumsum(-1)
+            lo = float(cdf[tok - 1]) if tok > 0 else 0.0
+            assert lo - 1e-5 <= u < float(cdf[tok]) + 1e-5, (i, tok, u, lo, float(cdf[tok]))
+
+
+def test_eos_stops_generation(model_dirs):
+    from llmserve import SamplingParams
+
+    prompt = traces.random_ids(256, 10, 9)
+    llm = _llm(model_dirs["a"], "a", "float32")
+    first = llm.generate([prompt], SamplingParams(max_new_tokens=1))[0].tokens[0]
+    r = llm.generate([prompt], SamplingParams(max_new_tokens=50, eos_token_id=first))[0]
+    assert r.tokens == [first] and r.finish_reason == "stop"
+    with pytest.raises(ValueError):
+        llm.generate([[1] * 128], SamplingParams(max_new_tokens=5))  # beyond max_position_embeddings
+
+
+def test_command_line(model_dirs):
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    out = subprocess.run([sys.executable, "-m", "llmserve.cli", "--model", "tiny", "--max-new-tokens", "8",
+                          "--dtype", "float32"], capture_output=True, text=True, env=env, timeout=120)
+    assert out.returncode == 0, out.stderr
+    lines = out.stdout.strip().splitlines()
+    assert len(eval(lines[0])) == 8 and lines[-1].startswith("[kv_cache] ttft=") and "peak mem=" in lines[-1]
+    naive = subprocess.run([sys.executable, "-m", "llmserve.cli", "--model", "tiny", "--max-new-tokens", "8",
+                            "--dtype", "float32", "--mode", "naive"], capture_output=True, text=True, env=env, timeout=120)
+    assert naive.returncode == 0, naive.stderr
+    assert naive.stdout.strip().splitlines()[0] == lines[0]  # same tokens with and without the cache
+    folder = subprocess.run([sys.executable, "-m", "llmserve.cli", "--model", str(model_dirs["a"]), "--prompt-ids",
+                             "5,6,7,8", "--max-new-tokens", "4", "--block-size", "16", "--num-blocks", "8"],
+                            capture_output=True, text=True, env=env, timeout=120)
+    assert folder.returncode == 0, folder.stderr
+    assert len(eval(folder.stdout.strip().splitlines()[0])) == 4

@@ -1,0 +1,205 @@
+"""The scheduler's decisions, on the CPU: the real cache manager and scheduler, with the plain
+implementation standing in for the GPU step function.  Workloads are the reference's own
+(tests/test_scheduler.py there), plus portions under a token budget."""
+
+import pytest
+import torch
+
+import plain_llama
+from conftest import TINY_A
+from fakes import PlainRunner, PlainSampler
+from llmserve.engine.scheduler import ContinuousBatchingEngine
+from llmserve.sampling import SamplingParams
+from llmserve.weights import random_tensors
+
+
+@pytest.fixture(scope="module")
+def weights():
+    from llmserve.config import architecture_of
+    from llmserve.parts.model import Model
+    from llmserve.parts.registry import BuildContext
+
+    arch = architecture_of(TINY_A)
+    model = Model(arch.build_spec(arch.config_class.from_dict(TINY_A)), BuildContext(torch.float32, torch.device("cpu")))
+    return random_tensors(model.param_infos(), 21, torch.float32)
+
+
+def prompt(n, seed):
+    return torch.randint(0, TINY_A["vocab_size"], (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def engine(weights, *, num_blocks=64, block_size=4, max_batch=4, budget=2048, chunk=None):
+    runner = PlainRunner(TINY_A, weights, num_blocks, block_size)
+    return ContinuousBatchingEngine(runner, PlainSampler(), max_num_seqs=max_batch, max_num_batched_tokens=budget,
+                                    max_prefill_chunk=chunk)
+
+
+_REFERENCE = {}
+
+
+def reference(weights, p, max_new):
+    key = (tuple(p), max_new)
+    if key not in _REFERENCE:
+        _REFERENCE[key] = plain_llama.generate(TINY_A, weights, p, max_new, torch.float32)
+    return _REFERENCE[key]
+
+
+WORKLOAD = [(5, 9), (13, 4), (8, 12), (3, 7), (17, 5), (6, 10)]  # (prompt_len, max_new)
+
+
+@pytest.mark.parametrize("budget,chunk", [(2048, None), (16, None), (8, 5), (4, 2)])
+def test_batched_outputs_equal_independent_generation(weights, budget, chunk):
+    eng = engine(weights, max_batch=3, budget=budget, chunk=chunk)
+    prompts = [prompt(n, 100 + i) for i, (n, _) in enumerate(WORKLOAD)]
+    ids = [eng.add_request(p, SamplingParams(max_new_tokens=m)) for p, (_, m) in zip(prompts, WORKLOAD)]
+    done = eng.run_until_complete()
+    for rid, p, (_, m) in zip(ids, prompts, WORKLOAD):
+        assert done[rid].generated == reference(weights, p, m), f"request {rid}"
+        assert done[rid].finish_reason == "length"
+    assert eng.manager.num_free_blocks == eng.manager.num_blocks and eng.manager.num_free_slots == eng.manager.max_seqs
+    assert all(sum(sizes) <= budget for sizes in eng.runner.step_sizes)
+    if chunk:
+        assert all(n <= chunk for sizes in eng.runner.step_sizes for n in sizes)
+    assert eng.stats.tokens_generated == sum(m for _, m in WORKLOAD)
+
+
+def test_portions_run_beside_decoding(weights):
+    eng = engine(weights, max_batch=2, budget=6)
+    a = eng.add_request(prompt(4, 1), SamplingParams(max_new_tokens=8))
+    eng.step()
+    b = eng.add_request(prompt(14, 2), SamplingParams(max_new_tokens=3))
+    eng.step()
+    assert eng.runner.step_sizes[-1] == [1, 5]  # one decoded token of a, a portion of b's prompt
+    eng.step()
+    assert eng.runner.step_sizes[-1] == [1, 5]
+    done = eng.run_until_complete()
+    assert done[a].generated == reference(weights, prompt(4, 1), 8)
+    assert done[b].generated == reference(weights, prompt(14, 2), 3)
+
+
+def test_requests_arriving_mid_flight_join_the_running_batch(weights):
+    eng = engine(weights, max_batch=4)
+    p0, p1 = prompt(6, 1), prompt(9, 2)
+    r0 = eng.add_request(p0, SamplingParams(max_new_tokens=10))
+    for _ in range(4):
+        eng.step()
+    assert len(eng.running) == 1
+    r1 = eng.add_request(p1, SamplingParams(max_new_tokens=6))
+    eng.step()
+    assert len(eng.running) == 2
+    done = eng.run_until_complete()
+    assert done[r0].generated == reference(weights, p0, 10) and done[r1].generated == reference(weights, p1, 6)
+
+
+def test_admission_is_in_order_and_keeps_headroom(weights):
+    eng = engine(weights, num_blocks=8, block_size=4, max_batch=4)
+    big = eng.add_request(prompt(20, 1), SamplingParams(max_new_tokens=4))  # 5 pages now, 6 at the end
+    eng.step()
+    assert [r.req_id for r in eng.running] == [big]
+    eng.add_request(prompt(12, 2), SamplingParams(max_new_tokens=2))  # 3 pages + 1 spare page per live request > 3 free
+    small = eng.add_request(prompt(2, 3), SamplingParams(max_new_tokens=2))  # would fit, but may not overtake
+    eng.step()
+    assert [r.req_id for r in eng.running] == [big] and len(eng.waiting) == 2
+    done = eng.run_until_complete()
+    assert done[small].generated == reference(weights, prompt(2, 3), 2)
+
+
+def test_preemption_recompute_preserves_greedy_outputs(weights):
+    # 14 pages of 4 and four (6, 14) requests cannot all grow (tests/test_scheduler.py:69-82 there)
+    eng = engine(weights, num_blocks=14, block_size=4, max_batch=4)
+    work = [(6, 14)] * 4
+    prompts = [prompt(n, 50 + i) for i, (n, _) in enumerate(work)]
+    ids = [eng.add_request(p, SamplingParams(max_new_tokens=m)) for p, (_, m) in zip(prompts, work)]
+    done = eng.run_until_complete()
+    assert eng.stats.preemptions > 0, "the test must exercise preemption"
+    assert sum(r.num_preemptions for r in done.values()) == eng.stats.preemptions
+    for rid, p, (_, m) in zip(ids, prompts, work):
+        assert done[rid].generated == reference(weights, p, m)
+    assert eng.manager.num_free_blocks == eng.manager.num_blocks
+    eng.manager.check_invariants()
+
+
+def test_preemption_takes_the_newest_and_requeues_it_first(weights):
+    eng = engine(weights, num_blocks=6, block_size=4, max_batch=3)
+    ids = [eng.add_request(prompt(4, 70 + i), SamplingParams(max_new_tokens=12)) for i in range(3)]
+    while eng.stats.preemptions == 0:
+        eng.step()
+    assert eng.waiting[0].req_id == ids[-1] or eng.waiting[0].req_id == ids[1]
+    assert eng.waiting[0].num_computed_tokens == 0 and eng.waiting[0].num_preemptions == 1
+    assert ids[0] in [r.req_id for r in eng.running]  # the oldest keeps running
+    eng.run_until_complete()
+    assert eng.manager.num_free_blocks == 6
+
+
+def test_eos_finishes_early_and_frees_blocks(weights):
+    p = prompt(7, 9)
+    first = reference(weights, p, 1)[0]
+    eng = engine(weights)
+    rid = eng.add_request(p, SamplingParams(max_new_tokens=20, eos_token_id=first))
+    done = eng.run_until_complete()
+    assert done[rid].generated == [first] and done[rid].finish_reason == "stop"
+    assert eng.manager.num_free_blocks == eng.manager.num_blocks
+
+
+def test_abort_waiting_and_running(weights):
+    eng = engine(weights, max_batch=1)
+    a = eng.add_request(prompt(5, 1), SamplingParams(max_new_tokens=30))
+    b = eng.add_request(prompt(5, 2), SamplingParams(max_new_tokens=30))
+    eng.step()
+    eng.step()
+    eng.abort(b)
+    eng.abort(a)
+    events = eng.step()
+    assert {e.req_id for e in events if e.finished} == {a, b}
+    assert all(e.token is None and e.finish_reason == "abort" for e in events)
+    assert not eng.has_unfinished() and eng.manager.num_free_blocks == eng.manager.num_blocks
+    assert eng.finished[a].finish_reason == "abort"
+
+
+def test_validate_rejects_impossible_requests(weights):
+    eng = engine(weights, num_blocks=4, block_size=4)  # 16 slots in all
+    with pytest.raises(ValueError, match="KV blocks"):
+        eng.add_request([1] * 10, SamplingParams(max_new_tokens=10))
+    with pytest.raises(ValueError, match="model limit"):
+        eng.add_request([1] * 200, SamplingParams(max_new_tokens=5))
+    with pytest.raises(ValueError, match="at least one token"):
+        eng.add_request([], SamplingParams(max_new_tokens=5))
+    with pytest.raises(ValueError, match="max_new_tokens"):
+        eng.add_request([1], SamplingParams(max_new_tokens=0))
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.add_request([999], SamplingParams(max_new_tokens=1))
+
+
+def test_seeded_sampling_is_reproducible_and_survives_batching(weights):
+    params = SamplingParams(temperature=0.9, top_k=20, seed=1234, max_new_tokens=12)
+    p = prompt(6, 3)
+    alone = []
+    for _ in range(2):
+        eng = engine(weights)
+        rid = eng.add_request(p, params)
+        alone.append(eng.run_until_complete()[rid].generated)
+    assert alone[0] == alone[1]
+    # the same request in a crowd, cut into portions, with a pool that forces preemption
+    eng = engine(weights, num_blocks=12, block_size=4, max_batch=3, budget=5)
+    others = [eng.add_request(prompt(5, 80 + i), SamplingParams(temperature=0.7, seed=i, max_new_tokens=14)) for i in range(2)]
+    rid = eng.add_request(p, params)
+    done = eng.run_until_complete()
+    assert done[rid].generated == alone[0] and len(done[others[0]].generated) == 14
+    assert len(set(alone[0])) > 1
+
+
+def test_snapshot_and_events(weights):
+    eng = engine(weights)
+    rid = eng.add_request(prompt(5, 4), SamplingParams(max_new_tokens=3))
+    events = eng.step()
+    assert [(e.req_id, e.finished) for e in events] == [(rid, False)]
+    snap = eng.snapshot()
+    assert snap["running"] == 1 and snap["waiting"] == 0 and snap["free_blocks"] < snap["total_blocks"]
+    assert 0 < snap["kv_utilization"] <= 1 and snap["prefill_tokens"] == 5
+    events = eng.step() + eng.step()
+    assert events[-1].finished and events[-1].finish_reason == "length"
+    assert eng.snapshot()["decode_tokens"] == 2
+    eng.add_request(prompt(5, 5), SamplingParams(max_new_tokens=3))
+    eng.step()
+    eng.reset()
+    assert not eng.has_unfinished() and eng.manager.num_free_blocks == eng.manager.num_blocks
