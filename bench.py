@@ -62,11 +62,15 @@ def main() -> int:
     elem = 2 if args.dtype == "bfloat16" else 4
     block_size = 16
     max_batch = 64 if not args.no_points else args.batch
-    decode_len = args.context + args.warmup + args.steps + 2
+    budget = max(PREFILL_TOKENS, max_batch)
+    # requests whose prompt went in first decode while the others' prompts still go in
+    slack = -(-max_batch * args.context // budget) + 2
+    new_tokens = args.warmup + args.steps + slack
+    decode_len = args.context + new_tokens + 1
     cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], PREFILL_TOKENS + 8, decode_len)
     pages = max(max_batch * -(-decode_len // block_size), -(-(PREFILL_TOKENS + 8) // block_size)) + 16
     engine_cfg = EngineConfig(dtype=args.dtype, block_size=block_size, num_blocks=pages, max_num_seqs=max_batch,
-                              max_num_batched_tokens=max(PREFILL_TOKENS, max_batch), seed=0)
+                              max_num_batched_tokens=budget, seed=0)
     runner = ModelRunner.from_random(cfg, seed=0, engine_config=engine_cfg)
     sampler = Sampler(runner.device)
     gen = torch.Generator().manual_seed(0)
@@ -79,7 +83,7 @@ def main() -> int:
         eng = ContinuousBatchingEngine(runner, sampler, max_num_seqs=batch,
                                        max_num_batched_tokens=engine_cfg.max_num_batched_tokens)
         for p in prompts(batch, args.context):
-            eng.add_request(p, SamplingParams(max_new_tokens=args.warmup + args.steps + 1))
+            eng.add_request(p, SamplingParams(max_new_tokens=new_tokens))
         while eng.waiting or any(len(r.all_ids) - r.num_computed_tokens > 1 for r in eng.running):
             eng.step()  # prompts in
         for _ in range(args.warmup):

@@ -37,10 +37,22 @@ def test_greedy_generation_matches_plain(model_dirs, name, lengths, new):
     assert llm.engine.manager.num_free_blocks == 64
     # the baseline without a cache between tokens gives the same tokens
     assert llm.generate_naive(prompts[1], SamplingParams(max_new_tokens=6)).tokens == want[1][:6]
-    # preemption by recompute: so few pages that requests are thrown out and come back
-    tight = _llm(model_dirs[name], name, "float32", num_blocks=max(-(-(n + new) // TINY[name][1]) for n in lengths) + 3)
-    assert [r.tokens for r in tight.generate(prompts, SamplingParams(max_new_tokens=new))] == want
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_preemption_by_recompute_keeps_greedy_tokens(model_dirs, name):
+    """14 pages of 4 tokens and four requests of 6 + 14 tokens cannot all grow: some are thrown
+    out and recomputed (the reference's case, tests/test_scheduler.py:69-82 there)."""
+    from llmserve import SamplingParams
+
+    vocab = TINY[name][0]["vocab_size"]
+    prompts = [traces.random_ids(vocab, 6, 50 + i) for i in range(4)]
+    cfg, w = plain_llama.read_model_dir(model_dirs[name], torch.float32)
+    want = [plain_llama.generate(cfg, w, p, 14, torch.float32) for p in prompts]
+    tight = _llm(model_dirs[name], name, "float32", block_size=4, num_blocks=14)
+    assert [r.tokens for r in tight.generate(prompts, SamplingParams(max_new_tokens=14))] == want
     assert tight.engine.stats.preemptions > 0
+    assert tight.engine.manager.num_free_blocks == 14
 
 
 def test_bfloat16_generation_follows_plain_logits(model_dirs):
