@@ -245,6 +245,45 @@ def gemm_fma(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Te
     return out
 
 
+def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the matrix-core kernels take these operands (else `gemm_fma` does)."""
+    k = a.shape[1]
+    return (a.dtype == torch.bfloat16 and k % 8 == 0 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
+def gemm_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
+              kernel: str | None = None) -> torch.Tensor:
+    """out[M,N] (bfloat16 or float32) = a[M,K] w[N,K]^T (+ bias) on the matrix cores, 32-bit sums.
+    `kernel`: "skinny" (M <= 64, weight streamed once) or "tile"; default by M."""
+    dev = _dev(out, a, w, bias)
+    if a.dim() != 2 or a.stride(1) != 1 or out.dim() != 2 or out.stride(1) != 1:
+        raise ValueError("a and out must be 2-d with unit inner stride")
+    _rows(w, "w", a.shape[1])
+    m, k = a.shape
+    n = w.shape[0]
+    if tuple(out.shape) != (m, n):
+        raise ValueError(f"out shape {tuple(out.shape)} is not {(m, n)}")
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise ValueError("gemm_bf16 takes bfloat16 operands")
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous bfloat16 vector of N elements")
+    if out.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("gemm_bf16 stores bfloat16 or float32")
+    if not gemm_bf16_supported(a, w):
+        raise ValueError(f"gemm_bf16 needs K ({k}) and the row stride of a ({a.stride(0)}) to be multiples of 8 "
+                         "and 16-byte aligned operands")
+    if m == 0:
+        return out
+    kernel = kernel or ("skinny" if m <= 64 else "tile")
+    if kernel == "skinny" and m > 64:
+        raise ValueError("the skinny kernel takes at most 64 rows")
+    fn = load("gemm_mfma").llms_gemm_bf16_skinny if kernel == "skinny" else load("gemm_mfma").llms_gemm_bf16_tile
+    _check(fn(c_int(_code(out)), _ptr(out), _ptr(a), _ptr(w), _ptr(bias), c_int(m), c_int(n), c_int(k),
+              c_int(a.stride(0)), c_int(out.stride(0)), _stream(dev)), f"gemm_bf16[{kernel}]")
+    return out
+
+
 # ------------------------------------------------------------------------------ attention
 
 

@@ -21,6 +21,6 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     if m == 0:
         return out
-    if x.dtype == torch.bfloat16 and ops.has_mfma():
+    if x.dtype == torch.bfloat16 and ops.gemm_bf16_supported(x, weight):
         return ops.gemm_bf16(out, x, weight, bias)
     return ops.gemm_fma(out, x, weight, bias)

@@ -1,0 +1,321 @@
+"""Each HIP kernel alone against a plain 32-bit reference of the same operation, at sizes other
+than the tiny models': ragged widths, head sizes in steps of 16, every group ratio, odd
+vocabularies, any page size."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_llama
+from kernel_helpers import attention_reference, bf16_round, make_paged
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def ops():
+    from llmserve.ops import library
+
+    return library
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    return scale * torch.randn(*shape, generator=torch.Generator().manual_seed(seed))
+
+
+def ulp(dtype, ref):
+    """One rounding of the largest value for bfloat16; accumulated 32-bit rounding otherwise."""
+    scale = max(1e-3, float(ref.abs().max()))
+    return scale * (2.0 ** -7 if dtype == torch.bfloat16 else 2e-6)
+
+
+# ------------------------------------------------------------------ row-wise kernels
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_gather(dtype):
+    table = rnd(333, 100, seed=1).to(dtype)
+    ids = torch.tensor([0, 332, 7, 7, 100], dtype=torch.int32)
+    out = torch.empty(5, 100, dtype=dtype, device=DEV)
+    ops().embed_gather(out, table.to(DEV), ids.to(DEV))
+    assert torch.equal(out.cpu(), table[ids.long()])
+    bad = torch.tensor([5, 333, -1], dtype=torch.int32)
+    out = torch.zeros(3, 100, dtype=dtype, device=DEV)
+    ops().embed_gather(out, table.to(DEV), bad.to(DEV))
+    assert torch.equal(out[0].cpu(), table[5]) and out[1:].isnan().all()  # a bad id is loud, not a stray read
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,eps", [(64, 1e-5), (100, 1e-6), (2048, 1e-5), (5000, 1e-6)])
+def test_rmsnorm(dtype, hidden, eps):
+    x = rnd(9, hidden, seed=2, scale=3.0).to(dtype)
+    delta = rnd(9, hidden, seed=3).to(dtype)
+    w = (1 + 0.1 * rnd(hidden, seed=4)).to(dtype)
+    ref = plain_llama.rms_norm(x, w, eps).float()
+    out = ops().rmsnorm(torch.empty_like(x, device=DEV), x.to(DEV), w.to(DEV), eps)
+    assert (out.float().cpu() - ref).abs().max() <= ulp(dtype, ref)
+    # residual sum in 32-bit, rounded once, written back, then normed
+    summed = (x.float() + delta.float()).to(dtype)
+    ref = plain_llama.rms_norm(summed, w, eps).float()
+    resid = x.clone().to(DEV)
+    out = ops().rmsnorm(torch.empty_like(resid), resid, w.to(DEV), eps, delta=delta.to(DEV), resid_out=resid)
+    assert torch.equal(resid.cpu(), summed)
+    assert (out.float().cpu() - ref).abs().max() <= ulp(dtype, ref)
+    # only some rows, nothing written back
+    rows = torch.tensor([8, 0, 3], dtype=torch.int32)
+    resid = x.clone().to(DEV)
+    out = torch.empty(3, hidden, dtype=dtype, device=DEV)
+    ops().rmsnorm(out, resid, w.to(DEV), eps, delta=delta.to(DEV), rows=rows.to(DEV))
+    assert (out.float().cpu() - ref[rows.long()]).abs().max() <= ulp(dtype, ref)
+    assert torch.equal(resid.cpu(), x)
+
+
+def test_rmsnorm_tiny_inputs_feel_eps():
+    x = rnd(2, 96, seed=5, scale=1e-3)
+    w = torch.ones(96)
+    for eps in (1e-5, 1e-6):
+        out = ops().rmsnorm(torch.empty(2, 96, device=DEV), x.to(DEV), w.to(DEV), eps)
+        assert torch.allclose(out.cpu(), plain_llama.rms_norm(x, w, eps), atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,bs,theta", [(4, 2, 16, 16, 1e4), (3, 1, 32, 8, 5e5), (8, 8, 64, 4, 1e4),
+                                               (5, 5, 48, 1, 1e6), (16, 2, 128, 32, 1e4)])
+def test_rope_store(dtype, nh, nkv, d, bs, theta):
+    n = 7
+    width = (nh + 2 * nkv) * d
+    qkv = rnd(n, width, seed=6).to(dtype)
+    positions = torch.tensor([0, 1, 2, 500, 1999, 37, 4095], dtype=torch.int32)
+    pages = 6
+    others = [s for s in torch.randperm(bs * pages, generator=torch.Generator().manual_seed(d)).tolist()
+              if s not in (0, bs * pages - 1)]
+    slots = torch.tensor([others[0], 0, bs * pages - 1, -1, others[1], others[2], others[3]], dtype=torch.int32)
+    inv_freq = 1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    k_pool = torch.full((pages, nkv, bs, d), 7.0, dtype=dtype, device=DEV)
+    v_pool = torch.full((pages, nkv, d, bs), 7.0, dtype=dtype, device=DEV)
+    dev_qkv = qkv.clone().to(DEV)
+    ops().rope_store(dev_qkv, inv_freq.to(DEV), positions.to(DEV), slots.to(DEV), k_pool, v_pool, nh, nkv, d, bs)
+    got = dev_qkv.cpu()
+    cos, sin = plain_llama.rope_cos_sin(positions, d, theta)
+    q = qkv[:, : nh * d].view(n, nh, d).transpose(0, 1)
+    k = qkv[:, nh * d: (nh + nkv) * d].view(n, nkv, d).transpose(0, 1)
+    v = qkv[:, (nh + nkv) * d:].view(n, nkv, d)
+    q_ref = plain_llama.apply_rope(q, cos, sin).transpose(0, 1).reshape(n, nh * d)
+    k_ref = plain_llama.apply_rope(k, cos, sin).transpose(0, 1)  # [n, nkv, d]
+    tol = ulp(dtype, q_ref.float()) if dtype == torch.bfloat16 else 2e-4 * float(q_ref.abs().max())  # sin/cos of large angles
+    assert (got[:, : nh * d].float() - q_ref.float()).abs().max() <= tol
+    assert torch.equal(got[:, (nh + nkv) * d:], qkv[:, (nh + nkv) * d:])  # v is left alone
+    kp, vp = k_pool.cpu(), v_pool.cpu()
+    written = torch.zeros(pages, bs, dtype=torch.bool)
+    for i, s in enumerate(slots.tolist()):
+        if s < 0:
+            continue
+        page, off = divmod(s, bs)
+        written[page, off] = True
+        assert (kp[page, :, off].float() - k_ref[i].float()).abs().max() <= tol
+        assert torch.equal(vp[page, :, :, off], v[i])
+    assert (kp.transpose(1, 2)[~written] == 7).all() and (vp.permute(0, 3, 1, 2)[~written] == 7).all()
+    # without frequencies nothing is rotated, keys are stored as they are
+    dev_qkv = qkv.clone().to(DEV)
+    ops().rope_store(dev_qkv, None, positions.to(DEV), slots.to(DEV), k_pool, v_pool, nh, nkv, d, bs)
+    assert torch.equal(dev_qkv.cpu(), qkv)
+    page, off = divmod(int(slots[0]), bs)
+    assert torch.equal(k_pool.cpu()[page, :, off], k.transpose(0, 1)[0])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("inter", [176, 5632, 33])
+def test_silu_mul(dtype, inter):
+    gu = rnd(5, 2 * inter, seed=7, scale=4.0).to(dtype)
+    ref = (plain_llama.silu(gu[:, :inter]) * gu[:, inter:]).float()
+    out = ops().silu_mul(torch.empty(5, inter, dtype=dtype, device=DEV), gu.to(DEV))
+    assert (out.float().cpu() - ref).abs().max() <= ulp(dtype, ref)
+
+
+# ------------------------------------------------------------------ matrix products
+@pytest.mark.parametrize("m,n,k", [(1, 256, 64), (5, 333, 96), (64, 100, 176), (130, 65, 17), (300, 513, 1000)])
+def test_gemm_fma(m, n, k):
+    a, w, b = rnd(m, k, seed=8), rnd(n, k, seed=9), rnd(n, seed=10)
+    ref = a.double() @ w.double().t() + b.double()
+    out = ops().gemm_fma(torch.empty(m, n, device=DEV), a.to(DEV), w.to(DEV), b.to(DEV))
+    assert (out.cpu().double() - ref).abs().max() <= 2e-6 * math.sqrt(k) * float(ref.abs().max())
+    ab, wb = a.bfloat16(), w.bfloat16()
+    ref = ab.double() @ wb.double().t()
+    out = ops().gemm_fma(torch.empty(m, n, device=DEV), ab.to(DEV), wb.to(DEV))  # bfloat16 in, 32-bit out
+    assert (out.cpu().double() - ref).abs().max() <= 2e-6 * math.sqrt(k) * float(ref.abs().max())
+    out = ops().gemm_fma(torch.empty(m, n, dtype=torch.bfloat16, device=DEV), ab.to(DEV), wb.to(DEV))
+    assert (out.float().cpu().double() - ref).abs().max() <= 2.0 ** -8 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("kernel,m", [("skinny", 1), ("skinny", 7), ("skinny", 16), ("skinny", 17), ("skinny", 33),
+                                      ("skinny", 64), ("tile", 5), ("tile", 65), ("tile", 128), ("tile", 300)])
+@pytest.mark.parametrize("n,k", [(16, 64), (333, 96), (100, 176), (2056, 2048), (512, 5632)])
+def test_gemm_bf16(kernel, m, n, k):
+    a, w, b = rnd(m, k, seed=11).bfloat16(), rnd(n, k, seed=12).bfloat16(), rnd(n, seed=13).bfloat16()
+    ref = a.double() @ w.double().t() + b.double()
+    out = ops().gemm_bf16(torch.empty(m, n, device=DEV), a.to(DEV), w.to(DEV), b.to(DEV), kernel=kernel)
+    assert (out.cpu().double() - ref).abs().max() <= 2e-6 * math.sqrt(k) * float(ref.abs().max())
+    out = ops().gemm_bf16(torch.empty(m, n, dtype=torch.bfloat16, device=DEV), a.to(DEV), w.to(DEV), kernel=kernel)
+    ref = a.double() @ w.double().t()
+    assert (out.float().cpu().double() - ref).abs().max() <= 2.0 ** -8 * float(ref.abs().max())
+
+
+def test_gemm_bf16_rows_do_not_depend_on_the_batch():
+    """A row's result is the same bits whatever else is in the batch (same kernel)."""
+    a, w = rnd(40, 2048, seed=14).bfloat16().to(DEV), rnd(320, 2048, seed=15).bfloat16().to(DEV)
+    full = ops().gemm_bf16(torch.empty(40, 320, device=DEV), a, w, kernel="skinny")
+    one = ops().gemm_bf16(torch.empty(1, 320, device=DEV), a[17:18].contiguous(), w, kernel="skinny")
+    assert torch.equal(full[17], one[0])
+
+
+def test_gemm_bf16_refuses_what_it_cannot_take():
+    a, w = torch.zeros(4, 100, dtype=torch.bfloat16, device=DEV), torch.zeros(8, 100, dtype=torch.bfloat16, device=DEV)
+    assert not ops().gemm_bf16_supported(a, w)
+    with pytest.raises(ValueError, match="multiples of 8"):
+        ops().gemm_bf16(torch.empty(4, 8, device=DEV), a, w)
+    with pytest.raises(ValueError, match="at most 64"):
+        ops().gemm_bf16(torch.empty(70, 8, device=DEV), torch.zeros(70, 64, dtype=torch.bfloat16, device=DEV),
+                        torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV), kernel="skinny")
+
+
+# ------------------------------------------------------------------ attention
+def run_attention(fn, dtype, nh, nkv, d, bs, lens, new, window=0, seed=0, craft=None):
+    """Requests of lengths `lens`, the last `new[b]` tokens of each are this step's queries."""
+    qs = [rnd(s, nh, d, seed=seed + 3 * b) for b, s in enumerate(lens)]
+    ks = [rnd(s, nkv, d, seed=seed + 3 * b + 1) for b, s in enumerate(lens)]
+    vs = [rnd(s, nkv, d, seed=seed + 3 * b + 2) for b, s in enumerate(lens)]
+    if craft:
+        craft(qs, ks, vs)
+    qs, ks, vs = ([t.to(dtype) for t in ts] for ts in (qs, ks, vs))
+    k_pool, v_pool, tables = make_paged(ks, vs, bs, dtype, seed=seed)
+    q_rows, token_seq, positions, refs = [], [], [], []
+    for b, (s, n) in enumerate(zip(lens, new)):
+        rows = list(range(s - n, s))
+        q_rows.append(qs[b][rows].reshape(n, nh * d))
+        token_seq += [b] * n
+        positions += rows
+        refs.append(attention_reference(qs[b], ks[b], vs[b], rows, window or None))
+    q = torch.cat(q_rows).contiguous().to(DEV)
+    out = torch.empty(q.shape[0], nh * d, dtype=dtype, device=DEV)
+    fn(out, q, k_pool.to(DEV), v_pool.to(DEV), tables.to(DEV), torch.tensor(token_seq, dtype=torch.int32, device=DEV),
+       torch.tensor(positions, dtype=torch.int32, device=DEV), nh, nkv, d, bs, window)
+    ref = torch.cat(refs)
+    got = out.float().cpu()
+    assert torch.isfinite(got).all(), "read a slot that was never written"
+    return got, ref
+
+
+ATT_CASES = [  # nh, nkv, d, bs, lens, new, window
+    (4, 2, 16, 16, [5, 17, 33], [5, 17, 33], 0),
+    (3, 1, 32, 8, [1, 7, 40, 100], [1, 1, 1, 1], 0),
+    (8, 1, 64, 16, [300, 64, 129], [1, 24, 2], 0),
+    (6, 2, 80, 4, [70, 19], [3, 19], 0),
+    (4, 4, 128, 32, [257, 31], [1, 31], 0),
+    (2, 1, 256, 16, [90], [7], 0),
+    (32, 4, 64, 16, [600], [1], 0),
+    (4, 2, 48, 1, [37], [37], 0),
+    (4, 2, 32, 8, [150, 40], [30, 1], 16),
+    (3, 3, 16, 16, [100], [100], 7),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", ATT_CASES)
+def test_attention_wave(dtype, case):
+    nh, nkv, d, bs, lens, new, window = case
+    got, ref = run_attention(ops().attention_wave, dtype, nh, nkv, d, bs, lens, new, window, seed=20)
+    tol = 2.0 ** -7 * float(ref.abs().max()) if dtype == torch.bfloat16 else 2e-5
+    assert (got - ref).abs().max() <= tol
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("needle", [0, 15, 16, 299, 300 - 17, 141])
+def test_attention_wave_finds_one_far_key(dtype, needle):
+    """One key among hundreds gets all the weight (query and key scaled up): the output must be
+    that key's value, wherever in the pages it lies."""
+    def craft(qs, ks, vs):
+        qs[0][-1] = 0
+        qs[0][-1, :, 0] = 12.0
+        ks[0][:, :, 0] = 0
+        ks[0][needle, :, 0] = 12.0
+
+    got, ref = run_attention(ops().attention_wave, dtype, 8, 2, 64, 16, [300], [1], 0, seed=30, craft=craft)
+    assert (got - ref).abs().max() <= (2.0 ** -7 * float(ref.abs().max()) if dtype == torch.bfloat16 else 2e-5)
+
+
+def test_attention_wave_window_edge():
+    """The key just inside the window counts, the key just outside does not."""
+    for needle, inside in ((100 - 8, False), (100 - 7, True)):
+        def craft(qs, ks, vs):
+            qs[0][-1] = 0
+            qs[0][-1, :, 1] = 10.0
+            ks[0][:, :, 1] = 0
+            ks[0][needle, :, 1] = 10.0
+            vs[0][needle] = 5.0
+
+        got, ref = run_attention(ops().attention_wave, torch.float32, 2, 1, 32, 8, [101], [1], 8, seed=31, craft=craft)
+        assert (got - ref).abs().max() <= 2e-5
+        assert (got.mean() > 4.0) == inside
+
+
+# ------------------------------------------------------------------ sampling
+@pytest.mark.parametrize("vocab", [5, 333, 32000, 50257])
+def test_argmax_lowest_index_wins(vocab):
+    logits = rnd(6, vocab, seed=40)
+    logits[1, 3 % vocab] = logits[1, vocab - 1] = 50.0  # a tie: the lower index wins
+    logits[2, vocab - 1] = 60.0
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    ops().sample_rows(out, logits.to(DEV))
+    want = [int(torch.argmax(row)) for row in logits]
+    want[1] = 3 % vocab
+    assert out.tolist() == want
+
+
+def test_sampler_reference_vector():
+    logits = torch.tensor([[0.1, 3.0, 0.2, 2.9, -1.0]] * 40, device=DEV)
+    u = torch.linspace(0, 0.999, 40, device=DEV)
+    ones, out = torch.ones(40, device=DEV), torch.empty(40, dtype=torch.int32, device=DEV)
+    k = lambda v: torch.full((40,), v, dtype=torch.int32, device=DEV)  # noqa: E731
+    ops().sample_rows(out, logits, temperature=ones, top_k=k(1), top_p=ones, uniform=u)
+    assert set(out.tolist()) == {1}
+    ops().sample_rows(out, logits, temperature=ones, top_k=k(0), top_p=torch.full((40,), 1e-6, device=DEV), uniform=u)
+    assert set(out.tolist()) == {1}
+    ops().sample_rows(out, logits, temperature=ones, top_k=k(2), top_p=ones, uniform=u)
+    assert set(out.tolist()) == {1, 3}
+    ops().sample_rows(out, logits, temperature=torch.zeros(40, device=DEV), top_k=k(0), top_p=ones, uniform=u)
+    assert set(out.tolist()) == {1}
+
+
+@pytest.mark.parametrize("vocab,temperature,top_k,top_p", [(333, 0.8, 0, 1.0), (32000, 1.0, 50, 1.0),
+                                                           (32000, 0.7, 0, 0.9), (5000, 1.3, 40, 0.5),
+                                                           (50257, 1.0, 0, 1.0)])
+def test_sample_rows_inverts_the_plain_cdf(vocab, temperature, top_k, top_p):
+    rows = 24
+    logits = rnd(rows, vocab, seed=41, scale=3.0)
+    u = torch.rand(rows, generator=torch.Generator().manual_seed(42))
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    ops().sample_rows(out, dev(logits), temperature=dev(torch.full((rows,), temperature)),
+                      top_k=dev(torch.full((rows,), top_k, dtype=torch.int32)),
+                      top_p=dev(torch.full((rows,), top_p)), uniform=dev(u))
+    for r, tok in enumerate(out.tolist()):
+        probs = plain_llama.filtered_probs(logits[r], temperature, top_k, top_p)
+        assert probs[tok] > 0, f"row {r}: token {tok} was filtered out by the plain sampler"
+        cdf = probs.cumsum(-1)
+        lo = float(cdf[tok - 1]) if tok > 0 else 0.0
+        assert lo - 1e-5 <= float(u[r]) <= float(cdf[tok]) + 1e-5, (r, tok, float(u[r]), lo, float(cdf[tok]))
+
+
+def test_sample_rows_mixed_batch_and_frequencies():
+    logits = torch.tensor([[0.0, 1.0, 2.0, 0.5]], device=DEV).repeat(4000, 1)
+    u = torch.rand(4000, generator=torch.Generator().manual_seed(43)).to(DEV)
+    temp = torch.full((4000,), 0.7, device=DEV)
+    temp[::2] = 0.0  # greedy rows beside sampled ones
+    out = torch.empty(4000, dtype=torch.int32, device=DEV)
+    ops().sample_rows(out, logits, temperature=temp, uniform=u)
+    got = out.cpu()
+    assert (got[::2] == 2).all()
+    freq = torch.bincount(got[1::2].long(), minlength=4).float() / 2000
+    assert torch.allclose(freq, torch.softmax(logits[0].cpu() / 0.7, -1), atol=0.04)
