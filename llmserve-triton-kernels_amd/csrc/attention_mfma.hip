@@ -1,0 +1,370 @@
+// bfloat16 causal attention over the paged cache on the gfx950 matrix cores, for prompts,
+// portions of prompts and decoded tokens alike.
+//
+// A wave owns a *column group*: up to 16 (token, query head) pairs of one request that share
+// one KV head (for 8 heads per KV head: 2 tokens x 8 heads; for 1: 16 tokens; for 16: 1 token),
+// and walks that request's keys in tiles of 32 through its block table:
+//   S^T[key, col] = K[key, :] . Q[col, :]      v_mfma_f32_16x16x32_bf16, A = key rows straight from
+//                                              the cache, B = queries held in registers
+//   online softmax per column in 32-bit        (max, sum, rescale), masked by position and window
+//   O^T[d, col] += V^T[d, key] . P^T[key, col] A = values, which the cache stores transposed inside
+//                                              a page, so 8 keys of one dimension are one 16-byte load
+// Nothing goes through LDS on the way to the matrix instruction.  The row-to-key assignment of
+// the two S^T tiles is chosen so that each lane ends up with 8 consecutive keys, which is what
+// the B operand of the second product wants: no exchange between lanes.
+//
+// Two arrangements of the 4 waves of a workgroup:
+//   SPLIT_WAVES = false (prompts): 4 consecutive column groups of one request.
+//   SPLIT_WAVES = true  (decoding): one column group; the key tiles are dealt to the 4 waves, and
+//     optionally to `num_splits` workgroups whose partial results a second kernel merges.
+// All merges run in a fixed order, so a token's result does not depend on the batch around it.
+//
+// Needs block_size % 8 == 0, head_dim % 16 == 0 and <= 256, 16-byte aligned rows.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+
+// Keep elements [first, last) of 8 packed bfloat16, zero the rest.
+__device__ __forceinline__ uint4 keep_elements(uint4 v, int first, int last) {
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = (2 * i >= first && 2 * i < last) ? 0x0000ffffu : 0u;
+        const uint32_t hi = (2 * i + 1 >= first && 2 * i + 1 < last) ? 0xffff0000u : 0u;
+        w[i] &= (lo | hi);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+struct AttnArgs {
+    bf16* out;
+    int out_stride;
+    const bf16* q;
+    int q_stride;
+    const bf16* k_pool;
+    const bf16* v_pool;
+    const int* block_tables;
+    int max_blocks;
+    const int* cu_seqlens;
+    const int* context_lens;
+    int seq_begin;
+    int n_heads, n_kv_heads, block_size, window;
+    float scale;
+    int num_splits;
+    float* ws_o;   // [token, head, split, D]
+    float* ws_ml;  // [token, head, split, 2]
+};
+
+template <int DB, bool SPLIT_WAVES>
+__global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnArgs a) {
+    constexpr int D = DB * 16;
+    constexpr int KS = (D + 31) / 32;  // k-steps of the score product
+    const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
+    const int col = lane % 16, g = lane / 16;
+
+    const int G = a.n_heads / a.n_kv_heads;
+    const int HG = G < 16 ? G : 16;       // heads of one column group
+    const int TPG = 16 / HG;              // tokens of one column group
+    const int HB = (G + HG - 1) / HG;     // column groups needed to cover a KV head's query heads
+    const int kvh = blockIdx.y / HB, hb = blockIdx.y % HB;
+    const int b = a.seq_begin + blockIdx.z;
+    const int tok0 = a.cu_seqlens[b], n_new = a.cu_seqlens[b + 1] - tok0;
+    const int ctx = a.context_lens[b];
+
+    int tile, split = 0;
+    if (SPLIT_WAVES) {
+        tile = blockIdx.x / a.num_splits;
+        split = blockIdx.x % a.num_splits;
+    } else {
+        tile = blockIdx.x * 4 + wave;
+    }
+    const int t_first = tile * TPG;  // first token (within the request's new tokens) of this group
+    if (t_first >= n_new) return;    // (uniform over the workgroup when SPLIT_WAVES)
+
+    // this lane's column
+    const int c_tok = t_first + col / HG, c_head_in = hb * HG + col % HG;
+    const bool col_ok = col < HG * TPG && c_tok < n_new && c_head_in < G;
+    const int head = kvh * G + c_head_in;
+    const int p_col = col_ok ? ctx - n_new + c_tok : -1;  // absolute position of the column's token
+    const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
+    // key range of the whole group
+    const int t_last = min(t_first + TPG, n_new) - 1;
+    const int p_max = ctx - n_new + t_last;
+    const int p_min = ctx - n_new + t_first;
+    const int lo_min = (a.window > 0 && p_min - a.window + 1 > 0) ? p_min - a.window + 1 : 0;
+    const int j_begin = lo_min & ~31;
+    const int n_tiles = (p_max - j_begin) / 32 + 1;
+
+    // queries of this lane's column: Q[col][32s + 8g .. +7]
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    uint4 qf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int d = 32 * s + 8 * g;
+        qf[s] = (col_ok && d < D)
+                    ? *reinterpret_cast<const uint4*>(a.q + (size_t)(tok0 + c_tok) * a.q_stride + (size_t)head * D + d)
+                    : zero;
+    }
+
+    f32x4 acc[DB];
+#pragma unroll
+    for (int m = 0; m < DB; ++m) acc[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    const int* table = a.block_tables + (size_t)b * a.max_blocks;
+    const size_t page_stride = (size_t)a.n_kv_heads * a.block_size * D;
+    const bf16* k_base = a.k_pool + (size_t)kvh * a.block_size * D;
+    const bf16* v_base = a.v_pool + (size_t)kvh * a.block_size * D;
+
+    int t_begin = 0, t_end = n_tiles, t_step = 1;
+    if (SPLIT_WAVES) {
+        const int per_split = (n_tiles + a.num_splits - 1) / a.num_splits;
+        t_begin = split * per_split + wave;
+        t_end = min(n_tiles, (split + 1) * per_split);
+        t_step = 4;
+    }
+    for (int t = t_begin; t < t_end; t += t_step) {
+        const int j0 = j_begin + 32 * t;
+        // ---- scores: rows of tile u (u = 0, 1) are the keys j0 + 8*(i/4) + 4u + i%4
+        f32x4 s_acc[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            s_acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            const int key = j0 + 8 * (col / 4) + 4 * u + (col % 4);  // `col` is the row index i here
+            const bool key_ok = key <= p_max;
+            const bf16* krow = nullptr;
+            if (key_ok) {
+                const int page = table[key / a.block_size];
+                krow = k_base + (size_t)page * page_stride + (size_t)(key % a.block_size) * D;
+            }
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                const int d = 32 * s + 8 * g;
+                const uint4 kf = (key_ok && d < D) ? *reinterpret_cast<const uint4*>(krow + d) : zero;
+                s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[s]), s_acc[u], 0, 0, 0);
+            }
+        }
+        // ---- values of the lane's 8 keys j0 + 8g .. +7, for every block of 16 dimensions
+        const int jk = j0 + 8 * g;
+        uint4 vf[DB];
+        {
+            const bool chunk_ok = jk <= p_max;
+            const bf16* vrow = nullptr;
+            if (chunk_ok) {
+                const int page = table[jk / a.block_size];
+                vrow = v_base + (size_t)page * page_stride + (jk % a.block_size);
+            }
+            // keys outside [lo_min, p_max] may be stale or never written: their values become 0
+            const int first = lo_min - jk, last = p_max + 1 - jk;
+#pragma unroll
+            for (int m = 0; m < DB; ++m) {
+                uint4 v = chunk_ok ? *reinterpret_cast<const uint4*>(vrow + (size_t)(16 * m + col) * a.block_size) : zero;
+                vf[m] = keep_elements(v, first, last);
+            }
+        }
+        // ---- online softmax of this lane's column over its 8 keys (and the 3 other lane groups)
+        float sc[8];
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int key = jk + e;
+            const bool ok = key >= lo_col && key <= p_col;
+            sc[e] = ok ? s_acc[e / 4][e % 4] * a.scale : -INFINITY;
+            tmax = fmaxf(tmax, sc[e]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, LLMS_WAVE));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, LLMS_WAVE));
+        const float m_new = fmaxf(m_run, tmax);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = __expf(m_run - m_safe);
+        float psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            sc[e] = __expf(sc[e] - m_safe);
+            psum += sc[e];
+        }
+        psum += __shfl_xor(psum, 16, LLMS_WAVE);
+        psum += __shfl_xor(psum, 32, LLMS_WAVE);
+        l_run = l_run * corr + psum;
+        m_run = m_new;
+        const uint4 pf = make_uint4(pack_bf16(sc[0], sc[1]), pack_bf16(sc[2], sc[3]), pack_bf16(sc[4], sc[5]),
+                                    pack_bf16(sc[6], sc[7]));
+#pragma unroll
+        for (int m = 0; m < DB; ++m) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[m][r] *= corr;
+            acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[m]), as_bf16x8(pf), acc[m], 0, 0, 0);
+        }
+    }
+
+    // acc[m][r] = O^T[d = 16m + 4g + r][col]
+    if (!SPLIT_WAVES) {
+        if (col_ok) {
+            const float inv = 1.f / l_run;
+            bf16* orow = a.out + (size_t)(tok0 + c_tok) * a.out_stride + (size_t)head * D;
+#pragma unroll
+            for (int m = 0; m < DB; ++m) {
+                uint2 w;
+                w.x = pack_bf16(acc[m][0] * inv, acc[m][1] * inv);
+                w.y = pack_bf16(acc[m][2] * inv, acc[m][3] * inv);
+                *reinterpret_cast<uint2*>(orow + 16 * m + 4 * g) = w;
+            }
+        }
+        return;
+    }
+
+    // ---- the 4 waves' partial results meet in LDS, wave 0 first, then 1, 2, 3
+    __shared__ float sh_acc[DB][LLMS_WAVE][4];
+    __shared__ float sh_m[16], sh_l[16];
+    for (int w = 0; w < 4; ++w) {
+        if (wave == w) {
+            if (w == 0) {
+#pragma unroll
+                for (int m = 0; m < DB; ++m)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) sh_acc[m][lane][r] = acc[m][r];
+                if (g == 0) {
+                    sh_m[col] = m_run;
+                    sh_l[col] = l_run;
+                }
+            } else {
+                const float m_old = sh_m[col], l_old = sh_l[col];
+                const float m_tot = fmaxf(m_old, m_run);
+                const float m_safe = (m_tot == -INFINITY) ? 0.f : m_tot;
+                const float wa = __expf(m_old - m_safe), wb = __expf(m_run - m_safe);
+#pragma unroll
+                for (int m = 0; m < DB; ++m)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) sh_acc[m][lane][r] = sh_acc[m][lane][r] * wa + acc[m][r] * wb;
+                __builtin_amdgcn_wave_barrier();  // all lanes have read sh_m/sh_l before lane group 0 rewrites them
+                if (g == 0) {
+                    sh_m[col] = m_tot;
+                    sh_l[col] = l_old * wa + l_run * wb;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (wave != 0 || !col_ok) return;
+    const float m_tot = sh_m[col], l_tot = sh_l[col];
+    if (a.num_splits == 1) {
+        const float inv = 1.f / l_tot;
+        bf16* orow = a.out + (size_t)(tok0 + c_tok) * a.out_stride + (size_t)head * D;
+#pragma unroll
+        for (int m = 0; m < DB; ++m) {
+            uint2 w;
+            w.x = pack_bf16(sh_acc[m][lane][0] * inv, sh_acc[m][lane][1] * inv);
+            w.y = pack_bf16(sh_acc[m][lane][2] * inv, sh_acc[m][lane][3] * inv);
+            *reinterpret_cast<uint2*>(orow + 16 * m + 4 * g) = w;
+        }
+    } else {
+        const size_t item = ((size_t)(tok0 + c_tok) * a.n_heads + head) * a.num_splits + split;
+        float* wo = a.ws_o + item * D;
+#pragma unroll
+        for (int m = 0; m < DB; ++m)
+            *reinterpret_cast<float4*>(wo + 16 * m + 4 * g) =
+                make_float4(sh_acc[m][lane][0], sh_acc[m][lane][1], sh_acc[m][lane][2], sh_acc[m][lane][3]);
+        if (g == 0) {
+            a.ws_ml[item * 2] = m_tot;
+            a.ws_ml[item * 2 + 1] = l_tot;
+        }
+    }
+}
+
+// Merge of the splits of one (token, head), split 0 first.
+__global__ void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ ws_o,
+                                  const float* __restrict__ ws_ml, int token_begin, int n_heads, int head_dim,
+                                  int num_splits) {
+    const int token = token_begin + blockIdx.x, head = blockIdx.y;
+    const size_t item0 = ((size_t)token * n_heads + head) * num_splits;
+    float m_tot = -INFINITY;
+    for (int s = 0; s < num_splits; ++s) m_tot = fmaxf(m_tot, ws_ml[(item0 + s) * 2]);
+    float l_tot = 0.f;
+    for (int s = 0; s < num_splits; ++s) {
+        const float m = ws_ml[(item0 + s) * 2];
+        if (m != -INFINITY) l_tot += ws_ml[(item0 + s) * 2 + 1] * __expf(m - m_tot);
+    }
+    const float inv = 1.f / l_tot;
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        float o = 0.f;
+        for (int s = 0; s < num_splits; ++s) {
+            const float m = ws_ml[(item0 + s) * 2];
+            if (m != -INFINITY) o += ws_o[(item0 + s) * head_dim + d] * __expf(m - m_tot);
+        }
+        out[(size_t)token * out_stride + (size_t)head * head_dim + d].bits = f32_to_bf16_bits(o * inv);
+    }
+}
+
+template <bool SPLIT_WAVES>
+static int launch_attn(int db, dim3 grid, const AttnArgs& a, hipStream_t stream) {
+#define ATT_CASE(N)                                                          \
+    case N:                                                                  \
+        attn_mfma_kernel<N, SPLIT_WAVES><<<grid, 256, 0, stream>>>(a);       \
+        break;
+    switch (db) {
+        ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
+        ATT_CASE(9) ATT_CASE(10) ATT_CASE(11) ATT_CASE(12) ATT_CASE(13) ATT_CASE(14) ATT_CASE(15) ATT_CASE(16)
+        default:
+            LLMS_REQUIRE(false, "attention_mfma: head_dim must be a multiple of 16 up to 256");
+    }
+#undef ATT_CASE
+    return LLMS_OK;
+}
+
+extern "C" {
+
+// Attention for the requests [seq_begin, seq_begin + n_seqs) of a step.  max_new: most new tokens any of
+// them brings.  split_waves = 1 deals the keys of each column group to 4 waves and `num_splits`
+// workgroups (decoding); with num_splits > 1 the caller provides ws_o [tokens * heads * splits * D] and
+// ws_ml [tokens * heads * splits * 2] floats, indexed by absolute token row.
+int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
+                        const void* v_pool, const int* block_tables, int max_blocks, const int* cu_seqlens,
+                        const int* context_lens, int seq_begin, int n_seqs, int max_new, int token_begin,
+                        int n_tokens, int n_heads, int n_kv_heads, int head_dim, int block_size, int window,
+                        float scale, int split_waves, int num_splits, float* ws_o, float* ws_ml,
+                        hipStream_t stream) {
+    LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && n_heads > 0 && n_kv_heads > 0, "attention_mfma: sizes must be positive");
+    LLMS_REQUIRE(n_heads % n_kv_heads == 0, "attention_mfma: n_heads must be a multiple of n_kv_heads");
+    LLMS_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256, "attention_mfma: head_dim must be a multiple of 16 up to 256");
+    LLMS_REQUIRE(block_size > 0 && block_size % 8 == 0, "attention_mfma: block_size must be a multiple of 8");
+    LLMS_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0, "attention_mfma: row strides must keep 16-byte (q) and 8-byte (out) alignment");
+    LLMS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 && ((uintptr_t)v_pool % 16) == 0 &&
+                     ((uintptr_t)out % 8) == 0, "attention_mfma: pointers must be 16-byte aligned");
+    LLMS_REQUIRE(window >= 0 && max_blocks > 0, "attention_mfma: bad window or max_blocks");
+    LLMS_REQUIRE(num_splits >= 1, "attention_mfma: num_splits must be >= 1");
+    LLMS_REQUIRE(split_waves || num_splits == 1, "attention_mfma: splits need split_waves");
+    LLMS_REQUIRE(num_splits == 1 || (ws_o && ws_ml), "attention_mfma: splits need a workspace");
+    LLMS_REQUIRE(n_seqs <= 65535, "attention_mfma: too many requests for one launch");
+    const int G = n_heads / n_kv_heads, HG = G < 16 ? G : 16, TPG = 16 / HG, HB = (G + HG - 1) / HG;
+    const int groups = (max_new + TPG - 1) / TPG;
+    AttnArgs a = {(bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pool, (const bf16*)v_pool,
+                  block_tables, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
+                  window, scale, num_splits, ws_o, ws_ml};
+    LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
+    if (split_waves) {
+        dim3 grid(groups * num_splits, n_kv_heads * HB, n_seqs);
+        if (int e = launch_attn<true>(head_dim / 16, grid, a, stream)) return e;
+        if (num_splits > 1) {
+            hipError_t e1 = hipGetLastError();
+            if (e1 != hipSuccess) {
+                fprintf(stderr, "llmserve kernel launch failed: %s\n", hipGetErrorString(e1));
+                return LLMS_ERR_LAUNCH;
+            }
+            attn_merge_kernel<<<dim3(n_tokens, n_heads), 64, 0, stream>>>((bf16*)out, out_stride, ws_o, ws_ml,
+                                                                          token_begin, n_heads, head_dim, num_splits);
+        }
+    } else {
+        dim3 grid((groups + 3) / 4, n_kv_heads * HB, n_seqs);
+        if (int e = launch_attn<false>(head_dim / 16, grid, a, stream)) return e;
+    }
+    LLMS_LAUNCH_CHECK();
+}
+
+}  // extern "C"

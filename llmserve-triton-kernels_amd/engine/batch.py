@@ -42,6 +42,7 @@ class StepBatch:
     num_decode: int = 0  # leading requests that bring exactly one token
     max_count: int = 0
     max_context: int = 0
+    max_decode_context: int = 0  # longest context among the leading single-token requests
 
 
 class BatchUploader:
@@ -126,4 +127,4 @@ def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[in
         token_seq=view(2, n_tokens), cu_seqlens=view(3, n_seqs + 1), context_lens=view(4, n_seqs),
         state_slots=view(5, n_seqs), logit_rows=view(6, len(logit_rows)), groups=groups,
         counts=list(counts), starts=list(starts), num_decode=num_decode, max_count=max(counts),
-        max_context=max(context))
+        max_context=max(context), max_decode_context=max(context[:num_decode], default=0))

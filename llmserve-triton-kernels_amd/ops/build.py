@@ -36,7 +36,7 @@ HIPCC_FLAGS = [
 # Which libraries a model of a given dtype needs.
 GROUPS = {
     "float32": ("elementwise", "gemm", "attention", "sampling"),
-    "bfloat16": ("elementwise", "gemm", "attention", "sampling", "gemm_mfma"),
+    "bfloat16": ("elementwise", "gemm", "attention", "sampling", "gemm_mfma", "attention_mfma"),
 }
 
 

@@ -333,6 +333,52 @@ def attention_wave(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
     return out
 
 
+def attention_mfma_supported(dtype: torch.dtype, head_dim: int, block_size: int) -> bool:
+    """Whether the matrix-core attention kernel takes this cache (else `attention_wave` does)."""
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and block_size % 8 == 0
+
+
+def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                   block_tables: torch.Tensor, cu_seqlens: torch.Tensor, context_lens: torch.Tensor,
+                   seq_begin: int, n_seqs: int, max_new: int, token_begin: int, n_tokens: int,
+                   n_heads: int, n_kv_heads: int, head_dim: int, block_size: int, window: int = 0,
+                   scale: float | None = None, split_waves: bool = False, num_splits: int = 1) -> torch.Tensor:
+    """bfloat16 causal attention on the matrix cores for requests [seq_begin, seq_begin + n_seqs) of a
+    step, whose new tokens are rows [token_begin, token_begin + n_tokens) of q and out and bring at most
+    `max_new` tokens each.  `split_waves` (with `num_splits`) spreads each request's keys over waves and
+    workgroups: the arrangement for single decoded tokens."""
+    dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens)
+    _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
+    if not attention_mfma_supported(q.dtype, head_dim, block_size):
+        raise ValueError(f"attention_mfma needs bfloat16, head_dim a multiple of 16 up to 256 and block_size a "
+                         f"multiple of 8; got {q.dtype}, {head_dim}, {block_size}")
+    b = block_tables.shape[0]
+    _i32(cu_seqlens, "cu_seqlens", b + 1)
+    _i32(context_lens, "context_lens", b)
+    if not (0 <= seq_begin and n_seqs >= 0 and seq_begin + n_seqs <= b):
+        raise ValueError("request range is outside the batch")
+    if not (0 <= token_begin and token_begin + n_tokens <= q.shape[0]):
+        raise ValueError("token range is outside the batch")
+    if q.stride(0) % 8 or q.data_ptr() % 16 or out.data_ptr() % 16:
+        raise ValueError("q rows must be 16-byte aligned")
+    if num_splits > 1 and not split_waves:
+        raise ValueError("num_splits > 1 needs split_waves")
+    if n_seqs == 0 or n_tokens == 0:
+        return out
+    ws_o = ws_ml = None
+    if num_splits > 1:
+        ws_o = torch.empty((q.shape[0] * n_heads * num_splits * head_dim,), dtype=torch.float32, device=dev)
+        ws_ml = torch.empty((q.shape[0] * n_heads * num_splits * 2,), dtype=torch.float32, device=dev)
+    scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
+    _check(load("attention_mfma").llms_attention_mfma(
+        _ptr(out), c_int(out.stride(0)), _ptr(q), c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool),
+        _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens), c_int(seq_begin),
+        c_int(n_seqs), c_int(max_new), c_int(token_begin), c_int(n_tokens), c_int(n_heads), c_int(n_kv_heads),
+        c_int(head_dim), c_int(block_size), c_int(window), c_float(scale), c_int(1 if split_waves else 0),
+        c_int(num_splits), _ptr(ws_o), _ptr(ws_ml), _stream(dev)), "attention_mfma")
+    return out
+
+
 # ------------------------------------------------------------------------------ sampling
 
 

@@ -83,6 +83,24 @@ class Attention(Mixer):
     def attend(self, out, qkv, cache, view, batch):
         """out[n] = attention of token n's query heads (the first nh*D columns of qkv) over its
         request's pages.  Picks the kernel by dtype and by what the step holds."""
-        ops.attention_wave(out, qkv, cache.k_pool, cache.v_pool, view.block_tables, batch.token_seq,
-                           batch.positions, self.num_heads, self.num_kv_heads, self.head_dim,
-                           cache.block_size, self.window or 0, self.scale)
+        nh, nkv, d, bs, window = self.num_heads, self.num_kv_heads, self.head_dim, cache.block_size, self.window or 0
+        if not ops.attention_mfma_supported(qkv.dtype, d, bs):
+            ops.attention_wave(out, qkv, cache.k_pool, cache.v_pool, view.block_tables, batch.token_seq,
+                               batch.positions, nh, nkv, d, bs, window, self.scale)
+            return
+        common = (out, qkv, cache.k_pool, cache.v_pool, view.block_tables, batch.cu_seqlens, batch.context_lens)
+        n_dec = batch.num_decode
+        if n_dec:  # requests that bring one token: their keys are spread over waves and workgroups
+            ops.attention_mfma(*common, 0, n_dec, 1, 0, n_dec, nh, nkv, d, bs, window, self.scale,
+                               split_waves=True, num_splits=self.decode_splits(n_dec, batch.max_decode_context))
+        if n_dec < batch.num_seqs:  # portions of prompts: one wave per group of tokens and heads
+            ops.attention_mfma(*common, n_dec, batch.num_seqs - n_dec, batch.max_count, n_dec,
+                               batch.num_tokens - n_dec, nh, nkv, d, bs, window, self.scale)
+
+    def decode_splits(self, n_requests: int, max_context: int) -> int:
+        """Workgroups per (request, KV head) for decoding: enough to fill the chip when the batch is
+        small, never more than there are stretches of 128 keys."""
+        g = self.num_heads // self.num_kv_heads
+        groups = n_requests * self.num_kv_heads * -(-g // 16)
+        reach = min(max_context, self.window) if self.window else max_context
+        return max(1, min(256 // groups, -(-reach // 128)))

@@ -319,3 +319,101 @@ def test_sample_rows_mixed_batch_and_frequencies():
     assert (got[::2] == 2).all()
     freq = torch.bincount(got[1::2].long(), minlength=4).float() / 2000
     assert torch.allclose(freq, torch.softmax(logits[0].cpu() / 0.7, -1), atol=0.04)
+
+
+# ------------------------------------------------------------------ attention on the matrix cores
+def run_attention_mfma(nh, nkv, d, bs, lens, new, window=0, seed=0, craft=None, split_waves=False, num_splits=1):
+    """As `run_attention`, for the bfloat16 matrix-core kernel and its request-wise arguments."""
+    dtype = torch.bfloat16
+    qs = [rnd(s, nh, d, seed=seed + 3 * b) for b, s in enumerate(lens)]
+    ks = [rnd(s, nkv, d, seed=seed + 3 * b + 1) for b, s in enumerate(lens)]
+    vs = [rnd(s, nkv, d, seed=seed + 3 * b + 2) for b, s in enumerate(lens)]
+    if craft:
+        craft(qs, ks, vs)
+    qs, ks, vs = ([t.to(dtype) for t in ts] for ts in (qs, ks, vs))
+    k_pool, v_pool, tables = make_paged(ks, vs, bs, dtype, seed=seed)
+    q_rows, refs, cu = [], [], [0]
+    for b, (s, n) in enumerate(zip(lens, new)):
+        rows = list(range(s - n, s))
+        q_rows.append(qs[b][rows].reshape(n, nh * d))
+        cu.append(cu[-1] + n)
+        refs.append(attention_reference(qs[b], ks[b], vs[b], rows, window or None))
+    # queries sit inside a wider row, as the q part of a qkv buffer does
+    q = torch.cat([torch.cat(q_rows), torch.full((cu[-1], 2 * nkv * d), float("nan"), dtype=dtype)], dim=1).contiguous().to(DEV)
+    out = torch.empty(cu[-1], nh * d, dtype=dtype, device=DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)  # noqa: E731
+    ops().attention_mfma(out, q, k_pool.to(DEV), v_pool.to(DEV), tables.to(DEV), i32(cu), i32(lens), 0, len(lens),
+                         max(new), 0, cu[-1], nh, nkv, d, bs, window, None, split_waves=split_waves,
+                         num_splits=num_splits)
+    got = out.float().cpu()
+    assert torch.isfinite(got).all(), "read a slot that was never written"
+    return got, torch.cat(refs)
+
+
+MFMA_CASES = [  # nh, nkv, d, bs, lens, new, window
+    (4, 2, 16, 16, [5, 17, 33], [5, 17, 33], 0),
+    (3, 1, 32, 8, [1, 7, 40, 100], [1, 1, 1, 1], 0),
+    (3, 1, 32, 8, [1, 7, 40, 100], [1, 7, 24, 2], 0),
+    (8, 1, 64, 16, [300, 64, 129], [1, 24, 2], 0),
+    (6, 2, 80, 8, [70, 19], [3, 19], 0),
+    (4, 4, 128, 32, [257, 31], [1, 31], 0),
+    (2, 1, 256, 16, [90], [7], 0),
+    (32, 4, 64, 16, [600, 31], [1, 1], 0),
+    (32, 1, 32, 8, [45], [3], 0),
+    (5, 1, 48, 8, [77], [20], 0),
+    (12, 1, 16, 24, [50], [50], 0),
+    (4, 2, 32, 8, [150, 40], [30, 1], 16),
+    (3, 3, 16, 16, [100], [100], 7),
+    (4, 1, 64, 16, [200], [64], 40),
+]
+
+
+@pytest.mark.parametrize("arrangement", [(False, 1), (True, 1), (True, 2), (True, 5)])
+@pytest.mark.parametrize("case", MFMA_CASES)
+def test_attention_mfma(case, arrangement):
+    nh, nkv, d, bs, lens, new, window = case
+    split_waves, num_splits = arrangement
+    got, ref = run_attention_mfma(nh, nkv, d, bs, lens, new, window, seed=50, split_waves=split_waves,
+                                  num_splits=num_splits)
+    assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("arrangement", [(False, 1), (True, 1), (True, 3)])
+@pytest.mark.parametrize("needle", [0, 15, 16, 31, 32, 299, 300 - 17, 141])
+def test_attention_mfma_finds_one_far_key(needle, arrangement):
+    def craft(qs, ks, vs):
+        qs[0][-1] = 0
+        qs[0][-1, :, 0] = 12.0
+        ks[0][:, :, 0] = 0
+        ks[0][needle, :, 0] = 12.0
+        vs[0][needle] = 3.0
+
+    got, ref = run_attention_mfma(8, 2, 64, 16, [300], [1], 0, seed=60, craft=craft, split_waves=arrangement[0],
+                                  num_splits=arrangement[1])
+    assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max()) and got.mean() > 2.9
+
+
+def test_attention_mfma_window_edge():
+    for needle, inside in ((100 - 8, False), (100 - 7, True)):
+        def craft(qs, ks, vs):
+            qs[0][-1] = 0
+            qs[0][-1, :, 1] = 10.0
+            ks[0][:, :, 1] = 0
+            ks[0][needle, :, 1] = 10.0
+            vs[0][needle] = 5.0
+
+        for split_waves in (False, True):
+            got, ref = run_attention_mfma(2, 1, 32, 8, [101], [1], 8, seed=61, craft=craft, split_waves=split_waves)
+            assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
+            assert (got.mean() > 4.0) == inside
+
+
+def test_attention_mfma_refuses_what_it_cannot_take():
+    assert not ops().attention_mfma_supported(torch.bfloat16, 64, 4)
+    assert not ops().attention_mfma_supported(torch.bfloat16, 40, 16)
+    assert not ops().attention_mfma_supported(torch.float32, 64, 16)
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)  # noqa: E731
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)  # noqa: E731
+    with pytest.raises(ValueError, match="multiple of 8"):
+        ops().attention_mfma(z(1, 64), z(1, 64), z(2, 1, 4, 64), z(2, 1, 64, 4), i32([[0]]), i32([0, 1]), i32([1]),
+                             0, 1, 1, 0, 1, 1, 1, 64, 4)
