@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnArgs a) {
         tile = blockIdx.x * 4 + wave;
     }
     const int t_first = tile * TPG;  // first token (within the request's new tokens) of this group
-    if (t_first >= n_new) return;    // (uniform over the workgroup when SPLIT_WAVES)
+    if (t_first >= n_new || ctx <= 0) return;  // (uniform over the workgroup when SPLIT_WAVES)
 
     // this lane's column
     const int c_tok = t_first + col / HG, c_head_in = hb * HG + col % HG;

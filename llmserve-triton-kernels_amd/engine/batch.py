@@ -128,3 +128,74 @@ def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[in
         state_slots=view(5, n_seqs), logit_rows=view(6, len(logit_rows)), groups=groups,
         counts=list(counts), starts=list(starts), num_decode=num_decode, max_count=max(counts),
         max_context=max(context), max_decode_context=max(context[:num_decode], default=0))
+
+
+class StaticDecodeBatch:
+    """Fixed device buffers for decode-only steps of up to `capacity` requests, so that such a step
+    can be captured once as a HIP graph and replayed: every step writes its tokens, positions, slots,
+    block tables and context lengths into the same memory with one copy.  Unused rows belong to
+    dummy requests of context length 0, which every kernel leaves alone or computes harmlessly
+    (rows never mix)."""
+
+    def __init__(self, capacity: int, table_width: int, group_ids: list[int], device: torch.device):
+        self.capacity = capacity
+        self.table_width = table_width
+        self.group_ids = list(group_ids)
+        c, w = capacity, table_width
+        pad = lambda n: n + (-n % 4)  # noqa: E731
+        sizes = [c, c, c, c + 1, c, c, c] + [x for _ in group_ids for x in (c, c * w)]
+        self._offsets, total = [], 0
+        for n in sizes:
+            self._offsets.append(total)
+            total += pad(n)
+        self._sizes = sizes
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.dev = torch.zeros(total, dtype=torch.int32, device=device)
+        self._event = None
+        v = self._view
+        groups = {g: GroupView(v(8 + 2 * j).view(c, w), v(7 + 2 * j)) for j, g in enumerate(group_ids)}
+        self.batch = StepBatch(
+            num_tokens=c, num_seqs=c, token_ids=v(0), positions=v(1), token_seq=v(2), cu_seqlens=v(3),
+            context_lens=v(4), state_slots=v(5), logit_rows=v(6), groups=groups, counts=[1] * c, starts=[0] * c,
+            num_decode=c, max_count=1, max_context=1, max_decode_context=1)
+        # what never changes: one token per request, every row's logits wanted
+        h = self._host_view
+        h(2)[:] = torch.arange(c, dtype=torch.int32)
+        h(3)[:] = torch.arange(c + 1, dtype=torch.int32)
+        h(6)[:] = torch.arange(c, dtype=torch.int32)
+        for j in range(len(group_ids)):
+            h(7 + 2 * j)[:] = -1  # until a step is filled in, no row stores anything
+        self.dev.copy_(self.host)
+
+    def _view(self, i: int) -> torch.Tensor:
+        return self.dev[self._offsets[i]: self._offsets[i] + self._sizes[i]]
+
+    def _host_view(self, i: int) -> torch.Tensor:
+        return self.host[self._offsets[i]: self._offsets[i] + self._sizes[i]]
+
+    def fill(self, layout: StepLayout, tokens: list[int]) -> None:
+        """Write a decode-only step (one token per request) into the buffers."""
+        n, c, w = len(tokens), self.capacity, self.table_width
+        if self._event is not None:
+            self._event.synchronize()  # the previous copy out of the pinned buffer has finished
+        h = self._host_view
+        h(0)[:n] = torch.tensor(tokens, dtype=torch.int32)
+        h(0)[n:] = 0
+        h(1)[:n] = torch.tensor(layout.starts, dtype=torch.int32)
+        h(1)[n:] = 0
+        h(4)[:n] = torch.tensor(layout.starts, dtype=torch.int32) + 1
+        h(4)[n:] = 0  # dummy requests: no keys, nothing to attend to
+        h(5)[:n] = torch.tensor(layout.state_slots, dtype=torch.int32)
+        h(5)[n:] = 0
+        for j, g in enumerate(self.group_ids):
+            h(7 + 2 * j)[:n] = torch.tensor(layout.slots[g], dtype=torch.int32)
+            h(7 + 2 * j)[n:] = -1  # dummy tokens store nothing
+            table = h(8 + 2 * j).view(c, w)
+            table.zero_()
+            for b, t in enumerate(layout.tables[g]):
+                if len(t) > w:
+                    raise ValueError(f"block table of {len(t)} pages exceeds the captured width {w}")
+                table[b, : len(t)] = torch.tensor([x if x >= 0 else 0 for x in t], dtype=torch.int32)
+        self.dev.copy_(self.host, non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record(torch.cuda.current_stream(self.dev.device))

@@ -61,7 +61,7 @@ def main(argv=None) -> int:
         ap.error("--max-tokens must be positive")
     num_blocks = -(-args.max_tokens // args.block_size)
     engine_config = EngineConfig(dtype=args.dtype, block_size=args.block_size, num_blocks=num_blocks,
-                                 max_num_seqs=args.max_seqs, use_graphs=False)
+                                 max_num_seqs=args.max_seqs)
     replayer = Replayer(ModelRunner.from_folder(args.model, engine_config))
 
     for line in sys.stdin:

@@ -23,7 +23,7 @@ from ..parts.model import Model
 from ..parts.registry import BuildContext
 from ..weights.loader import load_tensors
 from ..weights.random import random_tensors
-from .batch import BatchUploader, build_batch
+from .batch import BatchUploader, StaticDecodeBatch, build_batch
 
 _TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
@@ -65,6 +65,8 @@ class ModelRunner:
         self.storage = CacheStorage(groups, num_blocks, self.block_size, engine_config.max_num_seqs,
                                     self.dtype, device)
         self._uploader = BatchUploader(device)
+        self._graphs: dict[tuple[int, int], "_DecodeGraph"] = {}
+        self._use_graphs = engine_config.use_graphs
 
     # ---- construction ---------------------------------------------------------------------
     @staticmethod
@@ -147,7 +149,52 @@ class ModelRunner:
             row += len(e.tokens)
         logit_rows = [first_row[id(e)] + w for e in entries for w in e.want]
         self.storage.clear_state(layout.fresh_slots)
-        batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader)
-        logits = self.model.forward(batch, self.storage)
+        if self._use_graphs and all(len(e.tokens) == 1 for e in ordered):
+            logits = self._replay_decode(layout, [e.tokens[0] for e in ordered], logit_rows)
+        else:
+            batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader)
+            logits = self.model.forward(batch, self.storage)
         self.manager.release_passed(layout.seq_ids)
         return logits
+
+    # ---- decode-only steps as HIP graphs --------------------------------------------------------
+    def _replay_decode(self, layout, tokens: list[int], logit_rows: list[int]) -> torch.Tensor:
+        """A step of single tokens: replay the graph captured for this batch size and context range
+        (capture it at first use).  The logits it returns live in the graph's own memory and are
+        overwritten by the next replay of the same graph."""
+        n = len(tokens)
+        capacity = 1
+        while capacity < n:
+            capacity *= 2
+        context = max(layout.starts) + 1
+        reach = 256
+        while reach < context:
+            reach *= 2
+        key = (capacity, reach)
+        graph = self._graphs.get(key)
+        if graph is None:
+            graph = _DecodeGraph(self, capacity, reach)
+            self._graphs[key] = graph
+        graph.static.fill(layout, tokens)
+        graph.graph.replay()
+        if logit_rows == list(range(n)):
+            return graph.logits[:n]
+        return graph.logits[torch.tensor(logit_rows, dtype=torch.long, device=self.device)]
+
+
+class _DecodeGraph:
+    """One captured decode step for up to `capacity` requests whose contexts reach up to `reach` keys
+    (the reach only sets how the attention kernel spreads its work; longer contexts stay correct)."""
+
+    def __init__(self, runner: ModelRunner, capacity: int, reach: int):
+        width = -(-runner.max_model_len // runner.block_size)
+        group_ids = [g.group_id for g in runner.manager.paged_groups]
+        self.static = StaticDecodeBatch(capacity, width, group_ids, runner.device)
+        batch = self.static.batch
+        batch.max_context = batch.max_decode_context = reach
+        # a first run outside the capture: libraries load, memory pools warm up
+        runner.model.forward(batch, runner.storage)
+        torch.cuda.synchronize(runner.device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = runner.model.forward(batch, runner.storage)

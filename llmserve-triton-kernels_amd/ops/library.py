@@ -275,10 +275,13 @@ def gemm_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.T
                          "and 16-byte aligned operands")
     if m == 0:
         return out
-    kernel = kernel or ("skinny" if m <= 64 else "tile")
+    kernel = kernel or ("stream" if m <= 16 else "skinny" if m <= 64 else "tile")
     if kernel == "skinny" and m > 64:
         raise ValueError("the skinny kernel takes at most 64 rows")
-    fn = load("gemm_mfma").llms_gemm_bf16_skinny if kernel == "skinny" else load("gemm_mfma").llms_gemm_bf16_tile
+    if kernel == "stream" and m > 16:
+        raise ValueError("the stream kernel takes at most 16 rows")
+    lib = load("gemm_mfma")
+    fn = {"stream": lib.llms_gemm_bf16_stream, "skinny": lib.llms_gemm_bf16_skinny, "tile": lib.llms_gemm_bf16_tile}[kernel]
     _check(fn(c_int(_code(out)), _ptr(out), _ptr(a), _ptr(w), _ptr(bias), c_int(m), c_int(n), c_int(k),
               c_int(a.stride(0)), c_int(out.stride(0)), _stream(dev)), f"gemm_bf16[{kernel}]")
     return out

@@ -25,14 +25,14 @@ def sequences(name: str) -> dict[str, list[int]]:
     return {f"{name}{i}": traces.random_ids(vocab, n, 1000 + 17 * i) for i, n in enumerate(LENGTHS[name])}
 
 
-def replay_in_process(model_dir, dtype_name, steps, block_size, num_blocks):
+def replay_in_process(model_dir, dtype_name, steps, block_size, num_blocks, use_graphs=True):
     from llmserve.config import EngineConfig
     from llmserve.engine.replay import Replayer
     from llmserve.engine.runner import ModelRunner
 
     runner = ModelRunner.from_folder(model_dir, EngineConfig(dtype=dtype_name, block_size=block_size,
                                                               num_blocks=num_blocks, max_num_seqs=4,
-                                                              use_graphs=False))
+                                                              use_graphs=use_graphs))
     runner.storage.poison()  # a slot that was never written must never be read
     rep = Replayer(runner)
     outputs = {}
@@ -73,6 +73,19 @@ def test_replay_matches_plain(model_dirs, name, dtype_name, mode):
     num_blocks = traces.tokens_needed(steps, round_to=block_size) // block_size
     outputs = replay_in_process(model_dirs[name], dtype_name, steps, block_size, num_blocks)
     check_against_plain(model_dirs[name], dtype_name, seqs, steps, outputs)
+
+
+@pytest.mark.parametrize("mode", ["decode_tail", "mixed"])
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_replay_without_graphs(model_dirs, dtype_name, mode):
+    """Steps of single tokens are replayed from captured HIP graphs by default; the same steps launched
+    kernel by kernel must give the same answers."""
+    seqs = sequences("b")
+    steps = MODES[mode](seqs)
+    block_size = TINY["b"][1]
+    num_blocks = traces.tokens_needed(steps, round_to=block_size) // block_size
+    outputs = replay_in_process(model_dirs["b"], dtype_name, steps, block_size, num_blocks, use_graphs=False)
+    check_against_plain(model_dirs["b"], dtype_name, seqs, steps, outputs)
 
 
 def test_mixed_trace_reuses_pages(model_dirs):
