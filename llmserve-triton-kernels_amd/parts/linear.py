@@ -1,8 +1,12 @@
-"""y = x W^T (+ b) for the parts: picks the matrix-product kernel by dtype and shape.
+"""y = x W^T (+ b) for the parts: picks the matrix product by dtype and shape.
 
 float32: the 32-bit multiply-add kernel, always (no reduced-precision matrix mode).
-bfloat16: the matrix-core kernels for bfloat16 results and for 32-bit results (logits);
-few rows (decoding) go to the kernel that streams the weight once.
+bfloat16, up to 16 rows (decoding): the hand-written kernel that streams the weight once.
+bfloat16, more rows: the library's matrix product (hipBLASLt through torch.mm), which is
+  where the reference's engine uses a library too (nn.Linear, src/llmserve/model/llama.py:64-67);
+  sums are 32-bit, the result bfloat16 or, for logits, float32.
+Operands the matrix-core kernels cannot take (K not a multiple of 8) fall to the 32-bit
+multiply-add kernel, which takes anything.
 """
 
 from __future__ import annotations
@@ -10,6 +14,9 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
+
+
+LIBRARY_ABOVE_ROWS = 16
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
@@ -22,5 +29,9 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     if m == 0:
         return out
     if x.dtype == torch.bfloat16 and ops.gemm_bf16_supported(x, weight):
-        return ops.gemm_bf16(out, x, weight, bias)
+        if m <= LIBRARY_ABOVE_ROWS:
+            return ops.gemm_bf16(out, x, weight, bias)
+        if bias is None:
+            return torch.mm(x, weight.t(), out_dtype=out.dtype, out=out)
+        return torch.addmm(bias.to(out.dtype), x, weight.t(), out_dtype=out.dtype, out=out)
     return ops.gemm_fma(out, x, weight, bias)
