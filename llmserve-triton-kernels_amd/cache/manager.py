@@ -27,7 +27,7 @@ from .allocator import BlockAllocator, OutOfBlocks
 class CacheGroup:
     group_id: int
     spec: PagedCacheSpec | StateCacheSpec
-    layers: tuple[int, ...]  # layers that own storage in this group, in order
+    layers: tuple[int, ...]  # entries of the model's schedule that own storage in this group, in order
 
     @property
     def paged(self) -> bool:
@@ -35,7 +35,8 @@ class CacheGroup:
 
 
 def group_layers(cache_specs: list[PagedCacheSpec | StateCacheSpec | None]) -> list[CacheGroup]:
-    """Groups for a list of per-layer needs (None: the layer keeps nothing of its own)."""
+    """Groups for a list of needs, one per entry of the model's schedule (None: the entry keeps
+    nothing of its own)."""
     by_spec: dict = {}
     for layer, spec in enumerate(cache_specs):
         if spec is not None:

@@ -78,7 +78,8 @@ class CacheStorage:
         return sum(t.numel() * t.element_size() for d in (self.k, self.v, self.state) for t in d.values())
 
     def layer_cache(self, layer: int, source: int | None = None):
-        """Cache view for `layer`; with `source`, the storage of that other layer, read-only."""
+        """Cache view for entry `layer` of the model's schedule; with `source`, the storage of
+        that other entry, read-only."""
         owner = layer if source is None else source
         if owner not in self._owner:
             return None

@@ -130,45 +130,77 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnArgs a) {
         t_end = min(n_tiles, (split + 1) * per_split);
         t_step = 4;
     }
-    for (int t = t_begin; t < t_end; t += t_step) {
-        const int j0 = j_begin + 32 * t;
-        // ---- scores: rows of tile u (u = 0, 1) are the keys j0 + 8*(i/4) + 4u + i%4
-        f32x4 s_acc[2];
+    // page and offset of a key; block sizes that are powers of two avoid the division
+    const int bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
+    auto locate = [&](int key, int& page, int& off) {
+        int blk;
+        if (bs_shift >= 0) {
+            blk = key >> bs_shift;
+            off = key & (a.block_size - 1);
+        } else {
+            blk = key / a.block_size;
+            off = key - blk * a.block_size;
+        }
+        page = table[blk];
+    };
+    // operands of one tile of 32 keys starting at j0: key rows for the scores (rows of tile u are the
+    // keys j0 + 8*(i/4) + 4u + i%4) and, for every block of 16 dimensions, the values of the lane's 8
+    // keys j0 + 8g .. +7.  Keys outside [lo_min, p_max] may be stale or never written: they load as 0.
+    auto load_tile = [&](int j0, uint4 (&kf)[2][KS], uint4 (&vf)[DB]) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            s_acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
             const int key = j0 + 8 * (col / 4) + 4 * u + (col % 4);  // `col` is the row index i here
             const bool key_ok = key <= p_max;
             const bf16* krow = nullptr;
             if (key_ok) {
-                const int page = table[key / a.block_size];
-                krow = k_base + (size_t)page * page_stride + (size_t)(key % a.block_size) * D;
+                int page, off;
+                locate(key, page, off);
+                krow = k_base + (size_t)page * page_stride + (size_t)off * D;
             }
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
                 const int d = 32 * s + 8 * g;
-                const uint4 kf = (key_ok && d < D) ? *reinterpret_cast<const uint4*>(krow + d) : zero;
-                s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf), as_bf16x8(qf[s]), s_acc[u], 0, 0, 0);
+                kf[u][s] = (key_ok && d < D) ? *reinterpret_cast<const uint4*>(krow + d) : zero;
             }
         }
-        // ---- values of the lane's 8 keys j0 + 8g .. +7, for every block of 16 dimensions
         const int jk = j0 + 8 * g;
-        uint4 vf[DB];
-        {
-            const bool chunk_ok = jk <= p_max;
-            const bf16* vrow = nullptr;
-            if (chunk_ok) {
-                const int page = table[jk / a.block_size];
-                vrow = v_base + (size_t)page * page_stride + (jk % a.block_size);
-            }
-            // keys outside [lo_min, p_max] may be stale or never written: their values become 0
-            const int first = lo_min - jk, last = p_max + 1 - jk;
-#pragma unroll
-            for (int m = 0; m < DB; ++m) {
-                uint4 v = chunk_ok ? *reinterpret_cast<const uint4*>(vrow + (size_t)(16 * m + col) * a.block_size) : zero;
-                vf[m] = keep_elements(v, first, last);
-            }
+        const bool chunk_ok = jk <= p_max;
+        const bf16* vrow = nullptr;
+        if (chunk_ok) {
+            int page, off;
+            locate(jk, page, off);
+            vrow = v_base + (size_t)page * page_stride + off;
         }
+        const int first = lo_min - jk, last = p_max + 1 - jk;
+#pragma unroll
+        for (int m = 0; m < DB; ++m) {
+            const uint4 v = chunk_ok ? *reinterpret_cast<const uint4*>(vrow + (size_t)(16 * m + col) * a.block_size) : zero;
+            vf[m] = keep_elements(v, first, last);
+        }
+    };
+
+    // the next tile's operands are requested before this tile's arithmetic starts
+    uint4 kf_next[2][KS], vf_next[DB];
+    if (t_begin < t_end) load_tile(j_begin + 32 * t_begin, kf_next, vf_next);
+    for (int t = t_begin; t < t_end; t += t_step) {
+        const int j0 = j_begin + 32 * t;
+        uint4 kf[2][KS], vf[DB];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int s = 0; s < KS; ++s) kf[u][s] = kf_next[u][s];
+#pragma unroll
+        for (int m = 0; m < DB; ++m) vf[m] = vf_next[m];
+        if (t + t_step < t_end) load_tile(j_begin + 32 * (t + t_step), kf_next, vf_next);
+        f32x4 s_acc[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            s_acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; ++s)
+                s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u][s]), as_bf16x8(qf[s]), s_acc[u], 0, 0, 0);
+        }
+        const int jk = j0 + 8 * g;
         // ---- online softmax of this lane's column over its 8 keys (and the 3 other lane groups)
         float sc[8];
         float tmax = -INFINITY;

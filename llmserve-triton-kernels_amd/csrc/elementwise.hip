@@ -64,6 +64,7 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, const T* x, const T* __restr
 //   q, k: x' = x*cos + rotate_half(x)*sin with pairs (i, i + D/2) and angle
 //         float(position) * inv_freq[i]  (src/llmserve/model/llama.py:31-54), computed in
 //         32-bit and rounded once.  q is rotated in place.  inv_freq == nullptr: no rotation.
+//   Without pools (k_pool == nullptr) k is rotated in place as well and nothing is stored.  With pools
 //   k' goes to k_pool[page, kv_head, offset, :], v to v_pool[page, kv_head, :, offset]
 //   (values transposed inside a page so that attention reads keys of one dimension
 //   contiguously), page = slot / block_size, offset = slot % block_size.  slot < 0: no store.
@@ -94,7 +95,7 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const float* __restrict__
             ra = a * cs - b * sn;
             rb = b * cs + a * sn;
         }
-        if (h < n_heads) {
+        if (h < n_heads || k_pool == nullptr) {
             x[i] = from_f32<T>(ra);
             x[i + half] = from_f32<T>(rb);
         } else if (slot >= 0) {

@@ -39,6 +39,7 @@ class StepBatch:
     # host copies, for choosing kernels without a read-back
     counts: list[int] = field(default_factory=list)
     starts: list[int] = field(default_factory=list)
+    state_slot_list: list[int] = field(default_factory=list)  # host copy of state_slots
     num_decode: int = 0  # leading requests that bring exactly one token
     max_count: int = 0
     max_context: int = 0
@@ -126,8 +127,9 @@ def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[in
         num_tokens=n_tokens, num_seqs=n_seqs, token_ids=view(0, n_tokens), positions=view(1, n_tokens),
         token_seq=view(2, n_tokens), cu_seqlens=view(3, n_seqs + 1), context_lens=view(4, n_seqs),
         state_slots=view(5, n_seqs), logit_rows=view(6, len(logit_rows)), groups=groups,
-        counts=list(counts), starts=list(starts), num_decode=num_decode, max_count=max(counts),
-        max_context=max(context), max_decode_context=max(context[:num_decode], default=0))
+        counts=list(counts), starts=list(starts), state_slot_list=list(layout.state_slots),
+        num_decode=num_decode, max_count=max(counts), max_context=max(context),
+        max_decode_context=max(context[:num_decode], default=0))
 
 
 class StaticDecodeBatch:

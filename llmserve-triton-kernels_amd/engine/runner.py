@@ -66,7 +66,7 @@ class ModelRunner:
                                     self.dtype, device)
         self._uploader = BatchUploader(device)
         self._graphs: dict[tuple[int, int], "_DecodeGraph"] = {}
-        self._use_graphs = engine_config.use_graphs
+        self._use_graphs = engine_config.use_graphs and model.graph_safe()
 
     # ---- construction ---------------------------------------------------------------------
     @staticmethod

@@ -4,6 +4,7 @@ from .registry import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, 
                        BuildContext, FeedForward, Mixer, Norm, Part, PositionEncoding, register_block,
                        register_feed_forward, register_mixer, register_norm, register_position_encoding)
 from .spec import LayerSpec, ModelSpec, PagedCacheSpec, ParamInfo, PartSpec, StateCacheSpec
+from . import attention, block, embedding, rmsnorm, rope, swiglu  # noqa: E402,F401  (register the built-in parts)
 
 __all__ = [
     "BLOCKS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "Block",

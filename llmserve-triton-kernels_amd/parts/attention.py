@@ -23,6 +23,8 @@ from .spec import PagedCacheSpec, ParamInfo
 
 @register_mixer("attention")
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
         self.hidden = int(spec["hidden"])

@@ -14,6 +14,8 @@ from .spec import ParamInfo
 
 @EMBEDDINGS.register("embedding")
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
         self.vocab = int(spec["vocab"])
@@ -35,6 +37,8 @@ class TokenEmbedding(Part):
 class LMHead(Part):
     """Parameters: vocab, hidden, tied.  A tied head has no tensor of its own: the model
     hands it the embedding table."""
+    graph_safe = True
+
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)

@@ -25,6 +25,7 @@ class Model:
         self.final_norm = NORMS.build(spec.final_norm, ctx)
         self.head = HEADS.build(spec.head, ctx)
         self.blocks = []
+        self._sources = None
         for layer in spec.layers:
             self.blocks.append(BLOCKS.get(layer.block)(
                 MIXERS.build(layer.mixer, ctx), FEED_FORWARDS.build(layer.feed_forward, ctx),
@@ -58,18 +59,40 @@ class Model:
         if getattr(self.head, "tied", False):
             self.head.load({"weight": self.embedding.weight})
 
+    def graph_safe(self) -> bool:
+        """Whether a decode-only step through this model may be captured as a HIP graph."""
+        parts = [part for _, part in self._parts()]
+        parts += [getattr(blk.mixer, "position", None) for blk in self.blocks]
+        return all(p.graph_safe for p in parts if p is not None)
+
     def cache_specs(self) -> list:
-        """Per layer what its mixer keeps between steps (None when it borrows another layer's)."""
-        return [None if layer.cache_from is not None else blk.mixer.cache_spec()
-                for layer, blk in zip(self.spec.layers, self.blocks)]
+        """What each entry of the schedule keeps between steps (None when its layer borrows
+        another layer's cache).  A layer that runs twice keeps two caches, one per run: the keys
+        of its second run are not those of its first."""
+        return [None if self.spec.layers[i].cache_from is not None else self.blocks[i].mixer.cache_spec()
+                for i in self.spec.schedule]
+
+    def cache_sources(self) -> list:
+        """For each entry of the schedule the entry whose cache it reads instead of its own: the
+        latest earlier run of the layer named by `cache_from` (None: its own)."""
+        sources = []
+        for pos, i in enumerate(self.spec.schedule):
+            src = self.spec.layers[i].cache_from
+            if src is None:
+                sources.append(None)
+            else:
+                sources.append(max(p for p in range(pos) if self.spec.schedule[p] == src))
+        return sources
 
     # ---- one step ----------------------------------------------------------------------------
     def forward(self, batch, storage) -> torch.Tensor:
         """Logits [R, vocab] in 32-bit at `batch.logit_rows` (empty tensor when R = 0)."""
         x = self.embedding.forward(batch.token_ids)
         delta = None
-        for index in self.spec.schedule:
-            cache = storage.layer_cache(index, self.spec.layers[index].cache_from)
+        if self._sources is None:
+            self._sources = self.cache_sources()
+        for pos, index in enumerate(self.spec.schedule):
+            cache = storage.layer_cache(pos, self._sources[pos])
             x, delta = self.blocks[index].forward(x, delta, batch, cache)
         rows = batch.logit_rows
         if rows.numel() == 0:

@@ -35,7 +35,14 @@ class BuildContext:
 
 
 class Part:
-    """Base of every part.  `param_infos` lists its tensors under their own (local) names."""
+    """Base of every part.  `param_infos` lists its tensors under their own (local) names.
+
+    `graph_safe`: the part's forward only launches device work whose arguments do not depend
+    on the host-side fields of the batch (counts, starts, slot lists), so a decode-only step
+    through it may be captured once as a HIP graph and replayed.  A part that reads those
+    fields on the host leaves it False, and the engine then launches every step afresh."""
+
+    graph_safe = False
 
     def __init__(self, spec: PartSpec, ctx: BuildContext):
         self.spec = spec

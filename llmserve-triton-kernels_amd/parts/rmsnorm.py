@@ -12,6 +12,8 @@ from .spec import ParamInfo
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
         self.hidden = int(spec["hidden"])

@@ -17,6 +17,8 @@ from .registry import PositionEncoding, register_position_encoding
 
 @register_position_encoding("rope")
 class RotaryEncoding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
         self.head_dim = int(spec["head_dim"])
@@ -43,6 +45,8 @@ class RotaryEncoding(PositionEncoding):
 @register_position_encoding("none")
 class NoPositionEncoding(PositionEncoding):
     """Keys and queries are used as projected."""
+    graph_safe = True
+
 
     def rotate(self, qkv, positions, n_heads, n_kv_heads, head_dim):
         return None

@@ -32,7 +32,7 @@ class LayerSpec:
     `weights` maps each role ("mixer", "feed_forward", "mixer_norm", "feed_forward_norm")
     to the checkpoint prefix of that part's tensors; a part's own tensor names are appended
     to it.  `cache_from` names another layer whose cache this layer's mixer reads instead
-    of keeping one of its own.
+    of keeping one of its own (the cache of that layer's latest run earlier in the schedule).
     """
 
     mixer: PartSpec
@@ -74,6 +74,10 @@ class ModelSpec:
                 first_use = self.schedule.index(i) if i in self.schedule else None
                 if first_use is not None and (first_own is None or first_own > first_use):
                     raise ValueError(f"layer {i} reads the cache of layer {src} before that layer has run")
+                a, b = self.layers[i].mixer, self.layers[src].mixer
+                for key in ("num_kv_heads", "head_dim"):
+                    if a.get(key) != b.get(key):
+                        raise ValueError(f"layer {i} cannot read the cache of layer {src}: {key} differs")
 
 
 # ---------------------------------------------------------------- what a mixer keeps per request

@@ -15,6 +15,8 @@ from .spec import ParamInfo
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
         self.hidden = int(spec["hidden"])
