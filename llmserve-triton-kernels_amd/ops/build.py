@@ -33,10 +33,11 @@ HIPCC_FLAGS = [
     "-Wno-unused-result", "-Wno-unknown-warning-option",
 ]
 
-# Which libraries a model of a given dtype needs.
+# Which libraries the step function of a model of a given dtype needs (the sampler's library is
+# built when something is first sampled).
 GROUPS = {
-    "float32": ("elementwise", "gemm", "attention", "sampling"),
-    "bfloat16": ("elementwise", "gemm", "attention", "sampling", "gemm_mfma", "attention_mfma"),
+    "float32": ("elementwise", "gemm", "attention"),
+    "bfloat16": ("elementwise", "gemm", "attention", "gemm_mfma", "attention_mfma"),
 }
 
 

@@ -124,3 +124,74 @@ def test_trace_run_program(model_dirs, tmp_path, dtype_name):
         if wanted:
             outputs[rec["step"]] = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(wanted, vocab).copy())
     check_against_plain(model_dirs[name], dtype_name, seqs, steps, outputs)
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_long_decoding(model_dirs, dtype_name):
+    """A short prompt, then more than two hundred tokens one by one: every page edge is crossed by a
+    single token, and the replayed graphs see contexts far beyond the one they were captured at."""
+    ids = traces.random_ids(TINY["b"][0]["vocab_size"], 250, 4242)
+    seqs = {"long": ids}
+    steps = traces.prefill_then_decode(seqs, tail=230)
+    outputs = replay_in_process(model_dirs["b"], dtype_name, steps, 8, 32)
+    check_against_plain(model_dirs["b"], dtype_name, seqs, steps, outputs)
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+@pytest.mark.parametrize("name", list(TINY))
+def test_first_tokens(model_dirs, name, dtype_name):
+    """The first tokens of a sequence: prompts of one, two and three tokens, whole and token by token
+    (position 0 attends to itself only; a one-token prompt is prefill and decode at once)."""
+    vocab = TINY[name][0]["vocab_size"]
+    seqs = {f"s{n}": traces.random_ids(vocab, n, 70 + n) for n in (1, 2, 3, 4)}
+    for steps in (traces.whole(seqs), traces.prefill_then_decode(seqs, tail=8)):
+        outputs = replay_in_process(model_dirs[name], dtype_name, steps, TINY[name][1], 4)
+        check_against_plain(model_dirs[name], dtype_name, seqs, steps, outputs)
+    # all four at once, one token each per step
+    steps, pos = [], 0
+    while any(pos < len(ids) for ids in seqs.values()):
+        entries = [{"id": r, "tokens": [ids[pos]], "want": [0]} for r, ids in seqs.items() if pos < len(ids)]
+        steps.append({"step": pos, "entries": entries, "end": [r for r, ids in seqs.items() if pos == len(ids) - 1]})
+        pos += 1
+    outputs = replay_in_process(model_dirs[name], dtype_name, steps, TINY[name][1], 4)
+    check_against_plain(model_dirs[name], dtype_name, seqs, steps, outputs)
+
+
+@pytest.fixture(scope="module")
+def sharp_dir(model_dirs, tmp_path_factory):
+    """Tiny B with query and key projections scaled up, so that attention has favourites among the
+    keys instead of the near-uniform weights that small random matrices give: a key that is missed,
+    or read from the wrong page, then changes the logits by much more than the tolerance."""
+    import shutil
+
+    from safetensors.torch import load_file, save_file
+
+    d = tmp_path_factory.mktemp("tiny_b_sharp")
+    shutil.copy(model_dirs["b"] / "config.json", d / "config.json")
+    w = load_file(str(model_dirs["b"] / "model.safetensors"))
+    for k in w:
+        if k.endswith("q_proj.weight") or k.endswith("k_proj.weight"):
+            w[k] = w[k] * 6.0
+    save_file(w, str(d / "model.safetensors"))
+    return d
+
+
+@pytest.mark.parametrize("mode", ["portions", "mixed"])
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_replay_with_sharp_attention(sharp_dir, dtype_name, mode):
+    seqs = sequences("b")
+    ref = traces.plain_logits(sharp_dir, seqs["b5"], torch.float32)
+    flat = traces.plain_logits(TINY_DIRS["b"], seqs["b5"], torch.float32) if "b" in TINY_DIRS else None
+    steps = MODES[mode](seqs)
+    num_blocks = traces.tokens_needed(steps, round_to=8) // 8
+    outputs = replay_in_process(sharp_dir, dtype_name, steps, 8, num_blocks)
+    check_against_plain(sharp_dir, dtype_name, seqs, steps, outputs)
+    assert flat is None or (ref - flat).abs().max() > 1e-3
+
+
+TINY_DIRS: dict = {}
+
+
+@pytest.fixture(autouse=True)
+def _remember_dirs(model_dirs):
+    TINY_DIRS.update(model_dirs)
