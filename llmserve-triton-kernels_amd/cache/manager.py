@@ -54,7 +54,9 @@ class StepLayout:
     state_slots: list[int]
     fresh_slots: list[int]  # slots whose state must be cleared before this step runs
     slots: dict[int, list[int]] = field(default_factory=dict)  # group -> cache slot of every new token
-    tables: dict[int, list[list[int]]] = field(default_factory=dict)  # group -> block table per request
+    # group -> (state slot of the request, index in its block table, page) for every page taken in this
+    # step: what a device copy of the tables, one row per state slot, has to be told
+    table_updates: dict[int, list[tuple[int, int, int]]] = field(default_factory=dict)
 
 
 class CacheManager:
@@ -70,6 +72,7 @@ class CacheManager:
         self.tables: dict[int, dict] = {g.group_id: {} for g in self.paged_groups}
         self.lengths: dict = {}
         self.slot_of: dict = {}
+        self._windowed = [g for g in self.paged_groups if g.spec.window is not None]
         self._slot_alloc = BlockAllocator(max_seqs)
         self._fresh: set[int] = set()
 
@@ -176,17 +179,28 @@ class CacheManager:
         for g in self.paged_groups:
             alloc, tables = self.allocators[g.group_id], self.tables[g.group_id]
             token_slots: list[int] = []
-            for s, n, start in zip(seq_ids, counts, layout.starts):
+            updates: list[tuple[int, int, int]] = []
+            for s, n, start, row in zip(seq_ids, counts, layout.starts, layout.state_slots):
                 table = tables[s]
-                while len(table) < self.blocks_for(start + n):
-                    table.append(alloc.allocate())
-                for p in range(start, start + n):
-                    token_slots.append(table[p // bs] * bs + p % bs)
+                want = -(-(start + n) // bs)
+                while len(table) < want:
+                    page = alloc.allocate()
+                    updates.append((row, len(table), page))
+                    table.append(page)
+                if n == 1:
+                    token_slots.append(table[start // bs] * bs + start % bs)
+                else:
+                    for p in range(start, start + n):
+                        token_slots.append(table[p // bs] * bs + p % bs)
             layout.slots[g.group_id] = token_slots
-            layout.tables[g.group_id] = [list(tables[s]) for s in seq_ids]
+            layout.table_updates[g.group_id] = updates
         for s, n in zip(seq_ids, counts):
             self.lengths[s] += n
         return layout
+
+    def table(self, group_id: int, seq_id) -> list[int]:
+        """The request's block table in one group (-1: a page that was given back)."""
+        return self.tables[group_id][seq_id]
 
     def release_passed(self, seq_ids) -> int:
         """After a step: return the pages of windowed groups that no later query can reach.
@@ -196,10 +210,10 @@ class CacheManager:
         Returns the number of pages given back.
         """
         bs, freed = self.block_size, 0
-        for g in self.paged_groups:
+        if not self._windowed:
+            return 0
+        for g in self._windowed:
             window = g.spec.window
-            if window is None:
-                continue
             for s in seq_ids:
                 if s not in self.lengths:
                     continue

@@ -4,7 +4,8 @@ Per paged group and owning layer: keys `[pages, kv_heads, block_size, head_dim]`
 `[pages, kv_heads, head_dim, block_size]` (values are stored transposed inside a page, so a
 kernel reads the keys' worth of one value dimension contiguously).  The reference keeps
 `[layers, pages, kv_heads, block_size, head_dim]` for both (src/llmserve/kvcache/paged.py:126-128).
-Per state group and owning layer: `[slots, *shape]`.
+Per state group and owning layer: `[slots, *shape]`.  Per paged group the block tables, `[slots, width]`
+int32: a request's row is its state slot, entries beyond its length are stale and never read.
 """
 
 from __future__ import annotations
@@ -51,8 +52,13 @@ def num_blocks_for_budget(groups: list[CacheGroup], block_size: int, elem_size: 
 
 class CacheStorage:
     def __init__(self, groups: list[CacheGroup], num_blocks: int, block_size: int, max_seqs: int,
-                 dtype: torch.dtype, device: torch.device):
+                 dtype: torch.dtype, device: torch.device, table_width: int = 1):
+        """`table_width`: most pages a request can hold (longest request / block_size)."""
         self.groups = groups
+        self.max_seqs = max_seqs
+        self.table_width = table_width
+        # block tables live on the device, one row per state slot; a step only sends the pages it took
+        self.tables: dict[int, torch.Tensor] = {}
         self.block_size = block_size
         self.num_blocks = num_blocks
         self._owner: dict[int, tuple[int, int]] = {}  # layer -> (group, index in group)
@@ -69,6 +75,7 @@ class CacheStorage:
                                                  dtype=dtype, device=device)
                 self.v[g.group_id] = torch.zeros((n, num_blocks, s.num_kv_heads, s.head_dim, block_size),
                                                  dtype=dtype, device=device)
+                self.tables[g.group_id] = torch.zeros((max_seqs, table_width), dtype=torch.int32, device=device)
             else:
                 self.state[g.group_id] = torch.zeros((n, max_seqs, *g.spec.shape),
                                                      dtype=getattr(torch, g.spec.dtype), device=device)

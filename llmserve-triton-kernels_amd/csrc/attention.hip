@@ -16,8 +16,8 @@
 template <typename T>
 __global__ __launch_bounds__(ATT_WAVES* LLMS_WAVE) void attention_wave_kernel(
     T* __restrict__ out, int out_stride, const T* __restrict__ q, int q_stride, const T* __restrict__ k_pool,
-    const T* __restrict__ v_pool, const int* __restrict__ block_tables, int max_blocks,
-    const int* __restrict__ token_seq, const int* __restrict__ positions, int n_heads, int n_kv_heads,
+    const T* __restrict__ v_pool, const int* __restrict__ block_tables, const int* __restrict__ table_rows,
+    int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions, int n_heads, int n_kv_heads,
     int head_dim, int block_size, int window, float scale) {
     __shared__ float qs[ATT_WAVES][ATT_MAX_D];
     const int n = blockIdx.x;
@@ -32,7 +32,8 @@ __global__ __launch_bounds__(ATT_WAVES* LLMS_WAVE) void attention_wave_kernel(
     if (!active) return;
 
     const int p = positions[n];
-    const int* table = block_tables + (size_t)token_seq[n] * max_blocks;
+    const int seq = token_seq[n];
+    const int* table = block_tables + (size_t)(table_rows ? table_rows[seq] : seq) * max_blocks;
     const int kvh = h / (n_heads / n_kv_heads);
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
 
@@ -80,7 +81,8 @@ __global__ __launch_bounds__(ATT_WAVES* LLMS_WAVE) void attention_wave_kernel(
 extern "C" {
 
 int llms_attention_wave(int dtype, void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
-                        const void* v_pool, const int* block_tables, int max_blocks, const int* token_seq,
+                        const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
+                        const int* token_seq,
                         const int* positions, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                         int block_size, int window, float scale, hipStream_t stream) {
     LLMS_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0, "attention: sizes must be positive");
@@ -93,12 +95,12 @@ int llms_attention_wave(int dtype, void* out, int out_stride, const void* q, int
     if (dtype == 0) {
         attention_wave_kernel<float><<<grid, ATT_WAVES * LLMS_WAVE, 0, stream>>>(
             (float*)out, out_stride, (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool,
-            block_tables, max_blocks, token_seq, positions, n_heads, n_kv_heads, head_dim, block_size, window,
+            block_tables, table_rows, max_blocks, token_seq, positions, n_heads, n_kv_heads, head_dim, block_size, window,
             scale);
     } else if (dtype == 1) {
         attention_wave_kernel<bf16><<<grid, ATT_WAVES * LLMS_WAVE, 0, stream>>>(
             (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pool, (const bf16*)v_pool,
-            block_tables, max_blocks, token_seq, positions, n_heads, n_kv_heads, head_dim, block_size, window,
+            block_tables, table_rows, max_blocks, token_seq, positions, n_heads, n_kv_heads, head_dim, block_size, window,
             scale);
     } else {
         LLMS_REQUIRE(false, "attention: dtype must be 0 (float32) or 1 (bfloat16)");

@@ -51,6 +51,7 @@ struct AttnArgs {
     const bf16* k_pool;
     const bf16* v_pool;
     const int* block_tables;
+    const int* table_rows;  // row of block_tables of each request (null: the request's own index)
     int max_blocks;
     const int* cu_seqlens;
     const int* context_lens;
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnArgs a) {
     for (int m = 0; m < DB; ++m) acc[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    const int* table = a.block_tables + (size_t)b * a.max_blocks;
+    const int* table = a.block_tables + (size_t)(a.table_rows ? a.table_rows[b] : b) * a.max_blocks;
     const size_t page_stride = (size_t)a.n_kv_heads * a.block_size * D;
     const bf16* k_base = a.k_pool + (size_t)kvh * a.block_size * D;
     const bf16* v_base = a.v_pool + (size_t)kvh * a.block_size * D;
@@ -357,7 +358,8 @@ extern "C" {
 // workgroups (decoding); with num_splits > 1 the caller provides ws_o [tokens * heads * splits * D] and
 // ws_ml [tokens * heads * splits * 2] floats, indexed by absolute token row.
 int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
-                        const void* v_pool, const int* block_tables, int max_blocks, const int* cu_seqlens,
+                        const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
+                        const int* cu_seqlens,
                         const int* context_lens, int seq_begin, int n_seqs, int max_new, int token_begin,
                         int n_tokens, int n_heads, int n_kv_heads, int head_dim, int block_size, int window,
                         float scale, int split_waves, int num_splits, float* ws_o, float* ws_ml,
@@ -377,7 +379,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     const int G = n_heads / n_kv_heads, HG = G < 16 ? G : 16, TPG = 16 / HG, HB = (G + HG - 1) / HG;
     const int groups = (max_new + TPG - 1) / TPG;
     AttnArgs a = {(bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pool, (const bf16*)v_pool,
-                  block_tables, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
+                  block_tables, table_rows, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
                   window, scale, num_splits, ws_o, ws_ml};
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
     if (split_waves) {

@@ -59,6 +59,70 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, const T* x, const T* __restr
     }
 }
 
+// The same for bfloat16 rows of hidden % 8 == 0 and hidden <= 8 * RV_CHUNKS * blockDim: every thread keeps
+// its elements in registers (16-byte loads and stores), so the row is read once.
+#define RV_CHUNKS 4
+__global__ void rmsnorm_bf16_vec_kernel(bf16* __restrict__ out, const bf16* x, const bf16* __restrict__ delta,
+                                        bf16* resid_out, const bf16* __restrict__ weight,
+                                        const int* __restrict__ rows, float eps, int hidden) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const int s = rows ? rows[r] : r;
+    const uint4* xs = reinterpret_cast<const uint4*>(x + (size_t)s * hidden);
+    const uint4* ds = delta ? reinterpret_cast<const uint4*>(delta + (size_t)s * hidden) : nullptr;
+    uint4* rs = resid_out ? reinterpret_cast<uint4*>(resid_out + (size_t)s * hidden) : nullptr;
+    const int nchunks = hidden / 8;
+    float v[RV_CHUNKS][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < RV_CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nchunks) {
+            const uint4 xv = xs[i];
+            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+            uint32_t dw[4] = {0, 0, 0, 0};
+            if (ds) {
+                const uint4 dv = ds[i];
+                dw[0] = dv.x; dw[1] = dv.y; dw[2] = dv.z; dw[3] = dv.w;
+            }
+            uint32_t ow[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float lo = bf16_bits_to_f32((uint16_t)(xw[j] & 0xffffu)), hi = bf16_bits_to_f32((uint16_t)(xw[j] >> 16));
+                if (ds) {
+                    lo = bf16_bits_to_f32(f32_to_bf16_bits(lo + bf16_bits_to_f32((uint16_t)(dw[j] & 0xffffu))));
+                    hi = bf16_bits_to_f32(f32_to_bf16_bits(hi + bf16_bits_to_f32((uint16_t)(dw[j] >> 16))));
+                }
+                v[c][2 * j] = lo;
+                v[c][2 * j + 1] = hi;
+                ss += lo * lo + hi * hi;
+                ow[j] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+            }
+            if (rs) rs[i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+        }
+    }
+    ss = block_sum(ss, red);
+    const float inv = rsqrtf(ss / (float)hidden + eps);
+    const uint4* ws = reinterpret_cast<const uint4*>(weight);
+    uint4* o = reinterpret_cast<uint4*>(out + (size_t)r * hidden);
+#pragma unroll
+    for (int c = 0; c < RV_CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nchunks) {
+            const uint4 wv = ws[i];
+            const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+            uint32_t ow[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float lo = bf16_bits_to_f32((uint16_t)(ww[j] & 0xffffu)) * round_to<bf16>(v[c][2 * j] * inv);
+                const float hi = bf16_bits_to_f32((uint16_t)(ww[j] >> 16)) * round_to<bf16>(v[c][2 * j + 1] * inv);
+                ow[j] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+            }
+            o[i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ rotary encoding + cache store
 // qkv row n = [q heads | k heads | v heads], head_dim wide each.
 //   q, k: x' = x*cos + rotate_half(x)*sin with pairs (i, i + D/2) and angle
@@ -130,6 +194,41 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gate_
     out[idx] = from_f32<T>(s * u);
 }
 
+// bfloat16 rows of inter % 8 == 0: 8 elements per thread, 16-byte loads and stores.
+__global__ void silu_mul_bf16_vec_kernel(bf16* __restrict__ out, const bf16* __restrict__ gate_up, int inter,
+                                         size_t total_chunks) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total_chunks) return;
+    const int cpr = inter / 8;  // chunks per row
+    const size_t n = idx / cpr;
+    const int c = (int)(idx % cpr);
+    const uint4* row = reinterpret_cast<const uint4*>(gate_up + n * 2 * (size_t)inter);
+    const uint4 gv = row[c], uv = row[cpr + c];
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float r2[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float g = bf16_bits_to_f32((uint16_t)(h ? gw[j] >> 16 : gw[j] & 0xffffu));
+            const float u = bf16_bits_to_f32((uint16_t)(h ? uw[j] >> 16 : uw[j] & 0xffffu));
+            r2[h] = round_to<bf16>(g / (1.f + expf(-g))) * u;
+        }
+        ow[j] = (uint32_t)f32_to_bf16_bits(r2[0]) | ((uint32_t)f32_to_bf16_bits(r2[1]) << 16);
+    }
+    reinterpret_cast<uint4*>(out)[idx] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
+// ------------------------------------------------------------------ scattered int32 writes
+// dst[index[i]] = value[i] for index[i] >= 0: how a step's new pages reach the block tables that
+// stay on the device.
+__global__ void scatter_i32_kernel(int* __restrict__ dst, const int* __restrict__ index,
+                                   const int* __restrict__ value, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && index[i] >= 0) dst[index[i]] = value[i];
+}
+
 // ------------------------------------------------------------------ launchers
 #define DISPATCH_DTYPE(dtype, ...)                 \
     if ((dtype) == 0) {                            \
@@ -156,6 +255,16 @@ int llms_rmsnorm(int dtype, void* out, const void* x, const void* delta, void* r
                  const int* rows, float eps, int n_rows, int hidden, hipStream_t stream) {
     LLMS_REQUIRE(n_rows > 0 && hidden > 0, "rmsnorm: sizes must be positive");
     LLMS_REQUIRE(!(rows && resid_out), "rmsnorm: a row gather cannot also write the residual back");
+    if (dtype == 1 && hidden % 8 == 0 && hidden <= 8 * RV_CHUNKS * 256 && ((uintptr_t)x % 16) == 0 &&
+        ((uintptr_t)out % 16) == 0 && ((uintptr_t)weight % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0) &&
+        (!resid_out || ((uintptr_t)resid_out % 16) == 0)) {
+        const int chunks = hidden / 8;
+        const int threads = chunks <= 64 ? 64 : chunks <= 128 ? 128 : 256;
+        rmsnorm_bf16_vec_kernel<<<n_rows, threads, 0, stream>>>((bf16*)out, (const bf16*)x, (const bf16*)delta,
+                                                                (bf16*)resid_out, (const bf16*)weight, rows, eps,
+                                                                hidden);
+        LLMS_LAUNCH_CHECK();
+    }
     const int threads = hidden >= 2048 ? 512 : 256;
     DISPATCH_DTYPE(dtype, rmsnorm_kernel<T><<<n_rows, threads, 0, stream>>>(
                               (T*)out, (const T*)x, (const T*)delta, (T*)resid_out, (const T*)weight, rows,
@@ -176,9 +285,21 @@ int llms_rope_store(int dtype, void* qkv, const float* inv_freq, const int* posi
     LLMS_LAUNCH_CHECK();
 }
 
+int llms_scatter_i32(int* dst, const int* index, const int* value, int n, hipStream_t stream) {
+    LLMS_REQUIRE(n > 0 && dst && index && value, "scatter_i32: bad arguments");
+    scatter_i32_kernel<<<(n + 255) / 256, 256, 0, stream>>>(dst, index, value, n);
+    LLMS_LAUNCH_CHECK();
+}
+
 int llms_silu_mul(int dtype, void* out, const void* gate_up, int n_rows, int inter, hipStream_t stream) {
     LLMS_REQUIRE(n_rows > 0 && inter > 0, "silu_mul: sizes must be positive");
     const size_t total = (size_t)n_rows * inter;
+    if (dtype == 1 && inter % 8 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)gate_up % 16) == 0) {
+        const size_t chunks = total / 8;
+        silu_mul_bf16_vec_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, stream>>>((bf16*)out, (const bf16*)gate_up,
+                                                                                         inter, chunks);
+        LLMS_LAUNCH_CHECK();
+    }
     const unsigned blocks = (unsigned)((total + 255) / 256);
     DISPATCH_DTYPE(dtype, silu_mul_kernel<T><<<blocks, 256, 0, stream>>>((T*)out, (const T*)gate_up, inter,
                                                                           total);)

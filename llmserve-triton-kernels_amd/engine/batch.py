@@ -20,7 +20,7 @@ from ..cache.manager import StepLayout
 class GroupView:
     """One cache group's part of a step."""
 
-    block_tables: torch.Tensor  # int32 [B, M]; entries of returned pages are 0 and never read
+    block_tables: torch.Tensor  # int32 [state slots, M], resident on the device; request b owns row state_slots[b]
     slots: torch.Tensor  # int32 [N]: page * block_size + offset of every new token
 
 
@@ -77,9 +77,22 @@ class BatchUploader:
         return dev
 
 
-def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[int],
-                uploader: BatchUploader) -> StepBatch:
-    """Device tensors for a step whose pages `layout` has already fixed."""
+def _update_arrays(updates: list[tuple[int, int, int]], width: int, rows: int) -> tuple[list[int], list[int]]:
+    index, value = [], []
+    for row, i, page in updates:
+        if not (0 <= row < rows and 0 <= i < width):
+            raise ValueError(f"block table entry ({row}, {i}) is outside the device table [{rows}, {width}]")
+        index.append(row * width + i)
+        value.append(page)
+    return index, value
+
+
+def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[int], uploader: BatchUploader,
+                storage) -> StepBatch:
+    """Device tensors for a step whose pages `layout` has already fixed; the pages it took are written
+    into the device-resident block tables of `storage`."""
+    from ..ops import library as ops
+
     counts, starts = layout.counts, layout.starts
     n_seqs = len(counts)
     flat_tokens = [t for row in tokens for t in row]
@@ -93,17 +106,12 @@ def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[in
 
     sections: list[list[int]] = [flat_tokens, positions, token_seq, cu, context, layout.state_slots,
                                  list(logit_rows)]
-    group_ids = sorted(layout.tables)
-    widths = {}
+    group_ids = sorted(layout.slots)
+    n_updates = {}
     for g in group_ids:
-        width = max(1, max(len(t) for t in layout.tables[g]))
-        widths[g] = width
-        table_flat: list[int] = []
-        for t in layout.tables[g]:
-            table_flat.extend(b if b >= 0 else 0 for b in t)
-            table_flat.extend([0] * (width - len(t)))
-        sections.append(layout.slots[g])
-        sections.append(table_flat)
+        index, value = _update_arrays(layout.table_updates[g], storage.table_width, storage.max_seqs)
+        n_updates[g] = len(index)
+        sections += [layout.slots[g], index, value]
     flat: list[int] = []
     offsets = []
     for sec in sections:
@@ -117,9 +125,9 @@ def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[in
 
     groups = {}
     for j, g in enumerate(group_ids):
-        slots = view(7 + 2 * j, n_tokens)
-        tables = view(8 + 2 * j, n_seqs * widths[g]).view(n_seqs, widths[g])
-        groups[g] = GroupView(tables, slots)
+        if n_updates[g]:
+            ops.scatter_i32(storage.tables[g], view(8 + 3 * j, n_updates[g]), view(9 + 3 * j, n_updates[g]))
+        groups[g] = GroupView(storage.tables[g], view(7 + 3 * j, n_tokens))
     num_decode = 0
     while num_decode < n_seqs and counts[num_decode] == 1:
         num_decode += 1
@@ -135,69 +143,82 @@ def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[in
 class StaticDecodeBatch:
     """Fixed device buffers for decode-only steps of up to `capacity` requests, so that such a step
     can be captured once as a HIP graph and replayed: every step writes its tokens, positions, slots,
-    block tables and context lengths into the same memory with one copy.  Unused rows belong to
+    context lengths and newly taken pages into the same memory with one copy.  Unused rows belong to
     dummy requests of context length 0, which every kernel leaves alone or computes harmlessly
     (rows never mix)."""
 
-    def __init__(self, capacity: int, table_width: int, group_ids: list[int], device: torch.device):
+    def __init__(self, capacity: int, storage, group_ids: list[int], device: torch.device):
         self.capacity = capacity
-        self.table_width = table_width
+        self.storage = storage
         self.group_ids = list(group_ids)
-        c, w = capacity, table_width
-        pad = lambda n: n + (-n % 4)  # noqa: E731
-        sizes = [c, c, c, c + 1, c, c, c] + [x for _ in group_ids for x in (c, c * w)]
+        c = capacity
+        sizes = [c, c, c, c + 1, c, c, c] + [c] * (3 * len(group_ids))
         self._offsets, total = [], 0
         for n in sizes:
             self._offsets.append(total)
-            total += pad(n)
+            total += n + (-n % 4)
         self._sizes = sizes
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
         self.dev = torch.zeros(total, dtype=torch.int32, device=device)
         self._event = None
         v = self._view
-        groups = {g: GroupView(v(8 + 2 * j).view(c, w), v(7 + 2 * j)) for j, g in enumerate(group_ids)}
+        groups = {g: GroupView(storage.tables[g], v(7 + 3 * j)) for j, g in enumerate(group_ids)}
         self.batch = StepBatch(
             num_tokens=c, num_seqs=c, token_ids=v(0), positions=v(1), token_seq=v(2), cu_seqlens=v(3),
             context_lens=v(4), state_slots=v(5), logit_rows=v(6), groups=groups, counts=[1] * c, starts=[0] * c,
-            num_decode=c, max_count=1, max_context=1, max_decode_context=1)
+            state_slot_list=[0] * c, num_decode=c, max_count=1, max_context=1, max_decode_context=1)
         # what never changes: one token per request, every row's logits wanted
         h = self._host_view
-        h(2)[:] = torch.arange(c, dtype=torch.int32)
-        h(3)[:] = torch.arange(c + 1, dtype=torch.int32)
-        h(6)[:] = torch.arange(c, dtype=torch.int32)
+        h(2)[:] = range(c)
+        h(3)[:] = range(c + 1)
+        h(6)[:] = range(c)
         for j in range(len(group_ids)):
-            h(7 + 2 * j)[:] = -1  # until a step is filled in, no row stores anything
+            h(7 + 3 * j)[:] = -1  # until a step is filled in, no row stores anything
+            h(8 + 3 * j)[:] = -1  # and no block table entry is written
         self.dev.copy_(self.host)
 
     def _view(self, i: int) -> torch.Tensor:
         return self.dev[self._offsets[i]: self._offsets[i] + self._sizes[i]]
 
-    def _host_view(self, i: int) -> torch.Tensor:
-        return self.host[self._offsets[i]: self._offsets[i] + self._sizes[i]]
+    def _host_view(self, i: int):
+        return self.host_np[self._offsets[i]: self._offsets[i] + self._sizes[i]]
+
+    def apply_table_updates(self) -> None:
+        """Write the step's new pages into the device block tables (part of the captured graph)."""
+        from ..ops import library as ops
+
+        for j, g in enumerate(self.group_ids):
+            ops.scatter_i32(self.storage.tables[g], self._view(8 + 3 * j), self._view(9 + 3 * j))
 
     def fill(self, layout: StepLayout, tokens: list[int]) -> None:
         """Write a decode-only step (one token per request) into the buffers."""
-        n, c, w = len(tokens), self.capacity, self.table_width
+        n = len(tokens)
         if self._event is not None:
             self._event.synchronize()  # the previous copy out of the pinned buffer has finished
         h = self._host_view
-        h(0)[:n] = torch.tensor(tokens, dtype=torch.int32)
+        h(0)[:n] = tokens
         h(0)[n:] = 0
-        h(1)[:n] = torch.tensor(layout.starts, dtype=torch.int32)
+        h(1)[:n] = layout.starts
         h(1)[n:] = 0
-        h(4)[:n] = torch.tensor(layout.starts, dtype=torch.int32) + 1
-        h(4)[n:] = 0  # dummy requests: no keys, nothing to attend to
-        h(5)[:n] = torch.tensor(layout.state_slots, dtype=torch.int32)
+        ctx = h(4)
+        ctx[:n] = layout.starts
+        ctx[:n] += 1
+        ctx[n:] = 0  # dummy requests: no keys, nothing to attend to
+        h(5)[:n] = layout.state_slots
         h(5)[n:] = 0
         for j, g in enumerate(self.group_ids):
-            h(7 + 2 * j)[:n] = torch.tensor(layout.slots[g], dtype=torch.int32)
-            h(7 + 2 * j)[n:] = -1  # dummy tokens store nothing
-            table = h(8 + 2 * j).view(c, w)
-            table.zero_()
-            for b, t in enumerate(layout.tables[g]):
-                if len(t) > w:
-                    raise ValueError(f"block table of {len(t)} pages exceeds the captured width {w}")
-                table[b, : len(t)] = torch.tensor([x if x >= 0 else 0 for x in t], dtype=torch.int32)
+            slots = h(7 + 3 * j)
+            slots[:n] = layout.slots[g]
+            slots[n:] = -1  # dummy tokens store nothing
+            index, value = _update_arrays(layout.table_updates[g], self.storage.table_width, self.storage.max_seqs)
+            k = len(index)
+            if k > self.capacity:
+                raise ValueError("more new pages than requests in a decode step")
+            ui, uv = h(8 + 3 * j), h(9 + 3 * j)
+            ui[:k] = index
+            ui[k:] = -1
+            uv[:k] = value
         self.dev.copy_(self.host, non_blocking=True)
         self._event = torch.cuda.Event()
         self._event.record(torch.cuda.current_stream(self.dev.device))

@@ -63,7 +63,7 @@ class ModelRunner:
             num_blocks = min(num_blocks, most)
         self.manager = CacheManager(groups, num_blocks, self.block_size, engine_config.max_num_seqs)
         self.storage = CacheStorage(groups, num_blocks, self.block_size, engine_config.max_num_seqs,
-                                    self.dtype, device)
+                                    self.dtype, device, table_width=-(-self.max_model_len // self.block_size))
         self._uploader = BatchUploader(device)
         self._graphs: dict[tuple[int, int], "_DecodeGraph"] = {}
         self._use_graphs = engine_config.use_graphs and model.graph_safe()
@@ -152,7 +152,7 @@ class ModelRunner:
         if self._use_graphs and all(len(e.tokens) == 1 for e in ordered):
             logits = self._replay_decode(layout, [e.tokens[0] for e in ordered], logit_rows)
         else:
-            batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader)
+            batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
             logits = self.model.forward(batch, self.storage)
         self.manager.release_passed(layout.seq_ids)
         return logits
@@ -187,14 +187,15 @@ class _DecodeGraph:
     (the reach only sets how the attention kernel spreads its work; longer contexts stay correct)."""
 
     def __init__(self, runner: ModelRunner, capacity: int, reach: int):
-        width = -(-runner.max_model_len // runner.block_size)
         group_ids = [g.group_id for g in runner.manager.paged_groups]
-        self.static = StaticDecodeBatch(capacity, width, group_ids, runner.device)
+        self.static = StaticDecodeBatch(capacity, runner.storage, group_ids, runner.device)
         batch = self.static.batch
         batch.max_context = batch.max_decode_context = reach
         # a first run outside the capture: libraries load, memory pools warm up
+        self.static.apply_table_updates()
         runner.model.forward(batch, runner.storage)
         torch.cuda.synchronize(runner.device)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
+            self.static.apply_table_updates()
             self.logits = runner.model.forward(batch, runner.storage)

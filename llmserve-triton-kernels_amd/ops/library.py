@@ -204,6 +204,19 @@ def rope_store(qkv: torch.Tensor, inv_freq: torch.Tensor | None, positions: torc
         "rope_store")
 
 
+def scatter_i32(dst: torch.Tensor, index: torch.Tensor, value: torch.Tensor) -> None:
+    """dst.flatten()[index[i]] = value[i] wherever index[i] >= 0.  The caller has checked the indices."""
+    dev = _dev(dst, index, value)
+    if dst.dtype != torch.int32 or not dst.is_contiguous():
+        raise ValueError("dst must be a contiguous int32 tensor")
+    _i32(index, "index")
+    _i32(value, "value", index.numel())
+    if index.numel() == 0:
+        return
+    _check(load("elementwise").llms_scatter_i32(_ptr(dst), _ptr(index), _ptr(value), c_int(index.numel()),
+                                                _stream(dev)), "scatter_i32")
+
+
 def silu_mul(out: torch.Tensor, gate_up: torch.Tensor) -> torch.Tensor:
     """out = silu(gate_up[:, :I]) * gate_up[:, I:]."""
     dev = _dev(out, gate_up)
@@ -309,16 +322,24 @@ def _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head
         raise ValueError("n_heads must be a multiple of n_kv_heads")
 
 
+def _table_rows(table_rows, block_tables, n_seqs: int | None):
+    if table_rows is not None:
+        _i32(table_rows, "table_rows", n_seqs)
+    return table_rows
+
+
 def attention_wave(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                    block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
                    n_heads: int, n_kv_heads: int, head_dim: int, block_size: int, window: int = 0,
-                   scale: float | None = None) -> torch.Tensor:
+                   scale: float | None = None, table_rows: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention of N new tokens over the paged cache (one wave per token and head).
 
     q: rows of width >= n_heads*head_dim (the q part of a qkv buffer is fine); out [N, n_heads*head_dim];
-    token_seq[n] = row of block_tables for token n; positions[n] = its absolute position.
+    token_seq[n] = request (0..B-1) of token n; positions[n] = its absolute position; table_rows[b] =
+    row of block_tables that request b owns (default: b).
     """
-    dev = _dev(out, q, k_pool, v_pool, block_tables, token_seq, positions)
+    dev = _dev(out, q, k_pool, v_pool, block_tables, token_seq, positions, table_rows)
+    _table_rows(table_rows, block_tables, None)
     _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
     n = q.shape[0]
     _i32(token_seq, "token_seq", n)
@@ -330,7 +351,7 @@ def attention_wave(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
     scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
     _check(load("attention").llms_attention_wave(
         c_int(_code(q)), _ptr(out), c_int(out.stride(0)), _ptr(q), c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool),
-        _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(token_seq), _ptr(positions), c_int(n),
+        _ptr(block_tables), _ptr(table_rows), c_int(block_tables.shape[1]), _ptr(token_seq), _ptr(positions), c_int(n),
         c_int(n_heads), c_int(n_kv_heads), c_int(head_dim), c_int(block_size), c_int(window), c_float(scale),
         _stream(dev)), "attention_wave")
     return out
@@ -345,19 +366,24 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
                    block_tables: torch.Tensor, cu_seqlens: torch.Tensor, context_lens: torch.Tensor,
                    seq_begin: int, n_seqs: int, max_new: int, token_begin: int, n_tokens: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, block_size: int, window: int = 0,
-                   scale: float | None = None, split_waves: bool = False, num_splits: int = 1) -> torch.Tensor:
+                   scale: float | None = None, split_waves: bool = False, num_splits: int = 1,
+                   table_rows: torch.Tensor | None = None) -> torch.Tensor:
     """bfloat16 causal attention on the matrix cores for requests [seq_begin, seq_begin + n_seqs) of a
     step, whose new tokens are rows [token_begin, token_begin + n_tokens) of q and out and bring at most
     `max_new` tokens each.  `split_waves` (with `num_splits`) spreads each request's keys over waves and
     workgroups: the arrangement for single decoded tokens."""
-    dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens)
+    dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, table_rows)
     _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
     if not attention_mfma_supported(q.dtype, head_dim, block_size):
         raise ValueError(f"attention_mfma needs bfloat16, head_dim a multiple of 16 up to 256 and block_size a "
                          f"multiple of 8; got {q.dtype}, {head_dim}, {block_size}")
-    b = block_tables.shape[0]
-    _i32(cu_seqlens, "cu_seqlens", b + 1)
+    b = cu_seqlens.numel() - 1
+    _i32(cu_seqlens, "cu_seqlens")
     _i32(context_lens, "context_lens", b)
+    if table_rows is not None:
+        _i32(table_rows, "table_rows", b)
+    elif block_tables.shape[0] < b:
+        raise ValueError("block_tables has fewer rows than there are requests")
     if not (0 <= seq_begin and n_seqs >= 0 and seq_begin + n_seqs <= b):
         raise ValueError("request range is outside the batch")
     if not (0 <= token_begin and token_begin + n_tokens <= q.shape[0]):
@@ -375,7 +401,8 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
     scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
     _check(load("attention_mfma").llms_attention_mfma(
         _ptr(out), c_int(out.stride(0)), _ptr(q), c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool),
-        _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens), c_int(seq_begin),
+        _ptr(block_tables), _ptr(table_rows), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens),
+        c_int(seq_begin),
         c_int(n_seqs), c_int(max_new), c_int(token_begin), c_int(n_tokens), c_int(n_heads), c_int(n_kv_heads),
         c_int(head_dim), c_int(block_size), c_int(window), c_float(scale), c_int(1 if split_waves else 0),
         c_int(num_splits), _ptr(ws_o), _ptr(ws_ml), _stream(dev)), "attention_mfma")

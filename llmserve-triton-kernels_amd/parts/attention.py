@@ -88,21 +88,24 @@ class Attention(Mixer):
         nh, nkv, d, bs, window = self.num_heads, self.num_kv_heads, self.head_dim, cache.block_size, self.window or 0
         if not ops.attention_mfma_supported(qkv.dtype, d, bs):
             ops.attention_wave(out, qkv, cache.k_pool, cache.v_pool, view.block_tables, batch.token_seq,
-                               batch.positions, nh, nkv, d, bs, window, self.scale)
+                               batch.positions, nh, nkv, d, bs, window, self.scale, table_rows=batch.state_slots)
             return
         common = (out, qkv, cache.k_pool, cache.v_pool, view.block_tables, batch.cu_seqlens, batch.context_lens)
         n_dec = batch.num_decode
         if n_dec:  # requests that bring one token: their keys are spread over waves and workgroups
             ops.attention_mfma(*common, 0, n_dec, 1, 0, n_dec, nh, nkv, d, bs, window, self.scale,
-                               split_waves=True, num_splits=self.decode_splits(n_dec, batch.max_decode_context))
+                               split_waves=True, num_splits=self.decode_splits(n_dec, batch.max_decode_context),
+                               table_rows=batch.state_slots)
         if n_dec < batch.num_seqs:  # portions of prompts: one wave per group of tokens and heads
             ops.attention_mfma(*common, n_dec, batch.num_seqs - n_dec, batch.max_count, n_dec,
-                               batch.num_tokens - n_dec, nh, nkv, d, bs, window, self.scale)
+                               batch.num_tokens - n_dec, nh, nkv, d, bs, window, self.scale,
+                               table_rows=batch.state_slots)
 
     def decode_splits(self, n_requests: int, max_context: int) -> int:
-        """Workgroups per (request, KV head) for decoding: enough to fill the chip when the batch is
-        small, never more than there are stretches of 128 keys."""
+        """Workgroups per (request, KV head) for decoding.  A workgroup's 4 waves take 32 keys at a time,
+        so a stretch of 128 keys per workgroup gives every wave one tile and the shortest chain of
+        dependent loads; beyond a few thousand workgroups the stretches grow instead."""
         g = self.num_heads // self.num_kv_heads
         groups = n_requests * self.num_kv_heads * -(-g // 16)
         reach = min(max_context, self.window) if self.window else max_context
-        return max(1, min(256 // groups, -(-reach // 128)))
+        return max(1, min(-(-4096 // groups), -(-reach // 128)))

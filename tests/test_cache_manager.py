@@ -59,12 +59,16 @@ def test_tables_slots_and_lengths():
     m = CacheManager(full_groups(), num_blocks=8, block_size=4, max_seqs=3)
     m.add_sequence("x")
     lay = m.append(["x"], [6])
-    table = lay.tables[0][0]
+    table = list(m.table(0, "x"))
+    row = m.slot_of["x"]
     assert len(table) == 2 and lay.starts == [0] and m.lengths["x"] == 6
     assert lay.slots[0] == [table[p // 4] * 4 + p % 4 for p in range(6)]
+    assert lay.table_updates[0] == [(row, 0, table[0]), (row, 1, table[1])]  # what the device copy is told
     lay = m.append(["x"], [3])  # crosses into a third page
-    assert lay.starts == [6] and len(lay.tables[0][0]) == 3 and lay.tables[0][0][:2] == table
-    assert m.extra_blocks_needed("x", 3) == 0 and m.extra_blocks_needed("x", 4) == 1
+    assert lay.starts == [6] and len(m.table(0, "x")) == 3 and m.table(0, "x")[:2] == table
+    assert lay.table_updates[0] == [(row, 2, m.table(0, "x")[2])]
+    assert m.append(["x"], [1]).table_updates[0] == []
+    assert m.extra_blocks_needed("x", 2) == 0 and m.extra_blocks_needed("x", 3) == 1
     with pytest.raises(ValueError):
         m.add_sequence("x")
     m.free_sequence("x")
@@ -124,8 +128,8 @@ def test_window_release_never_takes_a_reachable_key():
     m.add_sequence(0)
     length = 0
     for n in [5, 1, 1, 9, 2, 1, 1, 1, 12, 1]:
-        lay = m.append([0], [n])
-        table = lay.tables[0][0]
+        m.append([0], [n])
+        table = m.table(0, 0)
         for p in range(length, length + n):  # every key a query of this step sees must still be held
             for j in range(max(0, p - window + 1), p + 1):
                 assert table[j // bs] >= 0, (p, j)

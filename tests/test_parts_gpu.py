@@ -129,7 +129,7 @@ def attention_harness(dtype, params, lens, cuts, block_size=8, seed=10, xs=None)
     xs = [x.to(dtype) for x in xs]
     groups = group_layers([att.cache_spec()])
     manager = CacheManager(groups, num_blocks=sum(-(-n // block_size) for n in lens), block_size=block_size, max_seqs=4)
-    storage = CacheStorage(groups, manager.num_blocks, block_size, 4, dtype, DEV)
+    storage = CacheStorage(groups, manager.num_blocks, block_size, 4, dtype, DEV, table_width=16)
     storage.poison()
     uploader = BatchUploader(DEV)
     outs = [[] for _ in lens]
@@ -139,7 +139,7 @@ def attention_harness(dtype, params, lens, cuts, block_size=8, seed=10, xs=None)
     for step in cuts:  # step: {request: tokens in this step}
         ids = sorted(step, key=lambda b: step[b] != 1)
         layout = manager.append(ids, [step[b] for b in ids])
-        batch = build_batch(layout, [[0] * step[b] for b in ids], [], uploader)
+        batch = build_batch(layout, [[0] * step[b] for b in ids], [], uploader, storage)
         x = torch.cat([xs[b][done[b]: done[b] + step[b]] for b in ids]).to(DEV)
         y = att.forward(x, batch, storage.layer_cache(0)).float().cpu()
         row = 0
