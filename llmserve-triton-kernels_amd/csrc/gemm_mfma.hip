@@ -104,7 +104,11 @@ __global__ __launch_bounds__(SK_WAVES* LLMS_WAVE) void gemm_skinny_kernel(
 #define ST_KC 512
 #define ST_WAVES 4
 
-template <typename TOut>
+// SWIGLU: the 16 weight rows of a workgroup are 8 gate rows followed by the 8 up rows of the same
+// features (the feed-forward part interleaves them at load); the epilogue writes
+// bf16(bf16(silu(bf16(gate))) * bf16(up)) for those 8 features, the rounding points of the unfused path,
+// so the gated feed-forward needs no activation kernel and no [M, 2I] buffer.
+template <typename TOut, bool SWIGLU>
 __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(
     TOut* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W, const bf16* __restrict__ bias,
     int M, int N, int K, int ldx, int ldc) {
@@ -147,7 +151,24 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[(wave * LLMS_WAVE + lane) * 4 + r] = acc[r];
     __syncthreads();
-    {
+    if (SWIGLU) {
+        const int idx = threadIdx.x;  // 128 outputs: 8 features of 16 rows
+        const int j = idx % 8, m = idx / 8;
+        if (idx < 128 && m < M && n0 + j + 8 < N) {
+            float gu[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int nl = j + 8 * h;
+                const int src_lane = (nl / 4) * 16 + m, r = nl % 4;
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < ST_WAVES; ++w) s += red[(w * LLMS_WAVE + src_lane) * 4 + r];
+                gu[h] = bf16_bits_to_f32(f32_to_bf16_bits(s));
+            }
+            const float act = bf16_bits_to_f32(f32_to_bf16_bits(gu[0] / (1.f + expf(-gu[0]))));
+            store_out<TOut>(C + (size_t)m * ldc + blockIdx.x * 8 + j, act * gu[1]);
+        }
+    } else {
         const int idx = threadIdx.x;  // 256 outputs: consecutive threads take consecutive features of one row
         const int nl = idx % 16, m = idx / 16, nn = n0 + nl;
         if (m < M && nn < N) {
@@ -291,19 +312,23 @@ int llms_gemm_bf16_skinny(int out_dtype, void* C, const void* X, const void* W, 
     LLMS_LAUNCH_CHECK();
 }
 
-// M <= 16.
+// M <= 16.  swiglu = 1: W is [2I, K] with gate and up rows interleaved in runs of 8, C is [M, I]
+// = silu(gate) * up (no bias).
 int llms_gemm_bf16_stream(int out_dtype, void* C, const void* X, const void* W, const void* bias, int M, int N,
-                          int K, int ldx, int ldc, hipStream_t stream) {
-    if (int e = check_common(C, X, W, M, N, K, ldx, ldc)) return e;
+                          int K, int ldx, int ldc, int swiglu, hipStream_t stream) {
+    if (int e = check_common(C, X, W, M, N, K, ldx, swiglu ? 2 * ldc : ldc)) return e;
     LLMS_REQUIRE(M <= 16, "gemm_bf16_stream: M must be <= 16");
     LLMS_REQUIRE(out_dtype == 0 || out_dtype == 1, "gemm_bf16_stream: out_dtype must be 0 or 1");
+    LLMS_REQUIRE(!swiglu || (N % 16 == 0 && bias == nullptr && ldc >= N / 2),
+                 "gemm_bf16_stream: the gated epilogue needs N % 16 == 0, no bias and an output of N/2 columns");
     const dim3 grid((N + 15) / 16), block(ST_WAVES * LLMS_WAVE);
-    if (out_dtype == 0)
-        gemm_stream_kernel<float><<<grid, block, 0, stream>>>((float*)C, (const bf16*)X, (const bf16*)W,
-                                                              (const bf16*)bias, M, N, K, ldx, ldc);
-    else
-        gemm_stream_kernel<bf16><<<grid, block, 0, stream>>>((bf16*)C, (const bf16*)X, (const bf16*)W,
-                                                             (const bf16*)bias, M, N, K, ldx, ldc);
+#define ST_LAUNCH(TO, SI) gemm_stream_kernel<TO, SI><<<grid, block, 0, stream>>>((TO*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, ldx, ldc)
+    if (out_dtype == 0) {
+        if (swiglu) ST_LAUNCH(float, true); else ST_LAUNCH(float, false);
+    } else {
+        if (swiglu) ST_LAUNCH(bf16, true); else ST_LAUNCH(bf16, false);
+    }
+#undef ST_LAUNCH
     LLMS_LAUNCH_CHECK();
 }
 

@@ -217,18 +217,21 @@ def scatter_i32(dst: torch.Tensor, index: torch.Tensor, value: torch.Tensor) -> 
                                                 _stream(dev)), "scatter_i32")
 
 
-def silu_mul(out: torch.Tensor, gate_up: torch.Tensor) -> torch.Tensor:
-    """out = silu(gate_up[:, :I]) * gate_up[:, I:]."""
+def silu_mul(out: torch.Tensor, gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+    """out = silu(gate) * up with gate_up = [gate | up], or, `interleaved`, gate and up alternating in
+    runs of 8 columns (bfloat16, I % 8 == 0)."""
     dev = _dev(out, gate_up)
     _rows(out, "out")
     _rows(gate_up, "gate_up", 2 * out.shape[1])
     if out.shape[0] != gate_up.shape[0] or out.dtype != gate_up.dtype:
         raise ValueError("out and gate_up disagree")
+    if interleaved and (out.dtype != torch.bfloat16 or out.shape[1] % 8):
+        raise ValueError("the interleaved layout is for bfloat16 rows of I % 8 == 0")
     if out.shape[0] == 0:
         return out
     _check(load("elementwise").llms_silu_mul(
-        c_int(_code(out)), _ptr(out), _ptr(gate_up), c_int(out.shape[0]), c_int(out.shape[1]), _stream(dev)),
-        "silu_mul")
+        c_int(_code(out)), _ptr(out), _ptr(gate_up), c_int(out.shape[0]), c_int(out.shape[1]),
+        c_int(1 if interleaved else 0), _stream(dev)), "silu_mul")
     return out
 
 
@@ -266,37 +269,48 @@ def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def gemm_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
-              kernel: str | None = None) -> torch.Tensor:
+              kernel: str | None = None, swiglu: bool = False) -> torch.Tensor:
     """out[M,N] (bfloat16 or float32) = a[M,K] w[N,K]^T (+ bias) on the matrix cores, 32-bit sums.
-    `kernel`: "skinny" (M <= 64, weight streamed once) or "tile"; default by M."""
+    `kernel`: "stream" (M <= 16), "skinny" (M <= 64) or "tile"; default by M.
+    `swiglu` ("stream" only): w is [2I, K] with gate and up rows interleaved in runs of 8 and
+    out[M, I] = silu(gate) * up."""
     dev = _dev(out, a, w, bias)
     if a.dim() != 2 or a.stride(1) != 1 or out.dim() != 2 or out.stride(1) != 1:
         raise ValueError("a and out must be 2-d with unit inner stride")
     _rows(w, "w", a.shape[1])
     m, k = a.shape
     n = w.shape[0]
-    if tuple(out.shape) != (m, n):
-        raise ValueError(f"out shape {tuple(out.shape)} is not {(m, n)}")
+    if swiglu and (n % 16 or bias is not None):
+        raise ValueError("the gated epilogue needs 2I % 16 == 0 and no bias")
+    if tuple(out.shape) != (m, n // 2 if swiglu else n):
+        raise ValueError(f"out shape {tuple(out.shape)} is not {(m, n // 2 if swiglu else n)}")
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ValueError("gemm_bf16 takes bfloat16 operands")
     if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n or not bias.is_contiguous()):
         raise ValueError("bias must be a contiguous bfloat16 vector of N elements")
     if out.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("gemm_bf16 stores bfloat16 or float32")
-    if not gemm_bf16_supported(a, w):
+    if not gemm_bf16_supported(a, w) or k % 8:
         raise ValueError(f"gemm_bf16 needs K ({k}) and the row stride of a ({a.stride(0)}) to be multiples of 8 "
                          "and 16-byte aligned operands")
     if m == 0:
         return out
     kernel = kernel or ("stream" if m <= 16 else "skinny" if m <= 64 else "tile")
+    if swiglu and kernel != "stream":
+        raise ValueError("only the stream kernel has the gated epilogue")
     if kernel == "skinny" and m > 64:
         raise ValueError("the skinny kernel takes at most 64 rows")
     if kernel == "stream" and m > 16:
         raise ValueError("the stream kernel takes at most 16 rows")
     lib = load("gemm_mfma")
-    fn = {"stream": lib.llms_gemm_bf16_stream, "skinny": lib.llms_gemm_bf16_skinny, "tile": lib.llms_gemm_bf16_tile}[kernel]
-    _check(fn(c_int(_code(out)), _ptr(out), _ptr(a), _ptr(w), _ptr(bias), c_int(m), c_int(n), c_int(k),
-              c_int(a.stride(0)), c_int(out.stride(0)), _stream(dev)), f"gemm_bf16[{kernel}]")
+    args = (c_int(_code(out)), _ptr(out), _ptr(a), _ptr(w), _ptr(bias), c_int(m), c_int(n), c_int(k),
+            c_int(a.stride(0)), c_int(out.stride(0)))
+    if kernel == "stream":
+        status = lib.llms_gemm_bf16_stream(*args, c_int(1 if swiglu else 0), _stream(dev))
+    else:
+        fn = {"skinny": lib.llms_gemm_bf16_skinny, "tile": lib.llms_gemm_bf16_tile}[kernel]
+        status = fn(*args, _stream(dev))
+    _check(status, f"gemm_bf16[{kernel}]")
     return out
 
 

@@ -1,14 +1,17 @@
 """Gated feed-forward: down(silu(gate(x)) * up(x)), no biases
 (src/llmserve/model/llama.py:112-120).  Parameters: hidden, intermediate.
 gate_proj and up_proj are stacked into one [2I, H] matrix at load, so one product
-feeds the activation kernel."""
+feeds the activation.  In bfloat16 (I % 8 == 0) their rows alternate in runs of 8, so that
+the 16 weight rows a workgroup of the few-row GEMM owns are 8 features' gate and up rows
+and its epilogue can apply silu(gate) * up itself; with more rows the library's product
+writes the same interleaved layout and the activation kernel reads it."""
 
 from __future__ import annotations
 
 import torch
 
 from ..ops import library as ops
-from .linear import linear
+from .linear import LIBRARY_ABOVE_ROWS, linear
 from .registry import FeedForward, register_feed_forward
 from .spec import ParamInfo
 
@@ -30,10 +33,20 @@ class SwiGLU(FeedForward):
                 "down_proj.weight": ParamInfo((h, i))}
 
     def load(self, tensors):
-        self.gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
+        gate, up = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        self.interleaved = gate.dtype == torch.bfloat16 and self.intermediate % 8 == 0
+        if self.interleaved:
+            h = self.hidden
+            self.gate_up = torch.stack([gate.view(-1, 8, h), up.view(-1, 8, h)], dim=1).reshape(-1, h).contiguous()
+        else:
+            self.gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.down = tensors["down_proj.weight"].contiguous()
 
     def forward(self, x):
-        gate_up = linear(x, self.gate_up)
-        act = ops.silu_mul(torch.empty((x.shape[0], self.intermediate), dtype=x.dtype, device=x.device), gate_up)
+        m = x.shape[0]
+        act = torch.empty((m, self.intermediate), dtype=x.dtype, device=x.device)
+        if self.interleaved and 0 < m <= LIBRARY_ABOVE_ROWS and ops.gemm_bf16_supported(x, self.gate_up):
+            ops.gemm_bf16(act, x, self.gate_up, kernel="stream", swiglu=True)  # activation in the epilogue
+        else:
+            ops.silu_mul(act, linear(x, self.gate_up), interleaved=self.interleaved)
         return linear(act, self.down)

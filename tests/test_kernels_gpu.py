@@ -162,6 +162,23 @@ def test_gemm_bf16(kernel, m, n, k):
     assert (out.float().cpu().double() - ref).abs().max() <= 2.0 ** -8 * float(ref.abs().max())
 
 
+@pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96)])
+def test_gemm_bf16_stream_with_gated_epilogue(m, inter, k):
+    """gate_up product of the gated feed-forward with silu(gate) * up applied in the epilogue, and the
+    activation kernel on the same interleaved layout."""
+    x = rnd(m, k, seed=16).bfloat16()
+    wg, wu = rnd(inter, k, seed=17, scale=0.2).bfloat16(), rnd(inter, k, seed=18, scale=0.2).bfloat16()
+    g, u = plain_llama.linear(x, wg), plain_llama.linear(x, wu)
+    ref = (plain_llama.silu(g) * u).float()
+    w = torch.stack([wg.view(-1, 8, k), wu.view(-1, 8, k)], dim=1).reshape(-1, k).contiguous()
+    out = ops().gemm_bf16(torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV), kernel="stream",
+                          swiglu=True)
+    assert (out.float().cpu() - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
+    gu = ops().gemm_bf16(torch.empty(m, 2 * inter, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV), kernel="stream")
+    act = ops().silu_mul(torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), gu, interleaved=True)
+    assert torch.equal(act, out)  # the same rounding points fused and unfused
+
+
 def test_gemm_bf16_rows_do_not_depend_on_the_batch():
     """A row's result is the same bits whatever else is in the batch (same kernel)."""
     a, w = rnd(40, 2048, seed=14).bfloat16().to(DEV), rnd(320, 2048, seed=15).bfloat16().to(DEV)
