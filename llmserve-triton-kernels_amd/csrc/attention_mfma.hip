@@ -131,58 +131,51 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnArgs a) {
         t_end = min(n_tiles, (split + 1) * per_split);
         t_step = 4;
     }
-    // page and offset of a key; block sizes that are powers of two avoid the division
+    // The request's page ids are held in registers, 64 blocks at a time (lane l: block blk_base + l), and
+    // handed around with lane shuffles, so finding a key's page costs no memory access in the loop.
     const int bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
-    auto locate = [&](int key, int& page, int& off) {
-        int blk;
-        if (bs_shift >= 0) {
-            blk = key >> bs_shift;
-            off = key & (a.block_size - 1);
-        } else {
-            blk = key / a.block_size;
-            off = key - blk * a.block_size;
-        }
-        page = table[blk];
+    auto block_of = [&](int key) { return bs_shift >= 0 ? key >> bs_shift : key / a.block_size; };
+    const int last_blk = block_of(p_max);
+    int blk_base = 0, pages_reg = 0;
+    auto load_pages = [&](int base) {
+        blk_base = base;
+        pages_reg = table[min(base + lane, last_blk)];
     };
-    // operands of one tile of 32 keys starting at j0: key rows for the scores (rows of tile u are the
-    // keys j0 + 8*(i/4) + 4u + i%4) and, for every block of 16 dimensions, the values of the lane's 8
-    // keys j0 + 8g .. +7.  Keys outside [lo_min, p_max] may be stale or never written: they load as 0.
+    // Operands of one tile of 32 keys starting at j0: key rows for the scores (rows of tile u are the keys
+    // j0 + 8*(i/4) + 4u + i%4) and, for every block of 16 dimensions, the values of the lane's 8 keys
+    // j0 + 8g .. +7.  Every load is unconditional (addresses are clamped to the last key of the group, which
+    // exists), so the number of loads in flight is known and the arithmetic of one tile overlaps the loads of
+    // the next.  Key rows beyond p_max hold real keys whose scores the mask discards; values outside
+    // [lo_min, p_max], which may be stale or never written, are zeroed after the load.
     auto load_tile = [&](int j0, uint4 (&kf)[2][KS], uint4 (&vf)[DB]) {
+        const int blk_first = block_of(j0);
+        if (blk_first < blk_base || block_of(min(j0 + 31, p_max)) >= blk_base + LLMS_WAVE) load_pages(blk_first);
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int key = j0 + 8 * (col / 4) + 4 * u + (col % 4);  // `col` is the row index i here
-            const bool key_ok = key <= p_max;
-            const bf16* krow = nullptr;
-            if (key_ok) {
-                int page, off;
-                locate(key, page, off);
-                krow = k_base + (size_t)page * page_stride + (size_t)off * D;
-            }
+            const int key = min(j0 + 8 * (col / 4) + 4 * u + (col % 4), p_max);  // `col` is the row index i here
+            const int blk = block_of(key);
+            const int page = __shfl(pages_reg, blk - blk_base, LLMS_WAVE);
+            const bf16* krow = k_base + (size_t)page * page_stride + (size_t)(key - blk * a.block_size) * D;
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
                 const int d = 32 * s + 8 * g;
-                kf[u][s] = (key_ok && d < D) ? *reinterpret_cast<const uint4*>(krow + d) : zero;
+                kf[u][s] = *reinterpret_cast<const uint4*>(krow + (d < D ? d : 0));
             }
         }
-        const int jk = j0 + 8 * g;
-        const bool chunk_ok = jk <= p_max;
-        const bf16* vrow = nullptr;
-        if (chunk_ok) {
-            int page, off;
-            locate(jk, page, off);
-            vrow = v_base + (size_t)page * page_stride + off;
-        }
-        const int first = lo_min - jk, last = p_max + 1 - jk;
+        const int jk = min(j0 + 8 * g, p_max & ~7);
+        const int blk = block_of(jk);
+        const int page = __shfl(pages_reg, blk - blk_base, LLMS_WAVE);
+        const bf16* vrow = v_base + (size_t)page * page_stride + (jk - blk * a.block_size);
 #pragma unroll
-        for (int m = 0; m < DB; ++m) {
-            const uint4 v = chunk_ok ? *reinterpret_cast<const uint4*>(vrow + (size_t)(16 * m + col) * a.block_size) : zero;
-            vf[m] = keep_elements(v, first, last);
-        }
+        for (int m = 0; m < DB; ++m) vf[m] = *reinterpret_cast<const uint4*>(vrow + (size_t)(16 * m + col) * a.block_size);
     };
 
     // the next tile's operands are requested before this tile's arithmetic starts
     uint4 kf_next[2][KS], vf_next[DB];
-    if (t_begin < t_end) load_tile(j_begin + 32 * t_begin, kf_next, vf_next);
+    if (t_begin < t_end) {
+        load_pages(block_of(j_begin + 32 * t_begin));
+        load_tile(j_begin + 32 * t_begin, kf_next, vf_next);
+    }
     for (int t = t_begin; t < t_end; t += t_step) {
         const int j0 = j_begin + 32 * t;
         uint4 kf[2][KS], vf[DB];
@@ -198,10 +191,17 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnArgs a) {
         for (int u = 0; u < 2; ++u) {
             s_acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < KS; ++s)
+            for (int s = 0; s < KS; ++s) {
+                // (queries beyond head_dim are zero, so a key chunk loaded from a clamped address adds nothing)
                 s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u][s]), as_bf16x8(qf[s]), s_acc[u], 0, 0, 0);
+            }
         }
         const int jk = j0 + 8 * g;
+        {
+            const int first = lo_min - jk, last = p_max + 1 - jk;
+#pragma unroll
+            for (int m = 0; m < DB; ++m) vf[m] = keep_elements(vf[m], first, last);
+        }
         // ---- online softmax of this lane's column over its 8 keys (and the 3 other lane groups)
         float sc[8];
         float tmax = -INFINITY;

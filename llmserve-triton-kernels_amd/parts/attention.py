@@ -102,10 +102,11 @@ class Attention(Mixer):
                                table_rows=batch.state_slots)
 
     def decode_splits(self, n_requests: int, max_context: int) -> int:
-        """Workgroups per (request, KV head) for decoding.  A workgroup's 4 waves take 32 keys at a time,
-        so a stretch of 128 keys per workgroup gives every wave one tile and the shortest chain of
-        dependent loads; beyond a few thousand workgroups the stretches grow instead."""
+        """Workgroups per (request, KV head) for decoding.  A workgroup's 4 waves take 32 keys at a time
+        each; a small batch is spread over more workgroups, down to stretches of 128 keys (one tile per
+        wave, the shortest chain of dependent steps), whose partial results a second kernel merges; once
+        the batch alone fills the chip (256 workgroups) nothing is split."""
         g = self.num_heads // self.num_kv_heads
         groups = n_requests * self.num_kv_heads * -(-g // 16)
         reach = min(max_context, self.window) if self.window else max_context
-        return max(1, min(-(-4096 // groups), -(-reach // 128)))
+        return max(1, min(256 // groups, -(-reach // 128)))
