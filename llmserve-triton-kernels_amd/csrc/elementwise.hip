@@ -194,17 +194,16 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gate_
     out[idx] = from_f32<T>(s * u);
 }
 
-// bfloat16 rows of inter % 8 == 0: 8 elements per thread, 16-byte loads and stores.  interleaved: the row
-// is [gate 0..7 | up 0..7 | gate 8..15 | up 8..15 | ...] instead of [gate | up].
+// bfloat16 rows of inter % 8 == 0: 8 elements per thread, 16-byte loads and stores.
 __global__ void silu_mul_bf16_vec_kernel(bf16* __restrict__ out, const bf16* __restrict__ gate_up, int inter,
-                                         size_t total_chunks, int interleaved) {
+                                         size_t total_chunks) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total_chunks) return;
     const int cpr = inter / 8;  // chunks per row
     const size_t n = idx / cpr;
     const int c = (int)(idx % cpr);
     const uint4* row = reinterpret_cast<const uint4*>(gate_up + n * 2 * (size_t)inter);
-    const uint4 gv = interleaved ? row[2 * c] : row[c], uv = interleaved ? row[2 * c + 1] : row[cpr + c];
+    const uint4 gv = row[c], uv = row[cpr + c];
     const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
     uint32_t ow[4];
 #pragma unroll
@@ -292,16 +291,13 @@ int llms_scatter_i32(int* dst, const int* index, const int* value, int n, hipStr
     LLMS_LAUNCH_CHECK();
 }
 
-int llms_silu_mul(int dtype, void* out, const void* gate_up, int n_rows, int inter, int interleaved,
-                  hipStream_t stream) {
+int llms_silu_mul(int dtype, void* out, const void* gate_up, int n_rows, int inter, hipStream_t stream) {
     LLMS_REQUIRE(n_rows > 0 && inter > 0, "silu_mul: sizes must be positive");
-    LLMS_REQUIRE(!interleaved || (dtype == 1 && inter % 8 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)gate_up % 16) == 0),
-                 "silu_mul: the interleaved layout is for bfloat16 rows of inter % 8 == 0");
     const size_t total = (size_t)n_rows * inter;
     if (dtype == 1 && inter % 8 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)gate_up % 16) == 0) {
         const size_t chunks = total / 8;
         silu_mul_bf16_vec_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, stream>>>((bf16*)out, (const bf16*)gate_up,
-                                                                                         inter, chunks, interleaved);
+                                                                                         inter, chunks);
         LLMS_LAUNCH_CHECK();
     }
     const unsigned blocks = (unsigned)((total + 255) / 256);

@@ -3,10 +3,11 @@
 // along K, which is how the matrix instructions want them: a lane holds 8 consecutive k of
 // one row (one 16-byte load).
 //
-//   gemm_skinny  M <= 64 (decoding): the weight is read once, straight from global memory into
-//                the matrix instruction; a workgroup owns 16 output features and its 8 waves
-//                split K; their partial sums meet in LDS in a fixed order.
-//   gemm_tile    any M (prompts): 128x128 tiles through double-buffered LDS, 4 waves of 64x64.
+//   gemm_skinny  M <= 64: the weight is read once, straight from global memory into the matrix
+//                instruction; a workgroup owns 16 output features and its 8 waves split K; their
+//                partial sums meet in LDS in a fixed order.
+//   gemm_tile    any M: 128x128 tiles through double-buffered LDS, 4 waves of 64x64.
+// (The product for up to 16 rows, with its fused prologue and epilogues, is gemm_stream.hip.)
 //
 // K must be a multiple of 8 and rows 16-byte aligned (the host checks); M, N are arbitrary.
 #include "common.h"
@@ -15,14 +16,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
-
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
-
-// 16-byte load that is not kept in the caches: weights are read once per step.
-__device__ __forceinline__ uint4 load_streaming(const void* p) {
-    return __builtin_bit_cast(uint4, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
-}
 
 template <typename TOut>
 __device__ __forceinline__ void store_out(TOut* p, float v);
@@ -92,93 +86,6 @@ __global__ __launch_bounds__(SK_WAVES* LLMS_WAVE) void gemm_skinny_kernel(
         for (int w = 0; w < SK_WAVES; ++w) s += red[w][mb][src_lane][r];
         if (bias) s += bf16_bits_to_f32(bias[nn].bits);
         store_out<TOut>(C + (size_t)m * ldc + nn, s);
-    }
-}
-
-// ------------------------------------------------------------------------------ streaming
-// M <= 16.  The weight is read with fully coalesced loads: one load instruction of a wave covers 1 KB
-// of one weight row (512 k), 16 such loads (16 rows) are in flight per wave before anything waits.
-// The 16 KB go through a wave-private, XOR-swizzled LDS tile to reach the layout the matrix
-// instruction wants.  A workgroup owns 16 output features; its 4 waves take the K chunks in turn and
-// add their partial sums in LDS in a fixed order.
-#define ST_KC 512
-#define ST_WAVES 4
-
-// SWIGLU: the 16 weight rows of a workgroup are 8 gate rows followed by the 8 up rows of the same
-// features (the feed-forward part interleaves them at load); the epilogue writes
-// bf16(bf16(silu(bf16(gate))) * bf16(up)) for those 8 features, the rounding points of the unfused path,
-// so the gated feed-forward needs no activation kernel and no [M, 2I] buffer.
-template <typename TOut, bool SWIGLU>
-__global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(
-    TOut* __restrict__ C, const bf16* __restrict__ X, const bf16* __restrict__ W, const bf16* __restrict__ bias,
-    int M, int N, int K, int ldx, int ldc) {
-    __shared__ uint4 lds[ST_WAVES * 16 * (ST_KC / 8)];  // 64 KB: per wave 16 rows x 64 chunks of 16 bytes
-    const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
-    const int r16 = lane % 16, g = lane / 16;
-    const int n0 = blockIdx.x * 16;
-    uint4* tile = lds + wave * 16 * (ST_KC / 8);
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-    f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
-    const int chunks = (K + ST_KC - 1) / ST_KC;
-    const bool m_ok = r16 < M;
-    const bf16* xrow = X + (size_t)(m_ok ? r16 : 0) * ldx;
-
-    for (int c = wave; c < chunks; c += ST_WAVES) {
-        const int k0 = c * ST_KC;
-        uint4 wreg[16];
-        const int kl = k0 + 8 * lane;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int n = n0 + i;
-            wreg[i] = (n < N && kl < K) ? load_streaming(W + (size_t)n * K + kl) : zero;
-        }
-        uint4 xreg[16];
-#pragma unroll
-        for (int s = 0; s < 16; ++s) {
-            const int k = k0 + 32 * s + 8 * g;
-            xreg[s] = (m_ok && k < K) ? *reinterpret_cast<const uint4*>(xrow + k) : zero;
-        }
-#pragma unroll
-        for (int i = 0; i < 16; ++i) tile[i * (ST_KC / 8) + (lane ^ i)] = wreg[i];
-#pragma unroll
-        for (int s = 0; s < 16; ++s) {
-            const uint4 a = tile[r16 * (ST_KC / 8) + ((4 * s + g) ^ r16)];
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(xreg[s]), acc, 0, 0, 0);
-        }
-    }
-    __syncthreads();  // every wave is done with its tile; the memory now carries the partial sums
-    float* red = reinterpret_cast<float*>(lds);  // [wave][lane][4]
-#pragma unroll
-    for (int r = 0; r < 4; ++r) red[(wave * LLMS_WAVE + lane) * 4 + r] = acc[r];
-    __syncthreads();
-    if (SWIGLU) {
-        const int idx = threadIdx.x;  // 128 outputs: 8 features of 16 rows
-        const int j = idx % 8, m = idx / 8;
-        if (idx < 128 && m < M && n0 + j + 8 < N) {
-            float gu[2];
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int nl = j + 8 * h;
-                const int src_lane = (nl / 4) * 16 + m, r = nl % 4;
-                float s = 0.f;
-#pragma unroll
-                for (int w = 0; w < ST_WAVES; ++w) s += red[(w * LLMS_WAVE + src_lane) * 4 + r];
-                gu[h] = bf16_bits_to_f32(f32_to_bf16_bits(s));
-            }
-            const float act = bf16_bits_to_f32(f32_to_bf16_bits(gu[0] / (1.f + expf(-gu[0]))));
-            store_out<TOut>(C + (size_t)m * ldc + blockIdx.x * 8 + j, act * gu[1]);
-        }
-    } else {
-        const int idx = threadIdx.x;  // 256 outputs: consecutive threads take consecutive features of one row
-        const int nl = idx % 16, m = idx / 16, nn = n0 + nl;
-        if (m < M && nn < N) {
-            const int src_lane = (nl / 4) * 16 + m, r = nl % 4;
-            float s = 0.f;
-#pragma unroll
-            for (int w = 0; w < ST_WAVES; ++w) s += red[(w * LLMS_WAVE + src_lane) * 4 + r];
-            if (bias) s += bf16_bits_to_f32(bias[nn].bits);
-            store_out<TOut>(C + (size_t)m * ldc + nn, s);
-        }
     }
 }
 
@@ -309,26 +216,6 @@ int llms_gemm_bf16_skinny(int out_dtype, void* C, const void* X, const void* W, 
         launch_skinny<float>((float*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, ldx, ldc, stream);
     else
         launch_skinny<bf16>((bf16*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, ldx, ldc, stream);
-    LLMS_LAUNCH_CHECK();
-}
-
-// M <= 16.  swiglu = 1: W is [2I, K] with gate and up rows interleaved in runs of 8, C is [M, I]
-// = silu(gate) * up (no bias).
-int llms_gemm_bf16_stream(int out_dtype, void* C, const void* X, const void* W, const void* bias, int M, int N,
-                          int K, int ldx, int ldc, int swiglu, hipStream_t stream) {
-    if (int e = check_common(C, X, W, M, N, K, ldx, swiglu ? 2 * ldc : ldc)) return e;
-    LLMS_REQUIRE(M <= 16, "gemm_bf16_stream: M must be <= 16");
-    LLMS_REQUIRE(out_dtype == 0 || out_dtype == 1, "gemm_bf16_stream: out_dtype must be 0 or 1");
-    LLMS_REQUIRE(!swiglu || (N % 16 == 0 && bias == nullptr && ldc >= N / 2),
-                 "gemm_bf16_stream: the gated epilogue needs N % 16 == 0, no bias and an output of N/2 columns");
-    const dim3 grid((N + 15) / 16), block(ST_WAVES * LLMS_WAVE);
-#define ST_LAUNCH(TO, SI) gemm_stream_kernel<TO, SI><<<grid, block, 0, stream>>>((TO*)C, (const bf16*)X, (const bf16*)W, (const bf16*)bias, M, N, K, ldx, ldc)
-    if (out_dtype == 0) {
-        if (swiglu) ST_LAUNCH(float, true); else ST_LAUNCH(float, false);
-    } else {
-        if (swiglu) ST_LAUNCH(bf16, true); else ST_LAUNCH(bf16, false);
-    }
-#undef ST_LAUNCH
     LLMS_LAUNCH_CHECK();
 }
 

@@ -1,0 +1,350 @@
+// bfloat16 matrix product for few rows (M <= 16, decoding):  C[M,N] = X[M,K] * W[N,K]^T, 32-bit sums on
+// the gfx950 matrix cores, built around reading the weight once at memory speed.
+//
+// A workgroup owns 16 weight rows; its 4 waves take the K chunks (512 wide) in turn.  One load instruction
+// of a wave covers 1 KB of one weight row (fully coalesced, non-temporal), 16 such loads are in flight per
+// wave before anything waits, and the next chunk's loads are issued before the arithmetic of this one.
+// The 16 KB go through a wave-private, XOR-swizzled LDS tile to reach the layout of
+// v_mfma_f32_16x16x32_bf16 (lane l: A[i = l%16][k = 8*(l/16) .. +7], here i = weight row; B likewise
+// with j = row m of X; D[i = 4*(l/16) + r][j = l%16]).  The waves' partial sums meet in LDS in a fixed order.
+//
+// Because a launch costs more than most of these products take, what surrounds the product is fused in:
+//   NORM      prologue: x = bf16(residual + delta) (written to resid_out by workgroup 0), then
+//             h = weight_n * bf16(x * rsqrt(mean(x^2) + eps)): the RMSNorm kernel's rounding points
+//             (src/llmserve/model/llama.py:24-28).  Each workgroup computes the row statistics itself.
+//   SWIGLU    the 16 rows are 8 gate rows and the 8 up rows of the same features; the epilogue writes
+//             bf16(bf16(silu(bf16(gate))) * bf16(up)) (src/llmserve/model/llama.py:120).
+//   ROPE_QKV  the 16 rows are 8 rows of one head and their 8 rotary partners (i, i + D/2); the epilogue
+//             rotates q and k (src/llmserve/model/llama.py:31-54), writes q, and stores k and v at the
+//             tokens' slots of the paged cache (values transposed inside a page).
+// Which weight rows a workgroup takes is only an index map, so the weights keep their stacked layout
+// ([q; k; v], [gate; up]) and the same tensors serve the library product used for more rows.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// 16-byte load that is not kept in the caches: weights are read once per step.
+__device__ __forceinline__ uint4 load_streaming(const void* p) {
+    return __builtin_bit_cast(uint4, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
+}
+
+__device__ __forceinline__ float bfr(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+template <typename TOut>
+__device__ __forceinline__ void store_out(TOut* p, float v);
+template <>
+__device__ __forceinline__ void store_out<float>(float* p, float v) { *p = v; }
+template <>
+__device__ __forceinline__ void store_out<bf16>(bf16* p, float v) { p->bits = f32_to_bf16_bits(v); }
+
+#define ST_KC 512
+#define ST_WAVES 4
+#define EPI_PLAIN 0
+#define EPI_SWIGLU 1
+#define EPI_ROPE_QKV 2
+
+struct StreamArgs {
+    void* C;
+    int ldc;
+    const bf16* X;
+    int ldx;
+    const bf16* W;
+    const bf16* bias;
+    int M, N, K;
+    // NORM
+    const bf16* delta;
+    const bf16* norm_w;
+    float eps;
+    bf16* resid_out;
+    // SWIGLU
+    int inter;
+    // ROPE_QKV
+    int n_heads, n_kv_heads, head_dim, block_size;
+    const float* inv_freq;
+    const int* positions;
+    const int* slots;
+    bf16* k_pool;
+    bf16* v_pool;
+};
+
+// 8 packed bfloat16 -> floats
+__device__ __forceinline__ void unpack8(uint4 v, float (&f)[8]) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        f[2 * j] = bf16_bits_to_f32((uint16_t)(w[j] & 0xffffu));
+        f[2 * j + 1] = bf16_bits_to_f32((uint16_t)(w[j] >> 16));
+    }
+}
+
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = (uint32_t)f32_to_bf16_bits(f[2 * j]) | ((uint32_t)f32_to_bf16_bits(f[2 * j + 1]) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+template <typename TOut, int EPI, bool NORM>
+__global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const StreamArgs a) {
+    __shared__ uint4 lds[ST_WAVES * 16 * (ST_KC / 8)];  // 64 KB: per wave 16 rows x 64 chunks of 16 bytes
+    const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
+    const int r16 = lane % 16, g = lane / 16;
+    const int tile_id = blockIdx.x;
+    const int M = a.M, N = a.N, K = a.K;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+
+    // ---- which 16 weight rows this workgroup owns (-1: none)
+    const int D = a.head_dim;
+    int rot_tiles = 0, spt = 1;
+    if (EPI == EPI_ROPE_QKV) {
+        spt = D / 16;
+        rot_tiles = (a.n_heads + a.n_kv_heads) * spt;
+    }
+    auto weight_row = [&](int i) -> int {
+        if (EPI == EPI_SWIGLU) {
+            const int f = tile_id * 8 + (i & 7);
+            return f < a.inter ? (i < 8 ? f : a.inter + f) : -1;
+        } else if (EPI == EPI_ROPE_QKV) {
+            if (tile_id < rot_tiles) {
+                const int h = tile_id / spt, s = tile_id % spt;
+                return h * D + 8 * s + (i & 7) + (i < 8 ? 0 : D / 2);
+            }
+            return (a.n_heads + a.n_kv_heads) * D + (tile_id - rot_tiles) * 16 + i;
+        } else {
+            const int n = tile_id * 16 + i;
+            return n < N ? n : -1;
+        }
+    };
+
+    uint4* tile = lds + wave * 16 * (ST_KC / 8);
+    const int chunks = (K + ST_KC - 1) / ST_KC;
+    uint4 wreg[16];
+    auto load_weights = [&](int c) {
+        const int kl = c * ST_KC + 8 * lane;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int n = weight_row(i);
+            wreg[i] = (n >= 0 && kl < K) ? load_streaming(a.W + (size_t)n * K + kl) : zero;
+        }
+    };
+    if (wave < chunks) load_weights(wave);  // in flight while the row statistics are computed
+
+    const bool m_ok = r16 < M;
+    const bf16* xrow = a.X + (size_t)(m_ok ? r16 : 0) * a.ldx;
+    const bf16* drow = (NORM && a.delta) ? a.delta + (size_t)(m_ok ? r16 : 0) * a.ldx : nullptr;
+    // x chunk of 8 at column k of this lane's row: the residual sum in 32-bit, rounded once
+    auto load_x = [&](int k) -> uint4 {
+        uint4 v = *reinterpret_cast<const uint4*>(xrow + k);
+        if (NORM && drow) {
+            float xf[8], df[8];
+            unpack8(v, xf);
+            unpack8(*reinterpret_cast<const uint4*>(drow + k), df);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xf[e] += df[e];
+            v = pack8(xf);
+        }
+        return v;
+    };
+
+    float inv_rms = 0.f;
+    if (NORM) {
+        float ss = 0.f;
+        for (int c = wave; c < chunks; c += ST_WAVES) {
+#pragma unroll 4
+            for (int s = 0; s < 16; ++s) {
+                const int k = c * ST_KC + 32 * s + 8 * g;
+                if (m_ok && k < K) {
+                    const uint4 v = load_x(k);
+                    float xf[8];
+                    unpack8(v, xf);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) ss += xf[e] * xf[e];
+                    if (a.resid_out && tile_id == 0) *reinterpret_cast<uint4*>(a.resid_out + (size_t)r16 * a.ldx + k) = v;
+                }
+            }
+        }
+        ss += __shfl_xor(ss, 16, LLMS_WAVE);
+        ss += __shfl_xor(ss, 32, LLMS_WAVE);
+        float* ss_lds = reinterpret_cast<float*>(lds);  // [wave][16]; the tiles are not in use yet
+        if (g == 0) ss_lds[wave * 16 + r16] = ss;
+        __syncthreads();
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < ST_WAVES; ++w) total += ss_lds[w * 16 + r16];
+        inv_rms = rsqrtf(total / (float)K + a.eps);
+        __syncthreads();  // all have read the sums before wave 0's tile overwrites them
+    }
+
+    f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int c = wave; c < chunks; c += ST_WAVES) {
+        const int k0 = c * ST_KC;
+        uint4 xreg[16];
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+            const int k = k0 + 32 * s + 8 * g;
+            if (m_ok && k < K) {
+                uint4 v = load_x(k);
+                if (NORM) {
+                    float xf[8], wf[8];
+                    unpack8(v, xf);
+                    unpack8(*reinterpret_cast<const uint4*>(a.norm_w + k), wf);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) xf[e] = wf[e] * bfr(xf[e] * inv_rms);
+                    v = pack8(xf);
+                }
+                xreg[s] = v;
+            } else {
+                xreg[s] = zero;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) tile[i * (ST_KC / 8) + (lane ^ i)] = wreg[i];
+        if (c + ST_WAVES < chunks) load_weights(c + ST_WAVES);  // the registers are free again
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+            const uint4 av = tile[r16 * (ST_KC / 8) + ((4 * s + g) ^ r16)];
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av), as_bf16x8(xreg[s]), acc, 0, 0, 0);
+        }
+    }
+    __syncthreads();  // every wave is done with its tile; the memory now carries the partial sums
+    float* red = reinterpret_cast<float*>(lds);  // [wave][lane][4]; acc[r] = D[row 4g + r][m = r16]
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[(wave * LLMS_WAVE + lane) * 4 + r] = acc[r];
+    __syncthreads();
+    // sum of the 4 waves for weight row i (0..15) of this tile and row m of X, wave 0 first
+    auto total_of = [&](int i, int m) -> float {
+        const int src_lane = (i / 4) * 16 + m, r = i % 4;
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < ST_WAVES; ++w) s += red[(w * LLMS_WAVE + src_lane) * 4 + r];
+        return s;
+    };
+    const int idx = threadIdx.x;
+    TOut* C = reinterpret_cast<TOut*>(a.C);
+
+    if (EPI == EPI_PLAIN) {
+        const int i = idx % 16, m = idx / 16, n = tile_id * 16 + i;  // consecutive threads: consecutive features
+        if (m < M && n < N) {
+            float s = total_of(i, m);
+            if (a.bias) s += bf16_bits_to_f32(a.bias[n].bits);
+            store_out<TOut>(C + (size_t)m * a.ldc + n, s);
+        }
+    } else if (EPI == EPI_SWIGLU) {
+        const int j = idx % 8, m = idx / 8, f = tile_id * 8 + j;
+        if (idx < 128 && m < M && f < a.inter) {
+            const float gate = bfr(total_of(j, m)), up = bfr(total_of(j + 8, m));
+            store_out<TOut>(C + (size_t)m * a.ldc + f, bfr(gate / (1.f + expf(-gate))) * up);
+        }
+    } else {
+        const int nh = a.n_heads, nkv = a.n_kv_heads, bs = a.block_size;
+        if (tile_id < rot_tiles) {
+            const int j = idx % 8, m = idx / 8;
+            if (idx < 128 && m < M) {
+                const int h = tile_id / spt, s = tile_id % spt, d = 8 * s + j;
+                float lo = total_of(j, m), hi = total_of(j + 8, m);
+                if (a.bias) {
+                    lo += bf16_bits_to_f32(a.bias[h * D + d].bits);
+                    hi += bf16_bits_to_f32(a.bias[h * D + d + D / 2].bits);
+                }
+                lo = bfr(lo);  // the projection's result is bfloat16 before it is rotated
+                hi = bfr(hi);
+                float ra = lo, rb = hi;
+                if (a.inv_freq) {
+                    float sn, cs;
+                    sincosf((float)a.positions[m] * a.inv_freq[d], &sn, &cs);
+                    ra = lo * cs - hi * sn;
+                    rb = hi * cs + lo * sn;
+                }
+                if (h < nh) {
+                    store_out<TOut>(C + (size_t)m * a.ldc + h * D + d, ra);
+                    store_out<TOut>(C + (size_t)m * a.ldc + h * D + d + D / 2, rb);
+                } else {
+                    const int slot = a.slots ? a.slots[m] : -1;
+                    if (slot >= 0) {
+                        const int page = slot / bs, off = slot % bs;
+                        bf16* dst = a.k_pool + (((size_t)page * nkv + (h - nh)) * bs + off) * D;
+                        dst[d].bits = f32_to_bf16_bits(ra);
+                        dst[d + D / 2].bits = f32_to_bf16_bits(rb);
+                    }
+                }
+            }
+        } else {
+            const int i = idx % 16, m = idx / 16;
+            const int slot = (a.slots && m < M) ? a.slots[m] : -1;
+            if (m < M && slot >= 0) {
+                const int f = (tile_id - rot_tiles) * 16 + i;  // feature among the value heads
+                float v = total_of(i, m);
+                if (a.bias) v += bf16_bits_to_f32(a.bias[(nh + nkv) * D + f].bits);
+                const int kvh = f / D, d = f % D, page = slot / bs, off = slot % bs;
+                a.v_pool[(((size_t)page * nkv + kvh) * D + d) * bs + off].bits = f32_to_bf16_bits(v);
+            }
+        }
+    }
+}
+
+template <typename TOut, int EPI>
+static void launch_stream(bool norm, unsigned grid, const StreamArgs& a, hipStream_t stream) {
+    if (norm)
+        gemm_stream_kernel<TOut, EPI, true><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(a);
+    else
+        gemm_stream_kernel<TOut, EPI, false><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(a);
+}
+
+extern "C" {
+
+// epilogue: 0 plain (C [M,N] + bias), 1 gated (W = [gate; up] of `inter` rows each, C [M, inter]),
+// 2 rotary q/k/v (W = [q; k; v], C = q [M, n_heads*head_dim], k and v stored at `slots` when given).
+// norm_w != null: X is the residual stream, `delta` (nullable) is added to it, the sum goes to resid_out
+// (nullable) and its RMSNorm with norm_w and eps is what is multiplied.  out_dtype: 0 float32, 1 bfloat16.
+int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* X, int ldx, const void* W,
+                     const void* bias, int M, int N, int K, const void* delta, const void* norm_w, float eps,
+                     void* resid_out, int inter, int n_heads, int n_kv_heads, int head_dim, int block_size,
+                     const float* inv_freq, const int* positions, const int* slots, void* k_pool, void* v_pool,
+                     hipStream_t stream) {
+    LLMS_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_stream: needs 1 <= M <= 16 and positive sizes");
+    LLMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "gemm_stream: K and the row stride of X must be multiples of 8");
+    LLMS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_stream: X and W must be 16-byte aligned");
+    LLMS_REQUIRE(C != nullptr && (out_dtype == 0 || out_dtype == 1), "gemm_stream: bad output");
+    LLMS_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_stream: epilogue must be 0, 1 or 2");
+    if (norm_w) {
+        LLMS_REQUIRE(((uintptr_t)norm_w % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0) &&
+                         (!resid_out || ((uintptr_t)resid_out % 16) == 0), "gemm_stream: norm operands must be 16-byte aligned");
+        LLMS_REQUIRE(resid_out != X, "gemm_stream: the summed residual needs a buffer of its own");
+    } else {
+        LLMS_REQUIRE(!delta && !resid_out, "gemm_stream: delta and resid_out need norm_w");
+    }
+    StreamArgs a = {C, ldc, (const bf16*)X, ldx, (const bf16*)W, (const bf16*)bias, M, N, K, (const bf16*)delta,
+                    (const bf16*)norm_w, eps, (bf16*)resid_out, inter, n_heads, n_kv_heads, head_dim, block_size,
+                    inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool};
+    unsigned grid;
+    if (epilogue == EPI_PLAIN) {
+        LLMS_REQUIRE(ldc >= N, "gemm_stream: ldc too small");
+        grid = (N + 15) / 16;
+    } else if (epilogue == EPI_SWIGLU) {
+        LLMS_REQUIRE(inter > 0 && inter % 8 == 0 && N == 2 * inter && bias == nullptr && ldc >= inter,
+                     "gemm_stream: the gated epilogue needs N = 2*inter, inter % 8 == 0, no bias");
+        grid = inter / 8;
+    } else {
+        LLMS_REQUIRE(n_heads > 0 && n_kv_heads > 0 && head_dim >= 16 && head_dim % 16 == 0 &&
+                         N == (n_heads + 2 * n_kv_heads) * head_dim && ldc >= n_heads * head_dim,
+                     "gemm_stream: the rotary epilogue needs head_dim % 16 == 0 and N = (heads + 2 kv heads) * head_dim");
+        LLMS_REQUIRE(positions != nullptr || inv_freq == nullptr, "gemm_stream: rotation needs positions");
+        LLMS_REQUIRE(slots == nullptr || (k_pool && v_pool && block_size > 0), "gemm_stream: slots given without pools");
+        grid = (n_heads + n_kv_heads) * (head_dim / 16) + n_kv_heads * head_dim / 16;
+    }
+    const bool norm = norm_w != nullptr;
+#define ST_EPI(E)                                                                  \
+    if (out_dtype == 0) launch_stream<float, E>(norm, grid, a, stream);           \
+    else launch_stream<bf16, E>(norm, grid, a, stream);
+    if (epilogue == EPI_PLAIN) { ST_EPI(EPI_PLAIN) }
+    else if (epilogue == EPI_SWIGLU) { ST_EPI(EPI_SWIGLU) }
+    else { ST_EPI(EPI_ROPE_QKV) }
+#undef ST_EPI
+    LLMS_LAUNCH_CHECK();
+}
+
+}  // extern "C"

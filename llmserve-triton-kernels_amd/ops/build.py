@@ -37,7 +37,7 @@ HIPCC_FLAGS = [
 # built when something is first sampled).
 GROUPS = {
     "float32": ("elementwise", "gemm", "attention"),
-    "bfloat16": ("elementwise", "gemm", "attention", "gemm_mfma", "attention_mfma"),
+    "bfloat16": ("elementwise", "gemm", "attention", "gemm_stream", "attention_mfma"),
 }
 
 

@@ -217,21 +217,18 @@ def scatter_i32(dst: torch.Tensor, index: torch.Tensor, value: torch.Tensor) -> 
                                                 _stream(dev)), "scatter_i32")
 
 
-def silu_mul(out: torch.Tensor, gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
-    """out = silu(gate) * up with gate_up = [gate | up], or, `interleaved`, gate and up alternating in
-    runs of 8 columns (bfloat16, I % 8 == 0)."""
+def silu_mul(out: torch.Tensor, gate_up: torch.Tensor) -> torch.Tensor:
+    """out = silu(gate_up[:, :I]) * gate_up[:, I:]."""
     dev = _dev(out, gate_up)
     _rows(out, "out")
     _rows(gate_up, "gate_up", 2 * out.shape[1])
     if out.shape[0] != gate_up.shape[0] or out.dtype != gate_up.dtype:
         raise ValueError("out and gate_up disagree")
-    if interleaved and (out.dtype != torch.bfloat16 or out.shape[1] % 8):
-        raise ValueError("the interleaved layout is for bfloat16 rows of I % 8 == 0")
     if out.shape[0] == 0:
         return out
     _check(load("elementwise").llms_silu_mul(
-        c_int(_code(out)), _ptr(out), _ptr(gate_up), c_int(out.shape[0]), c_int(out.shape[1]),
-        c_int(1 if interleaved else 0), _stream(dev)), "silu_mul")
+        c_int(_code(out)), _ptr(out), _ptr(gate_up), c_int(out.shape[0]), c_int(out.shape[1]), _stream(dev)),
+        "silu_mul")
     return out
 
 
@@ -269,48 +266,113 @@ def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def gemm_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
-              kernel: str | None = None, swiglu: bool = False) -> torch.Tensor:
+              kernel: str | None = None) -> torch.Tensor:
     """out[M,N] (bfloat16 or float32) = a[M,K] w[N,K]^T (+ bias) on the matrix cores, 32-bit sums.
-    `kernel`: "stream" (M <= 16), "skinny" (M <= 64) or "tile"; default by M.
-    `swiglu` ("stream" only): w is [2I, K] with gate and up rows interleaved in runs of 8 and
-    out[M, I] = silu(gate) * up."""
+    `kernel`: "stream" (M <= 16), "skinny" (M <= 64) or "tile"; default by M."""
     dev = _dev(out, a, w, bias)
     if a.dim() != 2 or a.stride(1) != 1 or out.dim() != 2 or out.stride(1) != 1:
         raise ValueError("a and out must be 2-d with unit inner stride")
     _rows(w, "w", a.shape[1])
     m, k = a.shape
     n = w.shape[0]
-    if swiglu and (n % 16 or bias is not None):
-        raise ValueError("the gated epilogue needs 2I % 16 == 0 and no bias")
-    if tuple(out.shape) != (m, n // 2 if swiglu else n):
-        raise ValueError(f"out shape {tuple(out.shape)} is not {(m, n // 2 if swiglu else n)}")
+    if tuple(out.shape) != (m, n):
+        raise ValueError(f"out shape {tuple(out.shape)} is not {(m, n)}")
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ValueError("gemm_bf16 takes bfloat16 operands")
     if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n or not bias.is_contiguous()):
         raise ValueError("bias must be a contiguous bfloat16 vector of N elements")
     if out.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("gemm_bf16 stores bfloat16 or float32")
-    if not gemm_bf16_supported(a, w) or k % 8:
+    if not gemm_bf16_supported(a, w):
         raise ValueError(f"gemm_bf16 needs K ({k}) and the row stride of a ({a.stride(0)}) to be multiples of 8 "
                          "and 16-byte aligned operands")
     if m == 0:
         return out
     kernel = kernel or ("stream" if m <= 16 else "skinny" if m <= 64 else "tile")
-    if swiglu and kernel != "stream":
-        raise ValueError("only the stream kernel has the gated epilogue")
+    if kernel == "stream":
+        return gemm_stream(out, a, w, bias)
     if kernel == "skinny" and m > 64:
         raise ValueError("the skinny kernel takes at most 64 rows")
-    if kernel == "stream" and m > 16:
-        raise ValueError("the stream kernel takes at most 16 rows")
     lib = load("gemm_mfma")
-    args = (c_int(_code(out)), _ptr(out), _ptr(a), _ptr(w), _ptr(bias), c_int(m), c_int(n), c_int(k),
-            c_int(a.stride(0)), c_int(out.stride(0)))
-    if kernel == "stream":
-        status = lib.llms_gemm_bf16_stream(*args, c_int(1 if swiglu else 0), _stream(dev))
-    else:
-        fn = {"skinny": lib.llms_gemm_bf16_skinny, "tile": lib.llms_gemm_bf16_tile}[kernel]
-        status = fn(*args, _stream(dev))
-    _check(status, f"gemm_bf16[{kernel}]")
+    fn = {"skinny": lib.llms_gemm_bf16_skinny, "tile": lib.llms_gemm_bf16_tile}[kernel]
+    _check(fn(c_int(_code(out)), _ptr(out), _ptr(a), _ptr(w), _ptr(bias), c_int(m), c_int(n), c_int(k),
+              c_int(a.stride(0)), c_int(out.stride(0)), _stream(dev)), f"gemm_bf16[{kernel}]")
+    return out
+
+
+def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, *,
+                norm: tuple | None = None, swiglu: bool = False, rope: dict | None = None) -> torch.Tensor:
+    """The product for up to 16 bfloat16 rows, with what surrounds it fused in.
+
+    plain:   out[M, N] = x w^T (+ bias).
+    norm = (delta | None, norm_weight, eps, resid_out | None): x is the residual stream; delta is added
+             to it (32-bit sum, rounded once), the sum is written to resid_out, and the product runs on the
+             RMSNorm of the sum.
+    swiglu:  w = [gate; up] ([2I, K]); out[M, I] = silu(gate) * up.
+    rope = dict(n_heads, n_kv_heads, head_dim, inv_freq | None, positions, slots | None, k_pool, v_pool,
+             block_size): w = [q; k; v]; out[M, n_heads * head_dim] = rotated q; rotated k and v are stored at
+             the tokens' cache slots."""
+    dev = _dev(out, x, w, bias)
+    if x.dim() != 2 or x.stride(1) != 1 or out.dim() != 2 or out.stride(1) != 1:
+        raise ValueError("x and out must be 2-d with unit inner stride")
+    _rows(w, "w", x.shape[1])
+    m, k = x.shape
+    n = w.shape[0]
+    if not 0 < m <= 16:
+        raise ValueError("gemm_stream takes 1..16 rows")
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or out.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("gemm_stream takes bfloat16 operands and stores bfloat16 or float32")
+    if not gemm_bf16_supported(x, w):
+        raise ValueError(f"gemm_stream needs K ({k}) and the row stride of x ({x.stride(0)}) to be multiples of 8 "
+                         "and 16-byte aligned operands")
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous bfloat16 vector of N elements")
+    if swiglu and rope is not None:
+        raise ValueError("one epilogue at a time")
+    delta = norm_w = resid_out = None
+    eps = 0.0
+    if norm is not None:
+        delta, norm_w, eps, resid_out = norm
+        for name, t in (("delta", delta), ("resid_out", resid_out)):
+            if t is not None and (t.shape != x.shape or t.dtype != x.dtype or t.stride() != x.stride()):
+                raise ValueError(f"{name} must match x in shape, dtype and strides")
+        if resid_out is not None and resid_out.data_ptr() == x.data_ptr():
+            raise ValueError("the summed residual needs a buffer of its own")
+        if norm_w.dtype != torch.bfloat16 or norm_w.numel() != k or not norm_w.is_contiguous():
+            raise ValueError(f"norm weight must be a contiguous bfloat16 vector of {k} elements")
+        _dev(delta, norm_w, resid_out, x)
+    epilogue, inter, cols = 0, 0, n
+    r = dict(n_heads=0, n_kv_heads=0, head_dim=0, block_size=0, inv_freq=None, positions=None, slots=None,
+             k_pool=None, v_pool=None)
+    if swiglu:
+        if n % 16 or bias is not None:
+            raise ValueError("the gated epilogue needs 2I % 16 == 0 and no bias")
+        epilogue, inter, cols = 1, n // 2, n // 2
+    elif rope is not None:
+        r.update(rope)
+        nh, nkv, d = r["n_heads"], r["n_kv_heads"], r["head_dim"]
+        if d % 16 or n != (nh + 2 * nkv) * d:
+            raise ValueError("the rotary epilogue needs head_dim % 16 == 0 and N = (heads + 2 kv heads) * head_dim")
+        _i32(r["positions"], "positions", m)
+        if r["inv_freq"] is not None:
+            _f32(r["inv_freq"], "inv_freq", d // 2)
+        if r["slots"] is not None:
+            _i32(r["slots"], "slots", m)
+            bs, kp, vp = r["block_size"], r["k_pool"], r["v_pool"]
+            pages = kp.shape[0]
+            if (tuple(kp.shape) != (pages, nkv, bs, d) or tuple(vp.shape) != (pages, nkv, d, bs)
+                    or not kp.is_contiguous() or not vp.is_contiguous() or kp.dtype != x.dtype or vp.dtype != x.dtype):
+                raise ValueError("pools do not have the cache layout [pages, kv, block, D] / [pages, kv, D, block]")
+        _dev(x, r["inv_freq"], r["positions"], r["slots"], r["k_pool"], r["v_pool"])
+        epilogue, cols = 2, nh * d
+    if tuple(out.shape) != (m, cols):
+        raise ValueError(f"out shape {tuple(out.shape)} is not {(m, cols)}")
+    _check(load("gemm_stream").llms_gemm_stream(
+        c_int(_code(out)), c_int(epilogue), _ptr(out), c_int(out.stride(0)), _ptr(x), c_int(x.stride(0)), _ptr(w),
+        _ptr(bias), c_int(m), c_int(n), c_int(k), _ptr(delta), _ptr(norm_w), c_float(eps), _ptr(resid_out),
+        c_int(inter), c_int(r["n_heads"]), c_int(r["n_kv_heads"]), c_int(r["head_dim"]), c_int(r["block_size"]),
+        _ptr(r["inv_freq"]), _ptr(r["positions"]), _ptr(r["slots"]), _ptr(r["k_pool"]), _ptr(r["v_pool"]),
+        _stream(dev)), "gemm_stream")
     return out
 
 

@@ -16,14 +16,16 @@ import math
 import torch
 
 from ..ops import library as ops
-from .linear import linear
-from .registry import POSITION_ENCODINGS, Mixer, register_mixer
+from .linear import FUSE_NORM_INTO_PRODUCT, LIBRARY_ABOVE_ROWS, linear
+from .registry import POSITION_ENCODINGS, DeferredNorm, Mixer, register_mixer
+from .rmsnorm import RMSNorm
 from .spec import PagedCacheSpec, ParamInfo
 
 
 @register_mixer("attention")
 class Attention(Mixer):
     graph_safe = True
+    accepts_deferred_norm = True
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
@@ -68,19 +70,55 @@ class Attention(Mixer):
     def forward(self, x, batch, cache):
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         view = batch.groups[cache.group_id]
-        qkv = linear(x, self.qkv_weight, self.qkv_bias)
         slots = view.slots if cache.store else None
-        fused = getattr(self.position, "rotate_and_store", None)
-        if fused is not None:
-            fused(qkv, batch.positions, slots, cache.k_pool, cache.v_pool, nh, nkv, d, cache.block_size)
-        else:
-            self.position.rotate(qkv, batch.positions, nh, nkv, d)
-            if slots is not None:
-                ops.rope_store(qkv, None, batch.positions, slots, cache.k_pool, cache.v_pool, nh, nkv, d,
-                               cache.block_size)
-        out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
-        self.attend(out, qkv, cache, view, batch)
+        q = self.project_few_rows(x, batch, cache, slots)
+        if q is None:
+            if isinstance(x, DeferredNorm):
+                x = x.materialize()
+            q = linear(x, self.qkv_weight, self.qkv_bias)  # q, k and v side by side; q is read in place
+            fused = getattr(self.position, "rotate_and_store", None)
+            if fused is not None:
+                fused(q, batch.positions, slots, cache.k_pool, cache.v_pool, nh, nkv, d, cache.block_size)
+            else:
+                self.position.rotate(q, batch.positions, nh, nkv, d)
+                if slots is not None:
+                    ops.rope_store(q, None, batch.positions, slots, cache.k_pool, cache.v_pool, nh, nkv, d,
+                                   cache.block_size)
+        out = torch.empty((q.shape[0], nh * d), dtype=q.dtype, device=q.device)
+        self.attend(out, q, cache, view, batch)
         return linear(out, self.o_weight)
+
+    def _few_rows_unfit(self, rows) -> bool:
+        m = rows.shape[0]
+        return (rows.dtype != torch.bfloat16 or not 0 < m <= LIBRARY_ABOVE_ROWS or self.head_dim % 16 != 0
+                or not ops.gemm_bf16_supported(rows, self.qkv_weight))
+
+    def project_few_rows(self, x, batch, cache, slots):
+        """With up to 16 bfloat16 rows one kernel does the residual sum, the norm, the projection, the
+        rotation and the cache store (ops.gemm_stream); returns the rotated queries, or None when that
+        kernel does not apply."""
+        if isinstance(x, DeferredNorm) and not FUSE_NORM_INTO_PRODUCT:
+            return None if self._few_rows_unfit(x.residual) else self.project_few_rows(x.materialize(), batch, cache, slots)
+        deferred = isinstance(x, DeferredNorm)
+        rows = x.residual if deferred else x
+        m = rows.shape[0]
+        if self._few_rows_unfit(rows) or (deferred and not isinstance(x.norm, RMSNorm)):
+            return None
+        frequencies = getattr(self.position, "rotary_frequencies", None)
+        if frequencies is None and not getattr(self.position, "identity", False):
+            return None  # a position encoding this kernel does not know
+        rope = dict(n_heads=self.num_heads, n_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
+                    inv_freq=frequencies() if frequencies is not None else None, positions=batch.positions,
+                    slots=slots, k_pool=cache.k_pool, v_pool=cache.v_pool, block_size=cache.block_size)
+        q = torch.empty((m, self.num_heads * self.head_dim), dtype=rows.dtype, device=rows.device)
+        if deferred:
+            new_residual = torch.empty_like(rows) if x.delta is not None else None
+            ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias,
+                            norm=(x.delta, x.norm.weight, x.norm.eps, new_residual), rope=rope)
+            x.resolve(new_residual)
+        else:
+            ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias, rope=rope)
+        return q
 
     def attend(self, out, qkv, cache, view, batch):
         """out[n] = attention of token n's query heads (the first nh*D columns of qkv) over its

@@ -8,13 +8,18 @@ sum is done, in 32-bit, by the norm kernel that needs its result.
 
 from __future__ import annotations
 
-from .registry import Block, register_block
+from .registry import Block, DeferredNorm, register_block
 
 
 @register_block("prenorm")
 class PreNormBlock(Block):
     def forward(self, x, delta, batch, cache):
-        h = self.mixer_norm.add_norm(x, delta)  # x += delta, h = norm(x)
-        a = self.mixer.forward(h, batch, cache)
-        h = self.feed_forward_norm.add_norm(x, a)  # x += a, h = norm(x)
-        return x, self.feed_forward.forward(h)
+        h = DeferredNorm(self.mixer_norm, x, delta)  # x + delta, normed: by the norm's kernel or by the mixer's
+        a = self.mixer.forward(h if self.mixer.accepts_deferred_norm else h.materialize(), batch, cache)
+        if not h.resolved:
+            raise RuntimeError(f"{type(self.mixer).__name__} took a deferred input and left it unresolved")
+        h2 = DeferredNorm(self.feed_forward_norm, h.residual, a)
+        f = self.feed_forward.forward(h2 if self.feed_forward.accepts_deferred_norm else h2.materialize())
+        if not h2.resolved:
+            raise RuntimeError(f"{type(self.feed_forward).__name__} took a deferred input and left it unresolved")
+        return h2.residual, f

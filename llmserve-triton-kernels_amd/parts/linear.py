@@ -17,6 +17,11 @@ from ..ops import library as ops
 
 
 LIBRARY_ABOVE_ROWS = 16
+# Whether the few-row product also does the residual sum and the norm in front of it
+# (ops.gemm_stream(norm=...)).  Off: every workgroup repeats the statistics and the rounding of its
+# rows with most lanes idle, which measured slower (TinyLlama shape, batch 1: 2.7 ms against
+# 1.4 ms a step) than the norm as a kernel of its own.
+FUSE_NORM_INTO_PRODUCT = False
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,

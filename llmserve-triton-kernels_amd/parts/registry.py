@@ -16,6 +16,9 @@ Interfaces (x is always the flat batch of new tokens, [N, hidden], in the model 
                     forward(x, batch, cache) -> y
   FeedForward       forward(x) -> y
   Block             forward(x, delta, batch, cache) -> (x, delta)   hidden state is x + delta
+
+A mixer or feed-forward that sets `accepts_deferred_norm` is handed a `DeferredNorm` instead of the
+normed tensor and may fold the residual sum and the norm into its own first kernel.
 """
 
 from __future__ import annotations
@@ -72,6 +75,39 @@ class Norm(Part):
         return self.forward(picked)
 
 
+class DeferredNorm:
+    """The input of a mixer or feed-forward before it is computed: norm(residual + delta).
+
+    The consumer either calls `materialize()` (the norm's own kernel: residual += delta in place, returns
+    the normed tensor) or computes the same thing inside a kernel of its own and reports the summed
+    residual with `resolve(new_residual)`.  Afterwards `residual` is the summed residual stream."""
+
+    def __init__(self, norm: "Norm", residual: torch.Tensor, delta: torch.Tensor | None):
+        self.norm = norm
+        self.residual = residual
+        self.delta = delta
+        self.resolved = False
+
+    @property
+    def num_rows(self) -> int:
+        return self.residual.shape[0]
+
+    def materialize(self) -> torch.Tensor:
+        if self.resolved:
+            raise RuntimeError("this input was already consumed")
+        self.resolved = True
+        return self.norm.add_norm(self.residual, self.delta)
+
+    def resolve(self, new_residual: torch.Tensor | None) -> None:
+        """The consumer has summed and normed by itself; `new_residual` holds residual + delta
+        (None: there was no delta, the residual is unchanged)."""
+        if self.resolved:
+            raise RuntimeError("this input was already consumed")
+        self.resolved = True
+        if new_residual is not None:
+            self.residual = new_residual
+
+
 class PositionEncoding(Part):
     def rotate(self, qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv_heads: int,
                head_dim: int) -> None:
@@ -79,6 +115,8 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    accepts_deferred_norm = False
+
     def cache_spec(self) -> PagedCacheSpec | StateCacheSpec | None:
         return None
 
@@ -87,6 +125,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    accepts_deferred_norm = False
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 

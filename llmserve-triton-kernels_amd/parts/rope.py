@@ -34,6 +34,11 @@ class RotaryEncoding(PositionEncoding):
     def load(self, tensors):
         self.inv_freq = self.frequencies().to(self.ctx.device)
 
+    def rotary_frequencies(self):
+        """float32 [head_dim / 2] on the device: the encoding is x' = x cos + rotate_half(x) sin with angle
+        position * frequency, which lets a mixer fold the rotation into a kernel of its own."""
+        return self.inv_freq
+
     def rotate(self, qkv, positions, n_heads, n_kv_heads, head_dim):
         ops.rope_store(qkv, self.inv_freq, positions, None, None, None, n_heads, n_kv_heads, head_dim, 1)
 
@@ -45,6 +50,8 @@ class RotaryEncoding(PositionEncoding):
 @register_position_encoding("none")
 class NoPositionEncoding(PositionEncoding):
     """Keys and queries are used as projected."""
+
+    identity = True
     graph_safe = True
 
 

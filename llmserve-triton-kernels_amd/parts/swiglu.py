@@ -1,24 +1,25 @@
 """Gated feed-forward: down(silu(gate(x)) * up(x)), no biases
 (src/llmserve/model/llama.py:112-120).  Parameters: hidden, intermediate.
-gate_proj and up_proj are stacked into one [2I, H] matrix at load, so one product
-feeds the activation.  In bfloat16 (I % 8 == 0) their rows alternate in runs of 8, so that
-the 16 weight rows a workgroup of the few-row GEMM owns are 8 features' gate and up rows
-and its epilogue can apply silu(gate) * up itself; with more rows the library's product
-writes the same interleaved layout and the activation kernel reads it."""
+gate_proj and up_proj are stacked into one [2I, H] matrix at load, so one product feeds
+the activation.  With few bfloat16 rows that product also does the residual sum and the
+norm before it and the activation after it (ops.gemm_stream); otherwise the norm, the
+product and the activation are kernels of their own."""
 
 from __future__ import annotations
 
 import torch
 
 from ..ops import library as ops
-from .linear import LIBRARY_ABOVE_ROWS, linear
-from .registry import FeedForward, register_feed_forward
+from .linear import FUSE_NORM_INTO_PRODUCT, LIBRARY_ABOVE_ROWS, linear
+from .registry import DeferredNorm, FeedForward, register_feed_forward
+from .rmsnorm import RMSNorm
 from .spec import ParamInfo
 
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
     graph_safe = True
+    accepts_deferred_norm = True
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
@@ -33,20 +34,26 @@ class SwiGLU(FeedForward):
                 "down_proj.weight": ParamInfo((h, i))}
 
     def load(self, tensors):
-        gate, up = tensors["gate_proj.weight"], tensors["up_proj.weight"]
-        self.interleaved = gate.dtype == torch.bfloat16 and self.intermediate % 8 == 0
-        if self.interleaved:
-            h = self.hidden
-            self.gate_up = torch.stack([gate.view(-1, 8, h), up.view(-1, 8, h)], dim=1).reshape(-1, h).contiguous()
-        else:
-            self.gate_up = torch.cat([gate, up], dim=0).contiguous()
+        self.gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
         self.down = tensors["down_proj.weight"].contiguous()
 
     def forward(self, x):
-        m = x.shape[0]
-        act = torch.empty((m, self.intermediate), dtype=x.dtype, device=x.device)
-        if self.interleaved and 0 < m <= LIBRARY_ABOVE_ROWS and ops.gemm_bf16_supported(x, self.gate_up):
-            ops.gemm_bf16(act, x, self.gate_up, kernel="stream", swiglu=True)  # activation in the epilogue
+        m = x.num_rows if isinstance(x, DeferredNorm) else x.shape[0]
+        dtype, device = self.gate_up.dtype, self.gate_up.device
+        act = torch.empty((m, self.intermediate), dtype=dtype, device=device)
+        few = dtype == torch.bfloat16 and 0 < m <= LIBRARY_ABOVE_ROWS and self.intermediate % 8 == 0
+        if isinstance(x, DeferredNorm):
+            norm = x.norm
+            if (FUSE_NORM_INTO_PRODUCT and few and isinstance(norm, RMSNorm)
+                    and ops.gemm_bf16_supported(x.residual, self.gate_up)):
+                new_residual = torch.empty_like(x.residual) if x.delta is not None else None
+                ops.gemm_stream(act, x.residual, self.gate_up, norm=(x.delta, norm.weight, norm.eps, new_residual),
+                                swiglu=True)
+                x.resolve(new_residual)
+                return linear(act, self.down)
+            x = x.materialize()
+        if few and ops.gemm_bf16_supported(x, self.gate_up):
+            ops.gemm_stream(act, x, self.gate_up, swiglu=True)  # activation in the product's epilogue
         else:
-            ops.silu_mul(act, linear(x, self.gate_up), interleaved=self.interleaved)
+            ops.silu_mul(act, linear(x, self.gate_up))
         return linear(act, self.down)

@@ -162,21 +162,79 @@ def test_gemm_bf16(kernel, m, n, k):
     assert (out.float().cpu().double() - ref).abs().max() <= 2.0 ** -8 * float(ref.abs().max())
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 16, 64), (3, 333, 96), (16, 2056, 2048), (7, 100, 5632), (9, 48, 176)])
+def test_gemm_stream_plain(m, n, k):
+    x, w, b = rnd(m, k, seed=11).bfloat16(), rnd(n, k, seed=12).bfloat16(), rnd(n, seed=13).bfloat16()
+    ref = x.double() @ w.double().t() + b.double()
+    out = ops().gemm_stream(torch.empty(m, n, device=DEV), x.to(DEV), w.to(DEV), b.to(DEV))
+    assert (out.cpu().double() - ref).abs().max() <= 2e-6 * math.sqrt(k) * float(ref.abs().max())
+
+
 @pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96)])
-def test_gemm_bf16_stream_with_gated_epilogue(m, inter, k):
-    """gate_up product of the gated feed-forward with silu(gate) * up applied in the epilogue, and the
-    activation kernel on the same interleaved layout."""
+def test_gemm_stream_gated_epilogue(m, inter, k):
+    """gate and up of the feed-forward in one product over [gate; up], silu(gate) * up in the epilogue:
+    the same bits as the product followed by the activation kernel."""
     x = rnd(m, k, seed=16).bfloat16()
-    wg, wu = rnd(inter, k, seed=17, scale=0.2).bfloat16(), rnd(inter, k, seed=18, scale=0.2).bfloat16()
-    g, u = plain_llama.linear(x, wg), plain_llama.linear(x, wu)
+    w = torch.cat([rnd(inter, k, seed=17, scale=0.2), rnd(inter, k, seed=18, scale=0.2)]).bfloat16()
+    g, u = plain_llama.linear(x, w[:inter]), plain_llama.linear(x, w[inter:])
     ref = (plain_llama.silu(g) * u).float()
-    w = torch.stack([wg.view(-1, 8, k), wu.view(-1, 8, k)], dim=1).reshape(-1, k).contiguous()
-    out = ops().gemm_bf16(torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV), kernel="stream",
-                          swiglu=True)
+    out = ops().gemm_stream(torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV), swiglu=True)
     assert (out.float().cpu() - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
-    gu = ops().gemm_bf16(torch.empty(m, 2 * inter, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV), kernel="stream")
-    act = ops().silu_mul(torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), gu, interleaved=True)
-    assert torch.equal(act, out)  # the same rounding points fused and unfused
+    gu = ops().gemm_stream(torch.empty(m, 2 * inter, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV))
+    act = ops().silu_mul(torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), gu)
+    assert torch.equal(act, out)
+
+
+@pytest.mark.parametrize("m,n,k,eps", [(1, 64, 64, 1e-5), (6, 320, 2048, 1e-6), (16, 100, 4096 + 96, 1e-5)])
+@pytest.mark.parametrize("with_delta", [False, True])
+def test_gemm_stream_norm_prologue(m, n, k, eps, with_delta):
+    """Residual sum and RMSNorm inside the product: the same bits of the summed residual as the norm
+    kernel writes, and a product that agrees with norm kernel + product."""
+    resid, delta = rnd(m, k, seed=19, scale=2.0).bfloat16(), rnd(m, k, seed=20).bfloat16()
+    wn, w = (1 + 0.1 * rnd(k, seed=21)).bfloat16(), rnd(n, k, seed=22).bfloat16()
+    summed = (resid.float() + delta.float()).bfloat16() if with_delta else resid
+    ref = plain_llama.rms_norm(summed, wn, eps).double() @ w.double().t()
+    new_resid = torch.full((m, k), 7.0, dtype=torch.bfloat16, device=DEV) if with_delta else None
+    out = ops().gemm_stream(torch.empty(m, n, device=DEV), resid.to(DEV), w.to(DEV),
+                            norm=(delta.to(DEV) if with_delta else None, wn.to(DEV), eps, new_resid))
+    # the statistics are summed in another order than on the CPU, so a normed element may round the other way
+    assert (out.cpu().double() - ref).abs().max() <= 2.0 ** -8 * float(ref.abs().max())
+    if with_delta:
+        assert torch.equal(new_resid.cpu(), summed)
+    with pytest.raises(ValueError, match="buffer of its own"):
+        r = resid.to(DEV)
+        ops().gemm_stream(torch.empty(m, n, device=DEV), r, w.to(DEV), norm=(delta.to(DEV), wn.to(DEV), eps, r))
+
+
+@pytest.mark.parametrize("nh,nkv,d,bs,theta,bias", [(4, 2, 16, 16, 1e4, False), (3, 1, 32, 8, 5e5, True),
+                                                    (8, 2, 64, 16, 1e4, False), (2, 2, 48, 8, None, True)])
+def test_gemm_stream_rotary_epilogue(nh, nkv, d, bs, theta, bias):
+    """q/k/v projection with the rotation and the cache store in the epilogue: the same bits as the
+    projection followed by the rotation kernel."""
+    m, k, pages = 5, 96, 6
+    n = (nh + 2 * nkv) * d
+    x, w = rnd(m, k, seed=23).bfloat16().to(DEV), rnd(n, k, seed=24, scale=0.3).bfloat16().to(DEV)
+    b = rnd(n, seed=25).bfloat16().to(DEV) if bias else None
+    positions = torch.tensor([0, 1, 77, 500, 4095], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([3, bs * pages - 1, -1, 0, bs * 2 + 1], dtype=torch.int32, device=DEV)
+    inv_freq = (1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV) if theta else None
+    pools = lambda: (torch.full((pages, nkv, bs, d), 7.0, dtype=torch.bfloat16, device=DEV),  # noqa: E731
+                     torch.full((pages, nkv, d, bs), 7.0, dtype=torch.bfloat16, device=DEV))
+    k1, v1 = pools()
+    qkv = ops().gemm_stream(torch.empty(m, n, dtype=torch.bfloat16, device=DEV), x, w, b)
+    ops().rope_store(qkv, inv_freq, positions, slots, k1, v1, nh, nkv, d, bs)
+    k2, v2 = pools()
+    q = ops().gemm_stream(torch.empty(m, nh * d, dtype=torch.bfloat16, device=DEV), x, w, b,
+                          rope=dict(n_heads=nh, n_kv_heads=nkv, head_dim=d, inv_freq=inv_freq, positions=positions,
+                                    slots=slots, k_pool=k2, v_pool=v2, block_size=bs))
+    assert torch.equal(q, qkv[:, : nh * d]) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert (k2 != 7).any() and (v2 != 7).any()
+    # without slots only q is produced
+    k3, v3 = pools()
+    q3 = ops().gemm_stream(torch.empty(m, nh * d, dtype=torch.bfloat16, device=DEV), x, w, b,
+                           rope=dict(n_heads=nh, n_kv_heads=nkv, head_dim=d, inv_freq=inv_freq, positions=positions,
+                                     slots=None, k_pool=k3, v_pool=v3, block_size=bs))
+    assert torch.equal(q3, q) and (k3 == 7).all() and (v3 == 7).all()
 
 
 def test_gemm_bf16_rows_do_not_depend_on_the_batch():
@@ -185,6 +243,9 @@ def test_gemm_bf16_rows_do_not_depend_on_the_batch():
     full = ops().gemm_bf16(torch.empty(40, 320, device=DEV), a, w, kernel="skinny")
     one = ops().gemm_bf16(torch.empty(1, 320, device=DEV), a[17:18].contiguous(), w, kernel="skinny")
     assert torch.equal(full[17], one[0])
+    full = ops().gemm_stream(torch.empty(16, 320, device=DEV), a[:16].contiguous(), w)
+    one = ops().gemm_stream(torch.empty(1, 320, device=DEV), a[9:10].contiguous(), w)
+    assert torch.equal(full[9], one[0])
 
 
 def test_gemm_bf16_refuses_what_it_cannot_take():
