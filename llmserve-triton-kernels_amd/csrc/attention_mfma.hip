@@ -28,7 +28,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+    return pack_bf16x2(lo, hi);
 }
 
 // Keep elements [first, last) of 8 packed bfloat16, zero the rest.

@@ -96,7 +96,7 @@ __global__ void rmsnorm_bf16_vec_kernel(bf16* __restrict__ out, const bf16* x, c
                 v[c][2 * j] = lo;
                 v[c][2 * j + 1] = hi;
                 ss += lo * lo + hi * hi;
-                ow[j] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+                ow[j] = pack_bf16x2(lo, hi);
             }
             if (rs) rs[i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
         }
@@ -116,7 +116,7 @@ __global__ void rmsnorm_bf16_vec_kernel(bf16* __restrict__ out, const bf16* x, c
             for (int j = 0; j < 4; ++j) {
                 const float lo = bf16_bits_to_f32((uint16_t)(ww[j] & 0xffffu)) * round_to<bf16>(v[c][2 * j] * inv);
                 const float hi = bf16_bits_to_f32((uint16_t)(ww[j] >> 16)) * round_to<bf16>(v[c][2 * j + 1] * inv);
-                ow[j] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+                ow[j] = pack_bf16x2(lo, hi);
             }
             o[i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
         }
@@ -215,7 +215,7 @@ __global__ void silu_mul_bf16_vec_kernel(bf16* __restrict__ out, const bf16* __r
             const float u = bf16_bits_to_f32((uint16_t)(h ? uw[j] >> 16 : uw[j] & 0xffffu));
             r2[h] = round_to<bf16>(g / (1.f + expf(-g))) * u;
         }
-        ow[j] = (uint32_t)f32_to_bf16_bits(r2[0]) | ((uint32_t)f32_to_bf16_bits(r2[1]) << 16);
+        ow[j] = pack_bf16x2(r2[0], r2[1]);
     }
     reinterpret_cast<uint4*>(out)[idx] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }

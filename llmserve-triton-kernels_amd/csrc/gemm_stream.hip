@@ -84,7 +84,7 @@ __device__ __forceinline__ void unpack8(uint4 v, float (&f)[8]) {
 __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
     uint32_t w[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) w[j] = (uint32_t)f32_to_bf16_bits(f[2 * j]) | ((uint32_t)f32_to_bf16_bits(f[2 * j + 1]) << 16);
+    for (int j = 0; j < 4; ++j) w[j] = pack_bf16x2(f[2 * j], f[2 * j + 1]);
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
