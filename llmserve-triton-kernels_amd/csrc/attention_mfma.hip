@@ -15,7 +15,7 @@
 //
 // Two arrangements of the 4 waves of a workgroup:
 //   SPLIT_WAVES = false (prompts): 4 consecutive column groups of one request.
-//   SPLIT_WAVES = true  (decoding): one column group; the key tiles are dealt to the 4 waves, and
+//   SPLIT_WAVES = true  (decoding): one column group; the key tiles are dealt to the 4 or 8 waves, and
 //     optionally to `num_splits` workgroups whose partial results a second kernel merges.
 // All merges run in a fixed order, so a token's result does not depend on the batch around it.
 //
@@ -64,7 +64,7 @@ struct AttnArgs {
 };
 
 template <int DB, bool SPLIT_WAVES>
-__global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(SPLIT_WAVES ? 512 : 256) void attn_mfma_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
     constexpr int KS = (D + 31) / 32;  // k-steps of the score product
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnArgs a) {
         const int per_split = (n_tiles + a.num_splits - 1) / a.num_splits;
         t_begin = split * per_split + wave;
         t_end = min(n_tiles, (split + 1) * per_split);
-        t_step = 4;
+        t_step = blockDim.x / LLMS_WAVE;  // 4 or 8 waves share the keys
     }
     // The request's page ids are held in registers, 64 blocks at a time (lane l: block blk_base + l), and
     // handed around with lane shuffles, so finding a key's page costs no memory access in the loop.
@@ -253,10 +253,10 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const AttnArgs a) {
         return;
     }
 
-    // ---- the 4 waves' partial results meet in LDS, wave 0 first, then 1, 2, 3
+    // ---- the waves' partial results meet in LDS, wave 0 first, then 1, 2, ...
     __shared__ float sh_acc[DB][LLMS_WAVE][4];
     __shared__ float sh_m[16], sh_l[16];
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < (int)(blockDim.x / LLMS_WAVE); ++w) {
         if (wave == w) {
             if (w == 0) {
 #pragma unroll
@@ -336,10 +336,10 @@ __global__ void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const 
 }
 
 template <bool SPLIT_WAVES>
-static int launch_attn(int db, dim3 grid, const AttnArgs& a, hipStream_t stream) {
+static int launch_attn(int db, dim3 grid, int threads, const AttnArgs& a, hipStream_t stream) {
 #define ATT_CASE(N)                                                          \
     case N:                                                                  \
-        attn_mfma_kernel<N, SPLIT_WAVES><<<grid, 256, 0, stream>>>(a);       \
+        attn_mfma_kernel<N, SPLIT_WAVES><<<grid, threads, 0, stream>>>(a);   \
         break;
     switch (db) {
         ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
@@ -354,15 +354,15 @@ static int launch_attn(int db, dim3 grid, const AttnArgs& a, hipStream_t stream)
 extern "C" {
 
 // Attention for the requests [seq_begin, seq_begin + n_seqs) of a step.  max_new: most new tokens any of
-// them brings.  split_waves = 1 deals the keys of each column group to 4 waves and `num_splits`
-// workgroups (decoding); with num_splits > 1 the caller provides ws_o [tokens * heads * splits * D] and
+// them brings.  split_waves = 1 deals the keys of each column group to `waves` (4 or 8) waves and
+// `num_splits` workgroups (decoding); with num_splits > 1 the caller provides ws_o [tokens * heads * splits * D] and
 // ws_ml [tokens * heads * splits * 2] floats, indexed by absolute token row.
 int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
                         const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
                         const int* cu_seqlens,
                         const int* context_lens, int seq_begin, int n_seqs, int max_new, int token_begin,
                         int n_tokens, int n_heads, int n_kv_heads, int head_dim, int block_size, int window,
-                        float scale, int split_waves, int num_splits, float* ws_o, float* ws_ml,
+                        float scale, int split_waves, int num_splits, int waves, float* ws_o, float* ws_ml,
                         hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && n_heads > 0 && n_kv_heads > 0, "attention_mfma: sizes must be positive");
     LLMS_REQUIRE(n_heads % n_kv_heads == 0, "attention_mfma: n_heads must be a multiple of n_kv_heads");
@@ -373,6 +373,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                      ((uintptr_t)out % 8) == 0, "attention_mfma: pointers must be 16-byte aligned");
     LLMS_REQUIRE(window >= 0 && max_blocks > 0, "attention_mfma: bad window or max_blocks");
     LLMS_REQUIRE(num_splits >= 1, "attention_mfma: num_splits must be >= 1");
+    LLMS_REQUIRE(waves == 4 || (split_waves && waves == 8), "attention_mfma: 4 waves, or 8 when the waves share the keys");
     LLMS_REQUIRE(split_waves || num_splits == 1, "attention_mfma: splits need split_waves");
     LLMS_REQUIRE(num_splits == 1 || (ws_o && ws_ml), "attention_mfma: splits need a workspace");
     LLMS_REQUIRE(n_seqs <= 65535, "attention_mfma: too many requests for one launch");
@@ -384,7 +385,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
     if (split_waves) {
         dim3 grid(groups * num_splits, n_kv_heads * HB, n_seqs);
-        if (int e = launch_attn<true>(head_dim / 16, grid, a, stream)) return e;
+        if (int e = launch_attn<true>(head_dim / 16, grid, waves * LLMS_WAVE, a, stream)) return e;
         if (num_splits > 1) {
             hipError_t e1 = hipGetLastError();
             if (e1 != hipSuccess) {
@@ -396,7 +397,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
         }
     } else {
         dim3 grid((groups + 3) / 4, n_kv_heads * HB, n_seqs);
-        if (int e = launch_attn<false>(head_dim / 16, grid, a, stream)) return e;
+        if (int e = launch_attn<false>(head_dim / 16, grid, 256, a, stream)) return e;
     }
     LLMS_LAUNCH_CHECK();
 }

@@ -1,7 +1,10 @@
-// bfloat16 matrix product for few rows (M <= 16, decoding):  C[M,N] = X[M,K] * W[N,K]^T, 32-bit sums on
-// the gfx950 matrix cores, built around reading the weight once at memory speed.
+// bfloat16 matrix product for few rows (decoding):  C[M,N] = X[M,K] * W[N,K]^T, 32-bit sums on the gfx950
+// matrix cores, built around reading the weight once at memory speed.
 //
-// A workgroup owns 16 weight rows; its 4 waves take the K chunks (512 wide) in turn.  One load instruction
+// A workgroup owns 16 weight rows and 16 rows of X; its 4 waves take the K chunks (512 wide) in turn.
+// (More than 16 rows of X, up to 64: one workgroup per block of 16 rows; the workgroups that share weight
+// rows get consecutive places on the same XCD, so the weights cross HBM once and come from that XCD's L2
+// for the others.)  One load instruction
 // of a wave covers 1 KB of one weight row (fully coalesced, non-temporal), 16 such loads are in flight per
 // wave before anything waits, and the next chunk's loads are issued before the arithmetic of this one.
 // The 16 KB go through a wave-private, XOR-swizzled LDS tile to reach the layout of
@@ -55,6 +58,7 @@ struct StreamArgs {
     const bf16* W;
     const bf16* bias;
     int M, N, K;
+    int num_tiles;  // tiles of 16 weight rows (8 features for the gated and rotary epilogues)
     // NORM
     const bf16* delta;
     const bf16* norm_w;
@@ -93,7 +97,12 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     __shared__ uint4 lds[ST_WAVES * 16 * (ST_KC / 8)];  // 64 KB: per wave 16 rows x 64 chunks of 16 bytes
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
     const int r16 = lane % 16, g = lane / 16;
-    const int tile_id = blockIdx.x;
+    // Workgroups go round the 8 XCDs; tile t lives on XCD t % 8, its blocks of 16 rows of X next to each other
+    const int m_blocks = (a.M + 15) / 16;
+    const int xcd = blockIdx.x % 8, place = blockIdx.x / 8;
+    const int tile_id = (place / m_blocks) * 8 + xcd;
+    const int m0 = (place % m_blocks) * 16;
+    if (tile_id >= a.num_tiles) return;
     const int M = a.M, N = a.N, K = a.K;
     const uint4 zero = make_uint4(0, 0, 0, 0);
 
@@ -133,9 +142,9 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     };
     if (wave < chunks) load_weights(wave);  // in flight while the row statistics are computed
 
-    const bool m_ok = r16 < M;
-    const bf16* xrow = a.X + (size_t)(m_ok ? r16 : 0) * a.ldx;
-    const bf16* drow = (NORM && a.delta) ? a.delta + (size_t)(m_ok ? r16 : 0) * a.ldx : nullptr;
+    const bool m_ok = m0 + r16 < M;
+    const bf16* xrow = a.X + (size_t)(m_ok ? m0 + r16 : 0) * a.ldx;
+    const bf16* drow = (NORM && a.delta) ? a.delta + (size_t)(m_ok ? m0 + r16 : 0) * a.ldx : nullptr;
     // x chunk of 8 at column k of this lane's row: the residual sum in 32-bit, rounded once
     auto load_x = [&](int k) -> uint4 {
         uint4 v = *reinterpret_cast<const uint4*>(xrow + k);
@@ -163,7 +172,7 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
                     unpack8(v, xf);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) ss += xf[e] * xf[e];
-                    if (a.resid_out && tile_id == 0) *reinterpret_cast<uint4*>(a.resid_out + (size_t)r16 * a.ldx + k) = v;
+                    if (a.resid_out && tile_id == 0) *reinterpret_cast<uint4*>(a.resid_out + (size_t)(m0 + r16) * a.ldx + k) = v;
                 }
             }
         }
@@ -215,9 +224,9 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[(wave * LLMS_WAVE + lane) * 4 + r] = acc[r];
     __syncthreads();
-    // sum of the 4 waves for weight row i (0..15) of this tile and row m of X, wave 0 first
-    auto total_of = [&](int i, int m) -> float {
-        const int src_lane = (i / 4) * 16 + m, r = i % 4;
+    // sum of the 4 waves for weight row i (0..15) of this tile and row m0 + ml of X, wave 0 first
+    auto total_of = [&](int i, int ml) -> float {
+        const int src_lane = (i / 4) * 16 + ml, r = i % 4;
         float s = 0.f;
 #pragma unroll
         for (int w = 0; w < ST_WAVES; ++w) s += red[(w * LLMS_WAVE + src_lane) * 4 + r];
@@ -227,25 +236,25 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     TOut* C = reinterpret_cast<TOut*>(a.C);
 
     if (EPI == EPI_PLAIN) {
-        const int i = idx % 16, m = idx / 16, n = tile_id * 16 + i;  // consecutive threads: consecutive features
+        const int i = idx % 16, ml = idx / 16, m = m0 + ml, n = tile_id * 16 + i;  // consecutive threads: consecutive features
         if (m < M && n < N) {
-            float s = total_of(i, m);
+            float s = total_of(i, ml);
             if (a.bias) s += bf16_bits_to_f32(a.bias[n].bits);
             store_out<TOut>(C + (size_t)m * a.ldc + n, s);
         }
     } else if (EPI == EPI_SWIGLU) {
-        const int j = idx % 8, m = idx / 8, f = tile_id * 8 + j;
+        const int j = idx % 8, ml = idx / 8, m = m0 + ml, f = tile_id * 8 + j;
         if (idx < 128 && m < M && f < a.inter) {
-            const float gate = bfr(total_of(j, m)), up = bfr(total_of(j + 8, m));
+            const float gate = bfr(total_of(j, ml)), up = bfr(total_of(j + 8, ml));
             store_out<TOut>(C + (size_t)m * a.ldc + f, bfr(gate / (1.f + expf(-gate))) * up);
         }
     } else {
         const int nh = a.n_heads, nkv = a.n_kv_heads, bs = a.block_size;
         if (tile_id < rot_tiles) {
-            const int j = idx % 8, m = idx / 8;
+            const int j = idx % 8, ml = idx / 8, m = m0 + ml;
             if (idx < 128 && m < M) {
                 const int h = tile_id / spt, s = tile_id % spt, d = 8 * s + j;
-                float lo = total_of(j, m), hi = total_of(j + 8, m);
+                float lo = total_of(j, ml), hi = total_of(j + 8, ml);
                 if (a.bias) {
                     lo += bf16_bits_to_f32(a.bias[h * D + d].bits);
                     hi += bf16_bits_to_f32(a.bias[h * D + d + D / 2].bits);
@@ -273,11 +282,11 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
                 }
             }
         } else {
-            const int i = idx % 16, m = idx / 16;
+            const int i = idx % 16, ml = idx / 16, m = m0 + ml;
             const int slot = (a.slots && m < M) ? a.slots[m] : -1;
             if (m < M && slot >= 0) {
                 const int f = (tile_id - rot_tiles) * 16 + i;  // feature among the value heads
-                float v = total_of(i, m);
+                float v = total_of(i, ml);
                 if (a.bias) v += bf16_bits_to_f32(a.bias[(nh + nkv) * D + f].bits);
                 const int kvh = f / D, d = f % D, page = slot / bs, off = slot % bs;
                 a.v_pool[(((size_t)page * nkv + kvh) * D + d) * bs + off].bits = f32_to_bf16_bits(v);
@@ -305,7 +314,8 @@ int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* 
                      void* resid_out, int inter, int n_heads, int n_kv_heads, int head_dim, int block_size,
                      const float* inv_freq, const int* positions, const int* slots, void* k_pool, void* v_pool,
                      hipStream_t stream) {
-    LLMS_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_stream: needs 1 <= M <= 16 and positive sizes");
+    LLMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_stream: needs 1 <= M <= 64 and positive sizes");
+    LLMS_REQUIRE(norm_w == nullptr || M <= 16, "gemm_stream: the norm prologue takes at most 16 rows");
     LLMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "gemm_stream: K and the row stride of X must be multiples of 8");
     LLMS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_stream: X and W must be 16-byte aligned");
     LLMS_REQUIRE(C != nullptr && (out_dtype == 0 || out_dtype == 1), "gemm_stream: bad output");
@@ -317,7 +327,7 @@ int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* 
     } else {
         LLMS_REQUIRE(!delta && !resid_out, "gemm_stream: delta and resid_out need norm_w");
     }
-    StreamArgs a = {C, ldc, (const bf16*)X, ldx, (const bf16*)W, (const bf16*)bias, M, N, K, (const bf16*)delta,
+    StreamArgs a = {C, ldc, (const bf16*)X, ldx, (const bf16*)W, (const bf16*)bias, M, N, K, 0, (const bf16*)delta,
                     (const bf16*)norm_w, eps, (bf16*)resid_out, inter, n_heads, n_kv_heads, head_dim, block_size,
                     inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool};
     unsigned grid;
@@ -336,6 +346,8 @@ int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* 
         LLMS_REQUIRE(slots == nullptr || (k_pool && v_pool && block_size > 0), "gemm_stream: slots given without pools");
         grid = (n_heads + n_kv_heads) * (head_dim / 16) + n_kv_heads * head_dim / 16;
     }
+    a.num_tiles = (int)grid;
+    grid = ((grid + 7) / 8) * 8 * ((M + 15) / 16);  // every XCD gets whole tiles with all their row blocks
     const bool norm = norm_w != nullptr;
 #define ST_EPI(E)                                                                  \
     if (out_dtype == 0) launch_stream<float, E>(norm, grid, a, stream);           \

@@ -302,7 +302,7 @@ def gemm_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.T
 
 def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, *,
                 norm: tuple | None = None, swiglu: bool = False, rope: dict | None = None) -> torch.Tensor:
-    """The product for up to 16 bfloat16 rows, with what surrounds it fused in.
+    """The product for up to 64 bfloat16 rows (built for up to 16), with what surrounds it fused in.
 
     plain:   out[M, N] = x w^T (+ bias).
     norm = (delta | None, norm_weight, eps, resid_out | None): x is the residual stream; delta is added
@@ -318,8 +318,10 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
     _rows(w, "w", x.shape[1])
     m, k = x.shape
     n = w.shape[0]
-    if not 0 < m <= 16:
-        raise ValueError("gemm_stream takes 1..16 rows")
+    if not 0 < m <= 64:
+        raise ValueError("gemm_stream takes 1..64 rows")
+    if norm is not None and m > 16:
+        raise ValueError("the norm prologue takes at most 16 rows")
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or out.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("gemm_stream takes bfloat16 operands and stores bfloat16 or float32")
     if not gemm_bf16_supported(x, w):
@@ -443,11 +445,11 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
                    seq_begin: int, n_seqs: int, max_new: int, token_begin: int, n_tokens: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, block_size: int, window: int = 0,
                    scale: float | None = None, split_waves: bool = False, num_splits: int = 1,
-                   table_rows: torch.Tensor | None = None) -> torch.Tensor:
+                   table_rows: torch.Tensor | None = None, waves: int = 4) -> torch.Tensor:
     """bfloat16 causal attention on the matrix cores for requests [seq_begin, seq_begin + n_seqs) of a
     step, whose new tokens are rows [token_begin, token_begin + n_tokens) of q and out and bring at most
-    `max_new` tokens each.  `split_waves` (with `num_splits`) spreads each request's keys over waves and
-    workgroups: the arrangement for single decoded tokens."""
+    `max_new` tokens each.  `split_waves` (with `waves` = 4 or 8 and `num_splits`) spreads each request's keys
+    over the waves of a workgroup and over workgroups: the arrangement for single decoded tokens."""
     dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, table_rows)
     _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
     if not attention_mfma_supported(q.dtype, head_dim, block_size):
@@ -468,6 +470,8 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
         raise ValueError("q rows must be 16-byte aligned")
     if num_splits > 1 and not split_waves:
         raise ValueError("num_splits > 1 needs split_waves")
+    if waves != 4 and not (split_waves and waves == 8):
+        raise ValueError("4 waves, or 8 when the waves share the keys")
     if n_seqs == 0 or n_tokens == 0:
         return out
     ws_o = ws_ml = None
@@ -481,7 +485,7 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
         c_int(seq_begin),
         c_int(n_seqs), c_int(max_new), c_int(token_begin), c_int(n_tokens), c_int(n_heads), c_int(n_kv_heads),
         c_int(head_dim), c_int(block_size), c_int(window), c_float(scale), c_int(1 if split_waves else 0),
-        c_int(num_splits), _ptr(ws_o), _ptr(ws_ml), _stream(dev)), "attention_mfma")
+        c_int(num_splits), c_int(waves), _ptr(ws_o), _ptr(ws_ml), _stream(dev)), "attention_mfma")
     return out
 
 

@@ -16,7 +16,7 @@ import math
 import torch
 
 from ..ops import library as ops
-from .linear import FUSE_NORM_INTO_PRODUCT, LIBRARY_ABOVE_ROWS, linear
+from .linear import FUSE_NORM_INTO_PRODUCT, STREAM_ROWS, few_rows, linear
 from .registry import POSITION_ENCODINGS, DeferredNorm, Mixer, register_mixer
 from .rmsnorm import RMSNorm
 from .spec import PagedCacheSpec, ParamInfo
@@ -89,20 +89,19 @@ class Attention(Mixer):
         return linear(out, self.o_weight)
 
     def _few_rows_unfit(self, rows) -> bool:
-        m = rows.shape[0]
-        return (rows.dtype != torch.bfloat16 or not 0 < m <= LIBRARY_ABOVE_ROWS or self.head_dim % 16 != 0
+        return (rows.dtype != torch.bfloat16 or not few_rows(rows.shape[0], self.qkv_weight) or self.head_dim % 16 != 0
                 or not ops.gemm_bf16_supported(rows, self.qkv_weight))
 
     def project_few_rows(self, x, batch, cache, slots):
-        """With up to 16 bfloat16 rows one kernel does the residual sum, the norm, the projection, the
-        rotation and the cache store (ops.gemm_stream); returns the rotated queries, or None when that
-        kernel does not apply."""
+        """With few bfloat16 rows one kernel does the projection, the rotation and the cache store (and,
+        if switched on, the residual sum and the norm before them): ops.gemm_stream.  Returns the rotated
+        queries, or None when that kernel does not apply."""
         if isinstance(x, DeferredNorm) and not FUSE_NORM_INTO_PRODUCT:
             return None if self._few_rows_unfit(x.residual) else self.project_few_rows(x.materialize(), batch, cache, slots)
         deferred = isinstance(x, DeferredNorm)
         rows = x.residual if deferred else x
         m = rows.shape[0]
-        if self._few_rows_unfit(rows) or (deferred and not isinstance(x.norm, RMSNorm)):
+        if self._few_rows_unfit(rows) or (deferred and (m > STREAM_ROWS or not isinstance(x.norm, RMSNorm))):
             return None
         frequencies = getattr(self.position, "rotary_frequencies", None)
         if frequencies is None and not getattr(self.position, "identity", False):
@@ -131,20 +130,25 @@ class Attention(Mixer):
         common = (out, qkv, cache.k_pool, cache.v_pool, view.block_tables, batch.cu_seqlens, batch.context_lens)
         n_dec = batch.num_decode
         if n_dec:  # requests that bring one token: their keys are spread over waves and workgroups
+            splits, waves = self.decode_arrangement(n_dec, batch.max_decode_context)
             ops.attention_mfma(*common, 0, n_dec, 1, 0, n_dec, nh, nkv, d, bs, window, self.scale,
-                               split_waves=True, num_splits=self.decode_splits(n_dec, batch.max_decode_context),
-                               table_rows=batch.state_slots)
+                               split_waves=True, num_splits=splits, waves=waves, table_rows=batch.state_slots)
         if n_dec < batch.num_seqs:  # portions of prompts: one wave per group of tokens and heads
             ops.attention_mfma(*common, n_dec, batch.num_seqs - n_dec, batch.max_count, n_dec,
                                batch.num_tokens - n_dec, nh, nkv, d, bs, window, self.scale,
                                table_rows=batch.state_slots)
 
-    def decode_splits(self, n_requests: int, max_context: int) -> int:
-        """Workgroups per (request, KV head) for decoding.  A workgroup's 4 waves take 32 keys at a time
-        each; a small batch is spread over more workgroups, down to stretches of 128 keys (one tile per
-        wave, the shortest chain of dependent steps), whose partial results a second kernel merges; once
-        the batch alone fills the chip (256 workgroups) nothing is split."""
+    def decode_arrangement(self, n_requests: int, max_context: int) -> tuple[int, int]:
+        """(workgroups per request and KV head, waves per workgroup) for decoding.  The waves of a
+        workgroup take 32 keys at a time each and merge inside the kernel; workgroups that share a
+        request need a second kernel to merge, which costs more than a few extra tiles per wave.  So a
+        small batch first gets 8 waves, and is split over workgroups only when a wave would still
+        walk more than 4 tiles; once the batch alone fills the chip (256 workgroups) nothing is split."""
         g = self.num_heads // self.num_kv_heads
         groups = n_requests * self.num_kv_heads * -(-g // 16)
         reach = min(max_context, self.window) if self.window else max_context
-        return max(1, min(256 // groups, -(-reach // 128)))
+        if groups >= 256:
+            return 1, 4
+        tiles = -(-reach // 32)
+        splits = max(1, min(256 // groups, -(-tiles // 32)))
+        return splits, 8

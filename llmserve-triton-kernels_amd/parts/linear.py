@@ -1,7 +1,9 @@
 """y = x W^T (+ b) for the parts: picks the matrix product by dtype and shape.
 
 float32: the 32-bit multiply-add kernel, always (no reduced-precision matrix mode).
-bfloat16, up to 16 rows (decoding): the hand-written kernel that streams the weight once.
+bfloat16, few rows (decoding): the hand-written kernel that streams the weight once
+  (ops.gemm_stream); it takes up to 64 rows, one workgroup per 16 rows and 16 weight rows, so
+  beyond 16 rows the weights are re-read from L2 and it only pays for the smaller matrices.
 bfloat16, more rows: the library's matrix product (hipBLASLt through torch.mm), which is
   where the reference's engine uses a library too (nn.Linear, src/llmserve/model/llama.py:64-67);
   sums are 32-bit, the result bfloat16 or, for logits, float32.
@@ -16,7 +18,19 @@ import torch
 from ..ops import library as ops
 
 
-LIBRARY_ABOVE_ROWS = 16
+STREAM_ROWS = 16  # up to here the streaming kernel always wins
+STREAM_MAX_ROWS = 64
+# beyond STREAM_ROWS: bytes of weight times blocks of 16 rows up to which the streaming kernel still beats
+# the library (measured on the TinyLlama shapes at 32 and 64 rows, with the epilogue it saves counted in)
+STREAM_REREAD_BYTES = 64e6
+
+
+def few_rows(m: int, weight: torch.Tensor) -> bool:
+    """Whether `m` bfloat16 rows against `weight` go to ops.gemm_stream."""
+    if m <= STREAM_ROWS:
+        return m > 0
+    return m <= STREAM_MAX_ROWS and -(-m // 16) * weight.numel() * 2 <= STREAM_REREAD_BYTES
+
 # Whether the few-row product also does the residual sum and the norm in front of it
 # (ops.gemm_stream(norm=...)).  Off: every workgroup repeats the statistics and the rounding of its
 # rows with most lanes idle, which measured slower (TinyLlama shape, batch 1: 2.7 ms against
@@ -34,8 +48,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     if m == 0:
         return out
     if x.dtype == torch.bfloat16 and ops.gemm_bf16_supported(x, weight):
-        if m <= LIBRARY_ABOVE_ROWS:
-            return ops.gemm_bf16(out, x, weight, bias)
+        if few_rows(m, weight):
+            return ops.gemm_stream(out, x, weight, bias)
         if bias is None:
             return torch.mm(x, weight.t(), out_dtype=out.dtype, out=out)
         return torch.addmm(bias.to(out.dtype), x, weight.t(), out_dtype=out.dtype, out=out)

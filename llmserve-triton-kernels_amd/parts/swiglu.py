@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .linear import FUSE_NORM_INTO_PRODUCT, LIBRARY_ABOVE_ROWS, linear
+from .linear import FUSE_NORM_INTO_PRODUCT, STREAM_ROWS, few_rows, linear
 from .registry import DeferredNorm, FeedForward, register_feed_forward
 from .rmsnorm import RMSNorm
 from .spec import ParamInfo
@@ -41,10 +41,10 @@ class SwiGLU(FeedForward):
         m = x.num_rows if isinstance(x, DeferredNorm) else x.shape[0]
         dtype, device = self.gate_up.dtype, self.gate_up.device
         act = torch.empty((m, self.intermediate), dtype=dtype, device=device)
-        few = dtype == torch.bfloat16 and 0 < m <= LIBRARY_ABOVE_ROWS and self.intermediate % 8 == 0
+        few = dtype == torch.bfloat16 and few_rows(m, self.gate_up) and self.intermediate % 8 == 0
         if isinstance(x, DeferredNorm):
             norm = x.norm
-            if (FUSE_NORM_INTO_PRODUCT and few and isinstance(norm, RMSNorm)
+            if (FUSE_NORM_INTO_PRODUCT and few and m <= STREAM_ROWS and isinstance(norm, RMSNorm)
                     and ops.gemm_bf16_supported(x.residual, self.gate_up)):
                 new_residual = torch.empty_like(x.residual) if x.delta is not None else None
                 ops.gemm_stream(act, x.residual, self.gate_up, norm=(x.delta, norm.weight, norm.eps, new_residual),

@@ -162,7 +162,8 @@ def test_gemm_bf16(kernel, m, n, k):
     assert (out.float().cpu().double() - ref).abs().max() <= 2.0 ** -8 * float(ref.abs().max())
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 16, 64), (3, 333, 96), (16, 2056, 2048), (7, 100, 5632), (9, 48, 176)])
+@pytest.mark.parametrize("m,n,k", [(1, 16, 64), (3, 333, 96), (16, 2056, 2048), (7, 100, 5632), (9, 48, 176),
+                                   (17, 333, 96), (64, 2056, 2048), (40, 100, 5632), (33, 48, 176)])
 def test_gemm_stream_plain(m, n, k):
     x, w, b = rnd(m, k, seed=11).bfloat16(), rnd(n, k, seed=12).bfloat16(), rnd(n, seed=13).bfloat16()
     ref = x.double() @ w.double().t() + b.double()
@@ -170,7 +171,7 @@ def test_gemm_stream_plain(m, n, k):
     assert (out.cpu().double() - ref).abs().max() <= 2e-6 * math.sqrt(k) * float(ref.abs().max())
 
 
-@pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96)])
+@pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96), (37, 5632, 2048), (64, 256, 1024)])
 def test_gemm_stream_gated_epilogue(m, inter, k):
     """gate and up of the feed-forward in one product over [gate; up], silu(gate) * up in the epilogue:
     the same bits as the product followed by the activation kernel."""
@@ -206,17 +207,22 @@ def test_gemm_stream_norm_prologue(m, n, k, eps, with_delta):
         ops().gemm_stream(torch.empty(m, n, device=DEV), r, w.to(DEV), norm=(delta.to(DEV), wn.to(DEV), eps, r))
 
 
-@pytest.mark.parametrize("nh,nkv,d,bs,theta,bias", [(4, 2, 16, 16, 1e4, False), (3, 1, 32, 8, 5e5, True),
-                                                    (8, 2, 64, 16, 1e4, False), (2, 2, 48, 8, None, True)])
-def test_gemm_stream_rotary_epilogue(nh, nkv, d, bs, theta, bias):
+@pytest.mark.parametrize("nh,nkv,d,bs,theta,bias,m", [(4, 2, 16, 16, 1e4, False, 5), (3, 1, 32, 8, 5e5, True, 5),
+                                                      (8, 2, 64, 16, 1e4, False, 64), (2, 2, 48, 8, None, True, 33)])
+def test_gemm_stream_rotary_epilogue(nh, nkv, d, bs, theta, bias, m):
     """q/k/v projection with the rotation and the cache store in the epilogue: the same bits as the
     projection followed by the rotation kernel."""
-    m, k, pages = 5, 96, 6
+    k, pages = 96, 12
     n = (nh + 2 * nkv) * d
     x, w = rnd(m, k, seed=23).bfloat16().to(DEV), rnd(n, k, seed=24, scale=0.3).bfloat16().to(DEV)
     b = rnd(n, seed=25).bfloat16().to(DEV) if bias else None
-    positions = torch.tensor([0, 1, 77, 500, 4095], dtype=torch.int32, device=DEV)
-    slots = torch.tensor([3, bs * pages - 1, -1, 0, bs * 2 + 1], dtype=torch.int32, device=DEV)
+    gen = torch.Generator().manual_seed(35)
+    positions = torch.randint(0, 4096, (m,), generator=gen).to(torch.int32)
+    positions[0] = 0
+    positions = positions.to(DEV)
+    slots = torch.randperm(bs * pages, generator=gen)[:m].to(torch.int32)
+    slots[m // 2] = -1
+    slots = slots.to(DEV)
     inv_freq = (1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV) if theta else None
     pools = lambda: (torch.full((pages, nkv, bs, d), 7.0, dtype=torch.bfloat16, device=DEV),  # noqa: E731
                      torch.full((pages, nkv, d, bs), 7.0, dtype=torch.bfloat16, device=DEV))
@@ -243,9 +249,9 @@ def test_gemm_bf16_rows_do_not_depend_on_the_batch():
     full = ops().gemm_bf16(torch.empty(40, 320, device=DEV), a, w, kernel="skinny")
     one = ops().gemm_bf16(torch.empty(1, 320, device=DEV), a[17:18].contiguous(), w, kernel="skinny")
     assert torch.equal(full[17], one[0])
-    full = ops().gemm_stream(torch.empty(16, 320, device=DEV), a[:16].contiguous(), w)
-    one = ops().gemm_stream(torch.empty(1, 320, device=DEV), a[9:10].contiguous(), w)
-    assert torch.equal(full[9], one[0])
+    full = ops().gemm_stream(torch.empty(40, 320, device=DEV), a, w)
+    one = ops().gemm_stream(torch.empty(1, 320, device=DEV), a[29:30].contiguous(), w)
+    assert torch.equal(full[29], one[0])
 
 
 def test_gemm_bf16_refuses_what_it_cannot_take():
@@ -400,7 +406,8 @@ def test_sample_rows_mixed_batch_and_frequencies():
 
 
 # ------------------------------------------------------------------ attention on the matrix cores
-def run_attention_mfma(nh, nkv, d, bs, lens, new, window=0, seed=0, craft=None, split_waves=False, num_splits=1):
+def run_attention_mfma(nh, nkv, d, bs, lens, new, window=0, seed=0, craft=None, split_waves=False, num_splits=1,
+                       waves=4):
     """As `run_attention`, for the bfloat16 matrix-core kernel and its request-wise arguments."""
     dtype = torch.bfloat16
     qs = [rnd(s, nh, d, seed=seed + 3 * b) for b, s in enumerate(lens)]
@@ -422,7 +429,7 @@ def run_attention_mfma(nh, nkv, d, bs, lens, new, window=0, seed=0, craft=None, 
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)  # noqa: E731
     ops().attention_mfma(out, q, k_pool.to(DEV), v_pool.to(DEV), tables.to(DEV), i32(cu), i32(lens), 0, len(lens),
                          max(new), 0, cu[-1], nh, nkv, d, bs, window, None, split_waves=split_waves,
-                         num_splits=num_splits)
+                         num_splits=num_splits, waves=waves)
     got = out.float().cpu()
     assert torch.isfinite(got).all(), "read a slot that was never written"
     return got, torch.cat(refs)
@@ -446,17 +453,17 @@ MFMA_CASES = [  # nh, nkv, d, bs, lens, new, window
 ]
 
 
-@pytest.mark.parametrize("arrangement", [(False, 1), (True, 1), (True, 2), (True, 5)])
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 4), (True, 2, 4), (True, 5, 4), (True, 1, 8), (True, 3, 8)])
 @pytest.mark.parametrize("case", MFMA_CASES)
 def test_attention_mfma(case, arrangement):
     nh, nkv, d, bs, lens, new, window = case
-    split_waves, num_splits = arrangement
+    split_waves, num_splits, waves = arrangement
     got, ref = run_attention_mfma(nh, nkv, d, bs, lens, new, window, seed=50, split_waves=split_waves,
-                                  num_splits=num_splits)
+                                  num_splits=num_splits, waves=waves)
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
 
 
-@pytest.mark.parametrize("arrangement", [(False, 1), (True, 1), (True, 3)])
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 4), (True, 3, 4), (True, 1, 8)])
 @pytest.mark.parametrize("needle", [0, 15, 16, 31, 32, 299, 300 - 17, 141])
 def test_attention_mfma_finds_one_far_key(needle, arrangement):
     def craft(qs, ks, vs):
@@ -467,7 +474,7 @@ def test_attention_mfma_finds_one_far_key(needle, arrangement):
         vs[0][needle] = 3.0
 
     got, ref = run_attention_mfma(8, 2, 64, 16, [300], [1], 0, seed=60, craft=craft, split_waves=arrangement[0],
-                                  num_splits=arrangement[1])
+                                  num_splits=arrangement[1], waves=arrangement[2])
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max()) and got.mean() > 2.9
 
 
