@@ -148,7 +148,7 @@ class Attention(Mixer):
         groups = n_requests * self.num_kv_heads * -(-g // 16)
         reach = min(max_context, self.window) if self.window else max_context
         if groups >= 256:
-            return 1, 4
+            return 1, 8
         tiles = -(-reach // 32)
         splits = max(1, min(256 // groups, -(-tiles // 32)))
         return splits, 8

@@ -9,13 +9,21 @@ bfloat16, more rows: the library's matrix product (hipBLASLt through torch.mm), 
   sums are 32-bit, the result bfloat16 or, for logits, float32.
 Operands the matrix-core kernels cannot take (K not a multiple of 8) fall to the 32-bit
 multiply-add kernel, which takes anything.
+
+LLMSERVE_GEMM=own in the environment keeps the library out altogether: products the streaming
+kernel does not take then go to this repository's tiled matrix-core kernels (ops.gemm_bf16), a
+few times slower than hipBLASLt on large shapes but free of any library.
 """
 
 from __future__ import annotations
 
+import os
+
 import torch
 
 from ..ops import library as ops
+
+OWN_KERNELS_ONLY = os.environ.get("LLMSERVE_GEMM", "") == "own"
 
 
 STREAM_ROWS = 16  # up to here the streaming kernel always wins
@@ -50,6 +58,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     if x.dtype == torch.bfloat16 and ops.gemm_bf16_supported(x, weight):
         if few_rows(m, weight):
             return ops.gemm_stream(out, x, weight, bias)
+        if OWN_KERNELS_ONLY:
+            return ops.gemm_bf16(out, x, weight, bias, kernel="skinny" if m <= 64 else "tile")
         if bias is None:
             return torch.mm(x, weight.t(), out_dtype=out.dtype, out=out)
         return torch.addmm(bias.to(out.dtype), x, weight.t(), out_dtype=out.dtype, out=out)

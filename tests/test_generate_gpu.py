@@ -125,3 +125,24 @@ def test_command_line(model_dirs):
                             capture_output=True, text=True, env=env, timeout=120)
     assert folder.returncode == 0, folder.stderr
     assert len(eval(folder.stdout.strip().splitlines()[0])) == 4
+
+
+def test_generation_without_the_library_product(model_dirs):
+    """LLMSERVE_GEMM=own: every matrix product on this repository's kernels, same tokens."""
+    code = ("import sys; sys.path[:0] = [%r, %r]\n"
+            "import torch, plain_llama, traces\n"
+            "from llmserve import LLM, EngineConfig, SamplingParams\n"
+            "from llmserve.parts import linear\n"
+            "assert linear.OWN_KERNELS_ONLY\n"
+            "d = %r\n"
+            "prompts = [traces.random_ids(333, n, 300 + i) for i, n in enumerate([7, 100])]\n"
+            "llm = LLM(d, dtype='bfloat16', engine=EngineConfig(block_size=8, num_blocks=64, max_num_seqs=4, max_num_batched_tokens=128))\n"
+            "toks = [r.tokens for r in llm.generate(prompts, SamplingParams(max_new_tokens=8))]\n"
+            "for p, t in zip(prompts, toks):\n"
+            "    ref = traces.plain_logits(d, p + t, torch.bfloat16)\n"
+            "    tol = traces.tolerance(torch.bfloat16, ref)[0]\n"
+            "    assert all(ref[len(p) - 1 + i].max() - ref[len(p) - 1 + i][x] <= 2 * tol for i, x in enumerate(t))\n"
+            "print('ok')\n") % (ROOT, os.path.join(ROOT, "tests"), str(model_dirs["b"]))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120,
+                         env=dict(os.environ, LLMSERVE_GEMM="own"))
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stderr[-2000:]
