@@ -38,6 +38,8 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--model", default="tinyllama-1.1b")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--phase", choices=["all", "decode", "prefill"], default="all",
+                    help="run one phase only (for profiles; the line then holds zeros for the other)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
@@ -61,7 +63,7 @@ def main() -> int:
     d = h // nh
     elem = 2 if args.dtype == "bfloat16" else 4
     block_size = 16
-    max_batch = 64 if not args.no_points else args.batch
+    max_batch = 64 if not args.no_points and args.phase == "all" else args.batch
     budget = max(PREFILL_TOKENS, max_batch)
     # requests whose prompt went in first decode while the others' prompts still go in
     slack = -(-max_batch * args.context // budget) + 2
@@ -111,11 +113,11 @@ def main() -> int:
             assert not eng.has_unfinished()
         return sorted(times[1:])[len(times[1:]) // 2]
 
-    value, step_s = decode_rate(args.batch)
+    value, step_s = decode_rate(args.batch) if args.phase != "prefill" else (0.0, float("inf"))
     points = {}
-    if not args.no_points:
+    if not args.no_points and args.phase == "all":
         points = {"decode_b1": round(decode_rate(1)[0], 1), "decode_b64": round(decode_rate(64)[0], 1)}
-    pre_s = prefill_time()
+    pre_s = prefill_time() if args.phase != "decode" else float("inf")
 
     # bytes a decode step must read: every matrix and norm once, the rows of the embedding it
     # gathers, and the keys and values of the live requests at their mean length in the timed steps
@@ -129,16 +131,19 @@ def main() -> int:
     linear = 2 * t * layers * ((nh + 2 * nkv) * d * h + h * nh * d + 3 * h * inter)
     attention = layers * 4 * nh * d * t * (t + 1) / 2
     flops = linear + attention + 2 * vocab * h
+    def ms(seconds):
+        return round(seconds * 1e3, 4) if seconds != float("inf") else 0.0
+
     line = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (TinyLlama 1.1B)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": ms(step_s), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": {"model": args.model, "global_batch": args.batch, "seq_len": args.context,
                    "parallelism": "single-gpu", "layers": layers, "layers_full": full_layers, "hidden": h,
                    "heads": nh, "kv_heads": nkv, "head_dim": d, "intermediate": inter, "vocab": vocab,
                    "block_size": block_size, "weights": "random", "prefill_tokens": PREFILL_TOKENS},
-        "prefill": {"value": round(t / pre_s, 1), "tokens": t, "ms": round(pre_s * 1e3, 3),
+        "prefill": {"value": round(t / pre_s, 1), "tokens": t, "ms": ms(pre_s),
                     "frac": round(flops / pre_s / PEAK_FLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},

@@ -13,8 +13,10 @@
 // the two S^T tiles is chosen so that each lane ends up with 8 consecutive keys, which is what
 // the B operand of the second product wants: no exchange between lanes.
 //
-// Two arrangements of the 4 waves of a workgroup:
-//   SPLIT_WAVES = false (prompts): 4 consecutive column groups of one request.
+// Arrangements of the waves of a workgroup:
+//   attn_prompt_kernel (prompts): 4 consecutive column groups of one request share each tile of keys through
+//     LDS (the exception to "nothing goes through LDS": 4 waves want the same bytes).
+//   SPLIT_WAVES = false: the same 4 column groups, every wave loading for itself (kept for comparison).
 //   SPLIT_WAVES = true  (decoding): one column group; the key tiles are dealt to the 4 or 8 waves, and
 //     optionally to `num_splits` workgroups whose partial results a second kernel merges.
 // All merges run in a fixed order, so a token's result does not depend on the batch around it.
@@ -63,8 +65,76 @@ struct AttnArgs {
     float* ws_ml;  // [token, head, split, 2]
 };
 
+// 2^x by the hardware's own instruction.  Scores are kept in units of log2(e) (scale_log2 = scale * log2 e), so
+// that a weight is one multiply-add and one exponential.
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ const bf16* page_ptr(const bf16* base, int page, uint32_t page_stride) {
+    return base + (uint64_t)(uint32_t)page * page_stride;  // one 32 x 32 -> 64 bit multiply-add
+}
+
+// One tile of 32 keys for a wave's 16 columns: scores, online softmax, weighted values.
+//   kf[u][s]: key rows of score tile u (row i = key 8*(i/4) + 4u + i%4), k-step s;  vf[m]: the lane's 8 keys
+//   (jk .. jk+7) of value dimensions 16m + col, already zero where the key is outside the group's range;
+//   qf[s]: the lane's column of queries.  acc[m][r] = O^T[16m + 4g + r][col] and the running max (times log2 e)
+//   and sum of the column are updated in place.  MASKED = false: every key of the tile is visible to every
+//   column of the wave (the caller knows), which saves the comparisons.  The accumulators are rescaled only
+//   when some column's maximum grew: a factor of exactly 1 otherwise, so the result is the same.
+template <int DB, int KS, bool MASKED>
+__device__ __forceinline__ void attend_tile(f32x4 (&acc)[DB], float& m_run, float& l_run, const uint4 (&kf)[2][KS],
+                                            const uint4 (&vf)[DB], const uint4 (&qf)[KS], int jk, int lo_col, int p_col,
+                                            float scale_log2) {
+    f32x4 s_acc[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        s_acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u][s]), as_bf16x8(qf[s]), s_acc[u], 0, 0, 0);
+    }
+    // the lane holds its column's scores for the keys jk .. jk+7; the other 24 keys sit in the 3 other lane groups
+    float sc[8];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        sc[e] = s_acc[e / 4][e % 4];
+        if (MASKED) {
+            const int key = jk + e;
+            if (!(key >= lo_col && key <= p_col)) sc[e] = -INFINITY;
+        }
+        tmax = fmaxf(tmax, sc[e]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, LLMS_WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, LLMS_WAVE));
+    const float m_new = fmaxf(m_run, tmax * scale_log2);  // (scale > 0)
+    const float m_safe = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
+    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+        const float corr = exp2_fast(m_run - m_safe);  // 0 while the column has seen no key
+        l_run *= corr;
+#pragma unroll
+        for (int m = 0; m < DB; ++m)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[m][r] *= corr;
+        m_run = m_new;
+    }
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        sc[e] = exp2_fast(fmaf(sc[e], scale_log2, -m_safe));
+        psum += sc[e];
+    }
+    psum += __shfl_xor(psum, 16, LLMS_WAVE);
+    psum += __shfl_xor(psum, 32, LLMS_WAVE);
+    l_run += psum;
+    const uint4 pf = make_uint4(pack_bf16(sc[0], sc[1]), pack_bf16(sc[2], sc[3]), pack_bf16(sc[4], sc[5]),
+                                pack_bf16(sc[6], sc[7]));
+#pragma unroll
+    for (int m = 0; m < DB; ++m)
+        acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[m]), as_bf16x8(pf), acc[m], 0, 0, 0);
+}
+
 template <int DB, bool SPLIT_WAVES>
-__global__ __launch_bounds__(SPLIT_WAVES ? 512 : 256) void attn_mfma_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(SPLIT_WAVES && DB <= 10 ? 512 : 256) void attn_mfma_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
     constexpr int KS = (D + 31) / 32;  // k-steps of the score product
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
@@ -120,9 +190,12 @@ __global__ __launch_bounds__(SPLIT_WAVES ? 512 : 256) void attn_mfma_kernel(cons
     float m_run = -INFINITY, l_run = 0.f;
 
     const int* table = a.block_tables + (size_t)(a.table_rows ? a.table_rows[b] : b) * a.max_blocks;
-    const size_t page_stride = (size_t)a.n_kv_heads * a.block_size * D;
+    const uint32_t page_stride = (uint32_t)a.n_kv_heads * a.block_size * D;
     const bf16* k_base = a.k_pool + (size_t)kvh * a.block_size * D;
     const bf16* v_base = a.v_pool + (size_t)kvh * a.block_size * D;
+    const float scale_log2 = a.scale * 1.44269504088896341f;
+    // first and last tile whose 32 keys every column of the group sees
+    const int lo_max = (a.window > 0 && p_max - a.window + 1 > 0) ? p_max - a.window + 1 : 0;
 
     int t_begin = 0, t_end = n_tiles, t_step = 1;
     if (SPLIT_WAVES) {
@@ -155,7 +228,7 @@ __global__ __launch_bounds__(SPLIT_WAVES ? 512 : 256) void attn_mfma_kernel(cons
             const int key = min(j0 + 8 * (col / 4) + 4 * u + (col % 4), p_max);  // `col` is the row index i here
             const int blk = block_of(key);
             const int page = __shfl(pages_reg, blk - blk_base, LLMS_WAVE);
-            const bf16* krow = k_base + (size_t)page * page_stride + (size_t)(key - blk * a.block_size) * D;
+            const bf16* krow = page_ptr(k_base, page, page_stride) + (uint32_t)((key - blk * a.block_size) * D);
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
                 const int d = 32 * s + 8 * g;
@@ -165,9 +238,9 @@ __global__ __launch_bounds__(SPLIT_WAVES ? 512 : 256) void attn_mfma_kernel(cons
         const int jk = min(j0 + 8 * g, p_max & ~7);
         const int blk = block_of(jk);
         const int page = __shfl(pages_reg, blk - blk_base, LLMS_WAVE);
-        const bf16* vrow = v_base + (size_t)page * page_stride + (jk - blk * a.block_size);
+        const bf16* vrow = page_ptr(v_base, page, page_stride) + (uint32_t)(jk - blk * a.block_size + col * a.block_size);
 #pragma unroll
-        for (int m = 0; m < DB; ++m) vf[m] = *reinterpret_cast<const uint4*>(vrow + (size_t)(16 * m + col) * a.block_size);
+        for (int m = 0; m < DB; ++m) vf[m] = *reinterpret_cast<const uint4*>(vrow + (uint32_t)(16 * m * a.block_size));
     };
 
     // the next tile's operands are requested before this tile's arithmetic starts
@@ -186,54 +259,15 @@ __global__ __launch_bounds__(SPLIT_WAVES ? 512 : 256) void attn_mfma_kernel(cons
 #pragma unroll
         for (int m = 0; m < DB; ++m) vf[m] = vf_next[m];
         if (t + t_step < t_end) load_tile(j_begin + 32 * (t + t_step), kf_next, vf_next);
-        f32x4 s_acc[2];
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            s_acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < KS; ++s) {
-                // (queries beyond head_dim are zero, so a key chunk loaded from a clamped address adds nothing)
-                s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u][s]), as_bf16x8(qf[s]), s_acc[u], 0, 0, 0);
-            }
-        }
+        // (queries beyond head_dim are zero, so a key chunk loaded from a clamped address adds nothing)
         const int jk = j0 + 8 * g;
-        {
+        if (j0 >= lo_max && j0 + 31 <= p_min) {  // (uniform over the wave; columns without a token are discarded)
+            attend_tile<DB, KS, false>(acc, m_run, l_run, kf, vf, qf, jk, lo_col, p_col, scale_log2);
+        } else {
             const int first = lo_min - jk, last = p_max + 1 - jk;
 #pragma unroll
             for (int m = 0; m < DB; ++m) vf[m] = keep_elements(vf[m], first, last);
-        }
-        // ---- online softmax of this lane's column over its 8 keys (and the 3 other lane groups)
-        float sc[8];
-        float tmax = -INFINITY;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int key = jk + e;
-            const bool ok = key >= lo_col && key <= p_col;
-            sc[e] = ok ? s_acc[e / 4][e % 4] * a.scale : -INFINITY;
-            tmax = fmaxf(tmax, sc[e]);
-        }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, LLMS_WAVE));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, LLMS_WAVE));
-        const float m_new = fmaxf(m_run, tmax);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = __expf(m_run - m_safe);
-        float psum = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            sc[e] = __expf(sc[e] - m_safe);
-            psum += sc[e];
-        }
-        psum += __shfl_xor(psum, 16, LLMS_WAVE);
-        psum += __shfl_xor(psum, 32, LLMS_WAVE);
-        l_run = l_run * corr + psum;
-        m_run = m_new;
-        const uint4 pf = make_uint4(pack_bf16(sc[0], sc[1]), pack_bf16(sc[2], sc[3]), pack_bf16(sc[4], sc[5]),
-                                    pack_bf16(sc[6], sc[7]));
-#pragma unroll
-        for (int m = 0; m < DB; ++m) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[m][r] *= corr;
-            acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[m]), as_bf16x8(pf), acc[m], 0, 0, 0);
+            attend_tile<DB, KS, true>(acc, m_run, l_run, kf, vf, qf, jk, lo_col, p_col, scale_log2);
         }
     }
 
@@ -271,7 +305,7 @@ __global__ __launch_bounds__(SPLIT_WAVES ? 512 : 256) void attn_mfma_kernel(cons
                 const float m_old = sh_m[col], l_old = sh_l[col];
                 const float m_tot = fmaxf(m_old, m_run);
                 const float m_safe = (m_tot == -INFINITY) ? 0.f : m_tot;
-                const float wa = __expf(m_old - m_safe), wb = __expf(m_run - m_safe);
+                const float wa = exp2_fast(m_old - m_safe), wb = exp2_fast(m_run - m_safe);
 #pragma unroll
                 for (int m = 0; m < DB; ++m)
 #pragma unroll
@@ -311,6 +345,165 @@ __global__ __launch_bounds__(SPLIT_WAVES ? 512 : 256) void attn_mfma_kernel(cons
     }
 }
 
+// Prompt portions, 4 consecutive column groups of one request and KV head per workgroup.  The 4 waves walk the
+// same keys, so each tile of 32 keys is fetched once per workgroup: every thread brings a 16-byte piece of the key
+// rows and of the (page-transposed) value rows into LDS, double-buffered, and the waves read their matrix operands
+// from there.  Key rows are stored in the order the score product wants them (row 16u + i holds key 8*(i/4) + 4u + i%4,
+// padded by one chunk per row against bank conflicts); values keep their [dimension][key] order.
+template <int DB>
+__global__ __launch_bounds__(256) void attn_prompt_kernel(const AttnArgs a) {
+    constexpr int D = DB * 16;
+    constexpr int KS = (D + 31) / 32;
+    constexpr int KCH = D / 8;          // 16-byte chunks of a key row
+    constexpr int KROW = KCH + 1;       // padded row stride in chunks
+    constexpr int PIECES = 4 * D;       // chunks of the key tile (32 x KCH) = chunks of the value tile (D x 4)
+    constexpr int PER_THREAD = (PIECES + 255) / 256;
+    __shared__ uint4 k_lds[2][32 * KROW];
+    __shared__ uint4 v_lds[2][D * 4];
+    const int tid = threadIdx.x, wave = tid / LLMS_WAVE, lane = tid % LLMS_WAVE;
+    const int col = lane % 16, g = lane / 16;
+
+    const int G = a.n_heads / a.n_kv_heads;
+    const int HG = G < 16 ? G : 16, TPG = 16 / HG, HB = (G + HG - 1) / HG;
+    const int kvh = blockIdx.y / HB, hb = blockIdx.y % HB;
+    const int b = a.seq_begin + blockIdx.z;
+    const int tok0 = a.cu_seqlens[b], n_new = a.cu_seqlens[b + 1] - tok0;
+    const int ctx = a.context_lens[b];
+    const int wg_first = blockIdx.x * 4 * TPG;  // first token of the workgroup within the request's new tokens
+    if (wg_first >= n_new || ctx <= 0) return;
+
+    const int t_first = wg_first + wave * TPG;
+    const int c_tok = t_first + col / HG, c_head_in = hb * HG + col % HG;
+    const bool col_ok = col < HG * TPG && c_tok < n_new && c_head_in < G;
+    const int head = kvh * G + c_head_in;
+    const int p_col = col_ok ? ctx - n_new + c_tok : -1;
+    const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
+    // key range of the whole workgroup
+    const int p_max = ctx - n_new + min(wg_first + 4 * TPG, n_new) - 1;
+    const int p_min = ctx - n_new + wg_first;
+    const int lo_min = (a.window > 0 && p_min - a.window + 1 > 0) ? p_min - a.window + 1 : 0;
+    const int j_begin = lo_min & ~31;
+    const int n_tiles = (p_max - j_begin) / 32 + 1;
+
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    uint4 qf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int d = 32 * s + 8 * g;
+        qf[s] = (col_ok && d < D)
+                    ? *reinterpret_cast<const uint4*>(a.q + (size_t)(tok0 + c_tok) * a.q_stride + (size_t)head * D + d)
+                    : zero;
+    }
+    f32x4 acc[DB];
+#pragma unroll
+    for (int m = 0; m < DB; ++m) acc[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    const int* table = a.block_tables + (size_t)(a.table_rows ? a.table_rows[b] : b) * a.max_blocks;
+    const uint32_t page_stride = (uint32_t)a.n_kv_heads * a.block_size * D;
+    const bf16* k_base = a.k_pool + (size_t)kvh * a.block_size * D;
+    const bf16* v_base = a.v_pool + (size_t)kvh * a.block_size * D;
+    const float scale_log2 = a.scale * 1.44269504088896341f;
+    // the tiles whose 32 keys every column of this wave sees: up to the wave's first token, from the window's
+    // start of its last one
+    const int w_last = min(t_first + TPG, n_new) - 1;
+    const int w_pmin = ctx - n_new + t_first, w_pmax = ctx - n_new + w_last;
+    const int w_lo_max = (a.window > 0 && w_pmax - a.window + 1 > 0) ? w_pmax - a.window + 1 : 0;
+    const int bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
+    auto block_of = [&](int key) { return bs_shift >= 0 ? key >> bs_shift : key / a.block_size; };
+    const int last_blk = block_of(p_max);
+    int blk_base = 0, pages_reg = 0;
+    auto load_pages = [&](int base) {
+        blk_base = base;
+        pages_reg = table[min(base + lane, last_blk)];
+    };
+
+    // this thread's pieces of a tile: key piece c -> key c / KCH, chunk c % KCH; value piece c -> dimension c / 4,
+    // keys 8*(c % 4) .. +7.  Addresses are clamped to the last key of the workgroup (which exists); value pieces
+    // are zeroed outside [lo_min, p_max] on their way into LDS (not earlier: that would wait for the load).
+    uint4 kreg[PER_THREAD], vreg[PER_THREAD];
+    auto load_tile = [&](int j0) {
+        const int blk_first = block_of(j0);
+        if (blk_first < blk_base || block_of(min(j0 + 31, p_max)) >= blk_base + LLMS_WAVE) load_pages(blk_first);
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) {
+            const int c = tid + 256 * i;
+            const bool piece_ok = c < PIECES;  // (D < 64: the upper threads have no piece)
+            {
+                const int key = min(j0 + (piece_ok ? c / KCH : 0), p_max), ch = piece_ok ? c % KCH : 0;
+                const int blk = block_of(key);
+                const int page = __shfl(pages_reg, blk - blk_base, LLMS_WAVE);
+                kreg[i] = *reinterpret_cast<const uint4*>(page_ptr(k_base, page, page_stride) +
+                                                           (uint32_t)((key - blk * a.block_size) * D + 8 * ch));
+            }
+            {
+                const int d = piece_ok ? c / 4 : 0, kc = piece_ok ? c % 4 : 0;
+                const int jk = j0 + 8 * kc, jc = min(jk, p_max & ~7);
+                const int blk = block_of(jc);
+                const int page = __shfl(pages_reg, blk - blk_base, LLMS_WAVE);
+                vreg[i] = *reinterpret_cast<const uint4*>(page_ptr(v_base, page, page_stride) +
+                                                           (uint32_t)(d * a.block_size + jc - blk * a.block_size));
+            }
+        }
+    };
+    auto store_tile = [&](int buf, int j0) {
+        const bool inside = j0 >= lo_min && j0 + 31 <= p_max;  // (uniform)
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) {
+            const int c = tid + 256 * i;
+            if (c < PIECES) {
+                if (!inside) {
+                    const int jk = j0 + 8 * (c % 4);
+                    vreg[i] = keep_elements(vreg[i], lo_min - jk, p_max + 1 - jk);
+                }
+                const int kl = c / KCH, ch = c % KCH;                    // key kl = 8a + 4u + b2 of the tile
+                const int row = ((kl >> 2) & 1) * 16 + (kl >> 3) * 4 + (kl & 3);  // -> row 16u + 4a + b2
+                k_lds[buf][row * KROW + ch] = kreg[i];
+                v_lds[buf][c] = vreg[i];                                  // [dimension][4 chunks of 8 keys]
+            }
+        }
+    };
+
+    load_pages(block_of(j_begin));
+    load_tile(j_begin);
+    store_tile(0, j_begin);
+    if (n_tiles > 1) load_tile(j_begin + 32);
+    __syncthreads();
+    for (int t = 0; t < n_tiles; ++t) {
+        const int buf = t & 1, j0 = j_begin + 32 * t;
+        uint4 kf[2][KS], vf[DB];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                const int ch = 4 * s + g;
+                kf[u][s] = k_lds[buf][(16 * u + col) * KROW + (ch < KCH ? ch : 0)];  // (beyond head_dim the queries are zero)
+            }
+#pragma unroll
+        for (int m = 0; m < DB; ++m) vf[m] = v_lds[buf][(16 * m + col) * 4 + g];
+        if (j0 >= w_lo_max && j0 + 31 <= w_pmin)  // (uniform over the wave; columns without a token are discarded)
+            attend_tile<DB, KS, false>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
+        else
+            attend_tile<DB, KS, true>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
+        if (t + 1 < n_tiles) {
+            store_tile(buf ^ 1, j0 + 32);  // last read two tiles ago, before the previous barrier
+            if (t + 2 < n_tiles) load_tile(j_begin + 32 * (t + 2));
+        }
+        __syncthreads();
+    }
+    if (col_ok) {
+        const float inv = 1.f / l_run;
+        bf16* orow = a.out + (size_t)(tok0 + c_tok) * a.out_stride + (size_t)head * D;
+#pragma unroll
+        for (int m = 0; m < DB; ++m) {
+            uint2 w;
+            w.x = pack_bf16(acc[m][0] * inv, acc[m][1] * inv);
+            w.y = pack_bf16(acc[m][2] * inv, acc[m][3] * inv);
+            *reinterpret_cast<uint2*>(orow + 16 * m + 4 * g) = w;
+        }
+    }
+}
+
 // Merge of the splits of one (token, head), split 0 first.
 __global__ void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ ws_o,
                                   const float* __restrict__ ws_ml, int token_begin, int n_heads, int head_dim,
@@ -322,17 +515,32 @@ __global__ void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const 
     float l_tot = 0.f;
     for (int s = 0; s < num_splits; ++s) {
         const float m = ws_ml[(item0 + s) * 2];
-        if (m != -INFINITY) l_tot += ws_ml[(item0 + s) * 2 + 1] * __expf(m - m_tot);
+        if (m != -INFINITY) l_tot += ws_ml[(item0 + s) * 2 + 1] * exp2_fast(m - m_tot);
     }
     const float inv = 1.f / l_tot;
     for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
         float o = 0.f;
         for (int s = 0; s < num_splits; ++s) {
             const float m = ws_ml[(item0 + s) * 2];
-            if (m != -INFINITY) o += ws_o[(item0 + s) * head_dim + d] * __expf(m - m_tot);
+            if (m != -INFINITY) o += ws_o[(item0 + s) * head_dim + d] * exp2_fast(m - m_tot);
         }
         out[(size_t)token * out_stride + (size_t)head * head_dim + d].bits = f32_to_bf16_bits(o * inv);
     }
+}
+
+static int launch_prompt(int db, dim3 grid, const AttnArgs& a, hipStream_t stream) {
+#define ATT_CASE(N)                                                  \
+    case N:                                                          \
+        attn_prompt_kernel<N><<<grid, 256, 0, stream>>>(a);          \
+        break;
+    switch (db) {
+        ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
+        ATT_CASE(9) ATT_CASE(10) ATT_CASE(11) ATT_CASE(12) ATT_CASE(13) ATT_CASE(14) ATT_CASE(15) ATT_CASE(16)
+        default:
+            LLMS_REQUIRE(false, "attention_mfma: head_dim must be a multiple of 16 up to 256");
+    }
+#undef ATT_CASE
+    return LLMS_OK;
 }
 
 template <bool SPLIT_WAVES>
@@ -354,7 +562,8 @@ static int launch_attn(int db, dim3 grid, int threads, const AttnArgs& a, hipStr
 extern "C" {
 
 // Attention for the requests [seq_begin, seq_begin + n_seqs) of a step.  max_new: most new tokens any of
-// them brings.  split_waves = 1 deals the keys of each column group to `waves` (4 or 8) waves and
+// them brings.  split_waves = 0: prompt portions (keys shared through LDS); -1: the same without LDS;
+// split_waves = 1 deals the keys of each column group to `waves` (4 or 8) waves and
 // `num_splits` workgroups (decoding); with num_splits > 1 the caller provides ws_o [tokens * heads * splits * D] and
 // ws_ml [tokens * heads * splits * 2] floats, indexed by absolute token row.
 int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
@@ -373,8 +582,11 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                      ((uintptr_t)out % 8) == 0, "attention_mfma: pointers must be 16-byte aligned");
     LLMS_REQUIRE(window >= 0 && max_blocks > 0, "attention_mfma: bad window or max_blocks");
     LLMS_REQUIRE(num_splits >= 1, "attention_mfma: num_splits must be >= 1");
-    LLMS_REQUIRE(waves == 4 || (split_waves && waves == 8), "attention_mfma: 4 waves, or 8 when the waves share the keys");
-    LLMS_REQUIRE(split_waves || num_splits == 1, "attention_mfma: splits need split_waves");
+    LLMS_REQUIRE(scale > 0.f, "attention_mfma: scale must be positive");
+    LLMS_REQUIRE((long long)n_kv_heads * block_size * head_dim < (1ll << 31), "attention_mfma: a page is too large");
+    LLMS_REQUIRE(waves == 4 || (split_waves > 0 && waves == 8), "attention_mfma: 4 waves, or 8 when the waves share the keys");
+    LLMS_REQUIRE(waves == 4 || head_dim <= 160, "attention_mfma: 8 waves take head_dim up to 160");
+    LLMS_REQUIRE(split_waves > 0 || num_splits == 1, "attention_mfma: splits need split_waves");
     LLMS_REQUIRE(num_splits == 1 || (ws_o && ws_ml), "attention_mfma: splits need a workspace");
     LLMS_REQUIRE(n_seqs <= 65535, "attention_mfma: too many requests for one launch");
     const int G = n_heads / n_kv_heads, HG = G < 16 ? G : 16, TPG = 16 / HG, HB = (G + HG - 1) / HG;
@@ -383,7 +595,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                   block_tables, table_rows, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
                   window, scale, num_splits, ws_o, ws_ml};
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
-    if (split_waves) {
+    if (split_waves > 0) {
         dim3 grid(groups * num_splits, n_kv_heads * HB, n_seqs);
         if (int e = launch_attn<true>(head_dim / 16, grid, waves * LLMS_WAVE, a, stream)) return e;
         if (num_splits > 1) {
@@ -397,7 +609,11 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
         }
     } else {
         dim3 grid((groups + 3) / 4, n_kv_heads * HB, n_seqs);
-        if (int e = launch_attn<false>(head_dim / 16, grid, 256, a, stream)) return e;
+        if (split_waves < 0) {  // the variant that reads every operand straight from global memory
+            if (int e = launch_attn<false>(head_dim / 16, grid, 256, a, stream)) return e;
+        } else {
+            if (int e = launch_prompt(head_dim / 16, grid, a, stream)) return e;
+        }
     }
     LLMS_LAUNCH_CHECK();
 }

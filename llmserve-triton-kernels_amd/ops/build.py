@@ -26,10 +26,13 @@ CSRC_DIR = PACKAGE_DIR / "csrc"
 LIB_DIR = PACKAGE_DIR / "lib"
 
 ARCH = "gfx950"
-# The target feature packed-fp32-ops is switched off for all device code.
+# The target feature packed-fp32-ops is switched off for all device code.  Matrix instructions keep
+# their accumulators in ordinary vector registers: the kernels here rescale and convert them between
+# products, and the other register file would cost a copy each way.
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-result", "-Wno-unknown-warning-option",
 ]
 

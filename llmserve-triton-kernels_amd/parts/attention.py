@@ -147,8 +147,9 @@ class Attention(Mixer):
         g = self.num_heads // self.num_kv_heads
         groups = n_requests * self.num_kv_heads * -(-g // 16)
         reach = min(max_context, self.window) if self.window else max_context
+        waves = 8 if self.head_dim <= 160 else 4  # (8 waves of wider heads would not fit the registers)
         if groups >= 256:
-            return 1, 8
+            return 1, waves
         tiles = -(-reach // 32)
-        splits = max(1, min(256 // groups, -(-tiles // 32)))
-        return splits, 8
+        splits = max(1, min(256 // groups, -(-tiles // (4 * waves))))
+        return splits, waves
