@@ -30,6 +30,15 @@
         return LLMS_OK;                                                \
     } while (0)
 
+#define LLMS_HIP_CHECK(call)                                           \
+    do {                                                               \
+        hipError_t e_ = (call);                                        \
+        if (e_ != hipSuccess) {                                        \
+            fprintf(stderr, "llmserve kernel set-up failed: %s\n", hipGetErrorString(e_)); \
+            return LLMS_ERR_LAUNCH;                                    \
+        }                                                              \
+    } while (0)
+
 // bfloat16 is carried as its 16 raw bits.
 struct bf16 {
     uint16_t bits;

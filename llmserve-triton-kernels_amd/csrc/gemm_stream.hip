@@ -14,7 +14,9 @@
 // Because a launch costs more than most of these products take, what surrounds the product is fused in:
 //   NORM      prologue: x = bf16(residual + delta) (written to resid_out by workgroup 0), then
 //             h = weight_n * bf16(x * rsqrt(mean(x^2) + eps)): the RMSNorm kernel's rounding points
-//             (src/llmserve/model/llama.py:24-28).  Each workgroup computes the row statistics itself.
+//             (src/llmserve/model/llama.py:24-28).  Every workgroup does this for all rows itself, a wave per
+//             pair of rows with coalesced loads, while its first weights are in flight; the normed rows
+//             wait in LDS (dynamic, rows x (K/8 + 1) chunks) for the matrix instructions.
 //   SWIGLU    the 16 rows are 8 gate rows and the 8 up rows of the same features; the epilogue writes
 //             bf16(bf16(silu(bf16(gate))) * bf16(up)) (src/llmserve/model/llama.py:120).
 //   ROPE_QKV  the 16 rows are 8 rows of one head and their 8 rotary partners (i, i + D/2); the epilogue
@@ -144,48 +146,67 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
 
     const bool m_ok = m0 + r16 < M;
     const bf16* xrow = a.X + (size_t)(m_ok ? m0 + r16 : 0) * a.ldx;
-    const bf16* drow = (NORM && a.delta) ? a.delta + (size_t)(m_ok ? m0 + r16 : 0) * a.ldx : nullptr;
-    // x chunk of 8 at column k of this lane's row: the residual sum in 32-bit, rounded once
-    auto load_x = [&](int k) -> uint4 {
-        uint4 v = *reinterpret_cast<const uint4*>(xrow + k);
-        if (NORM && drow) {
-            float xf[8], df[8];
-            unpack8(v, xf);
-            unpack8(*reinterpret_cast<const uint4*>(drow + k), df);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) xf[e] += df[e];
-            v = pack8(xf);
-        }
-        return v;
-    };
 
-    float inv_rms = 0.f;
+    // ---- NORM: summed residual, statistics and normed rows, kept in LDS as h[row][K/8 + 1] chunks of 8
+    extern __shared__ uint4 h_lds[];
+    const int hstride = K / 8 + 1;  // (one chunk of padding: the 16 rows of a matrix operand fall into different banks)
     if (NORM) {
-        float ss = 0.f;
-        for (int c = wave; c < chunks; c += ST_WAVES) {
+        // a wave takes the rows wave, wave + 4, ..., two at a time so that their loads are in flight together;
+        // a lane norms the chunks it summed itself, so nothing but the end needs a barrier
+        for (int ma = wave; ma < M; ma += 2 * ST_WAVES) {
+            const int rows[2] = {ma, ma + ST_WAVES};
+            const int nrows = rows[1] < M ? 2 : 1;
+            float ss[2] = {0.f, 0.f};
 #pragma unroll 4
-            for (int s = 0; s < 16; ++s) {
-                const int k = c * ST_KC + 32 * s + 8 * g;
-                if (m_ok && k < K) {
-                    const uint4 v = load_x(k);
-                    float xf[8];
-                    unpack8(v, xf);
+            for (int c8 = lane; c8 < K / 8; c8 += LLMS_WAVE) {
+                uint4 v[2], d[2];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) ss += xf[e] * xf[e];
-                    if (a.resid_out && tile_id == 0) *reinterpret_cast<uint4*>(a.resid_out + (size_t)(m0 + r16) * a.ldx + k) = v;
+                for (int j = 0; j < 2; ++j) {
+                    if (j < nrows) {
+                        v[j] = *reinterpret_cast<const uint4*>(a.X + (size_t)rows[j] * a.ldx + 8 * c8);
+                        if (a.delta) d[j] = *reinterpret_cast<const uint4*>(a.delta + (size_t)rows[j] * a.ldx + 8 * c8);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    if (j < nrows) {
+                        float xf[8];
+                        unpack8(v[j], xf);
+                        if (a.delta) {  // the residual sum in 32-bit, rounded once
+                            float df[8];
+                            unpack8(d[j], df);
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) xf[e] = bfr(xf[e] + df[e]);
+                            v[j] = pack8(xf);
+                            if (a.resid_out && tile_id == 0)
+                                *reinterpret_cast<uint4*>(a.resid_out + (size_t)rows[j] * a.ldx + 8 * c8) = v[j];
+                        }
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) ss[j] += xf[e] * xf[e];
+                        h_lds[rows[j] * hstride + c8] = v[j];
+                    }
+                }
+            }
+            float inv_rms[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) inv_rms[j] = rsqrtf(wave_sum(ss[j]) / (float)K + a.eps);
+#pragma unroll 2
+            for (int c8 = lane; c8 < K / 8; c8 += LLMS_WAVE) {
+                float wf[8];
+                unpack8(*reinterpret_cast<const uint4*>(a.norm_w + 8 * c8), wf);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    if (j < nrows) {
+                        float xf[8];
+                        unpack8(h_lds[rows[j] * hstride + c8], xf);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) xf[e] = wf[e] * bfr(xf[e] * inv_rms[j]);
+                        h_lds[rows[j] * hstride + c8] = pack8(xf);
+                    }
                 }
             }
         }
-        ss += __shfl_xor(ss, 16, LLMS_WAVE);
-        ss += __shfl_xor(ss, 32, LLMS_WAVE);
-        float* ss_lds = reinterpret_cast<float*>(lds);  // [wave][16]; the tiles are not in use yet
-        if (g == 0) ss_lds[wave * 16 + r16] = ss;
-        __syncthreads();
-        float total = 0.f;
-#pragma unroll
-        for (int w = 0; w < ST_WAVES; ++w) total += ss_lds[w * 16 + r16];
-        inv_rms = rsqrtf(total / (float)K + a.eps);
-        __syncthreads();  // all have read the sums before wave 0's tile overwrites them
+        __syncthreads();  // the normed rows are complete
     }
 
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -195,20 +216,10 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
 #pragma unroll
         for (int s = 0; s < 16; ++s) {
             const int k = k0 + 32 * s + 8 * g;
-            if (m_ok && k < K) {
-                uint4 v = load_x(k);
-                if (NORM) {
-                    float xf[8], wf[8];
-                    unpack8(v, xf);
-                    unpack8(*reinterpret_cast<const uint4*>(a.norm_w + k), wf);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) xf[e] = wf[e] * bfr(xf[e] * inv_rms);
-                    v = pack8(xf);
-                }
-                xreg[s] = v;
-            } else {
+            if (m_ok && k < K)
+                xreg[s] = NORM ? h_lds[r16 * hstride + k / 8] : *reinterpret_cast<const uint4*>(xrow + k);
+            else
                 xreg[s] = zero;
-            }
         }
 #pragma unroll
         for (int i = 0; i < 16; ++i) tile[i * (ST_KC / 8) + (lane ^ i)] = wreg[i];
@@ -295,12 +306,23 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     }
 }
 
+#define ST_NORM_LDS_MAX (96 * 1024)  // beside the 64 KB of weight tiles, of the 160 KB a workgroup may hold
+
 template <typename TOut, int EPI>
-static void launch_stream(bool norm, unsigned grid, const StreamArgs& a, hipStream_t stream) {
-    if (norm)
-        gemm_stream_kernel<TOut, EPI, true><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(a);
-    else
+static int launch_stream(bool norm, unsigned grid, const StreamArgs& a, hipStream_t stream) {
+    if (norm) {
+        static bool raised = false;  // (per instantiation) allow more dynamic LDS than the default limit
+        if (!raised) {
+            LLMS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<TOut, EPI, true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, ST_NORM_LDS_MAX));
+            raised = true;
+        }
+        const size_t h_bytes = (size_t)a.M * (a.K / 8 + 1) * 16;
+        gemm_stream_kernel<TOut, EPI, true><<<grid, ST_WAVES * LLMS_WAVE, h_bytes, stream>>>(a);
+    } else {
         gemm_stream_kernel<TOut, EPI, false><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(a);
+    }
+    return LLMS_OK;
 }
 
 extern "C" {
@@ -315,7 +337,8 @@ int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* 
                      const float* inv_freq, const int* positions, const int* slots, void* k_pool, void* v_pool,
                      hipStream_t stream) {
     LLMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_stream: needs 1 <= M <= 64 and positive sizes");
-    LLMS_REQUIRE(norm_w == nullptr || M <= 16, "gemm_stream: the norm prologue takes at most 16 rows");
+    LLMS_REQUIRE(norm_w == nullptr || (M <= 16 && (size_t)M * (K / 8 + 1) * 16 <= ST_NORM_LDS_MAX),
+                 "gemm_stream: the norm prologue takes at most 16 rows and rows * (K + 8) * 2 bytes up to 96 KB");
     LLMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "gemm_stream: K and the row stride of X must be multiples of 8");
     LLMS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_stream: X and W must be 16-byte aligned");
     LLMS_REQUIRE(C != nullptr && (out_dtype == 0 || out_dtype == 1), "gemm_stream: bad output");
@@ -349,9 +372,10 @@ int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* 
     a.num_tiles = (int)grid;
     grid = ((grid + 7) / 8) * 8 * ((M + 15) / 16);  // every XCD gets whole tiles with all their row blocks
     const bool norm = norm_w != nullptr;
-#define ST_EPI(E)                                                                  \
-    if (out_dtype == 0) launch_stream<float, E>(norm, grid, a, stream);           \
-    else launch_stream<bf16, E>(norm, grid, a, stream);
+#define ST_EPI(E)                                                                                  \
+    if (int e = out_dtype == 0 ? launch_stream<float, E>(norm, grid, a, stream)                    \
+                               : launch_stream<bf16, E>(norm, grid, a, stream))                    \
+        return e;
     if (epilogue == EPI_PLAIN) { ST_EPI(EPI_PLAIN) }
     else if (epilogue == EPI_SWIGLU) { ST_EPI(EPI_SWIGLU) }
     else { ST_EPI(EPI_ROPE_QKV) }

@@ -300,6 +300,10 @@ def gemm_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.T
     return out
 
 
+STREAM_NORM_ROWS = 16  # what gemm_stream's norm prologue takes: rows, and bytes of LDS for them
+STREAM_NORM_LDS_BYTES = 96 * 1024
+
+
 def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, *,
                 norm: tuple | None = None, swiglu: bool = False, rope: dict | None = None) -> torch.Tensor:
     """The product for up to 64 bfloat16 rows (built for up to 16), with what surrounds it fused in.
@@ -320,8 +324,8 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
     n = w.shape[0]
     if not 0 < m <= 64:
         raise ValueError("gemm_stream takes 1..64 rows")
-    if norm is not None and m > 16:
-        raise ValueError("the norm prologue takes at most 16 rows")
+    if norm is not None and (m > STREAM_NORM_ROWS or m * (k // 8 + 1) * 16 > STREAM_NORM_LDS_BYTES):
+        raise ValueError("the norm prologue takes at most 16 rows, and rows * (K + 8) * 2 bytes up to 96 KB")
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or out.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("gemm_stream takes bfloat16 operands and stores bfloat16 or float32")
     if not gemm_bf16_supported(x, w):

@@ -16,7 +16,7 @@ import math
 import torch
 
 from ..ops import library as ops
-from .linear import FUSE_NORM_INTO_PRODUCT, STREAM_ROWS, few_rows, linear
+from .linear import few_rows, linear, norm_fusable
 from .registry import POSITION_ENCODINGS, DeferredNorm, Mixer, register_mixer
 from .rmsnorm import RMSNorm
 from .spec import PagedCacheSpec, ParamInfo
@@ -96,12 +96,12 @@ class Attention(Mixer):
         """With few bfloat16 rows one kernel does the projection, the rotation and the cache store (and,
         if switched on, the residual sum and the norm before them): ops.gemm_stream.  Returns the rotated
         queries, or None when that kernel does not apply."""
-        if isinstance(x, DeferredNorm) and not FUSE_NORM_INTO_PRODUCT:
+        if isinstance(x, DeferredNorm) and not (norm_fusable(*x.residual.shape) and isinstance(x.norm, RMSNorm)):
             return None if self._few_rows_unfit(x.residual) else self.project_few_rows(x.materialize(), batch, cache, slots)
         deferred = isinstance(x, DeferredNorm)
         rows = x.residual if deferred else x
         m = rows.shape[0]
-        if self._few_rows_unfit(rows) or (deferred and (m > STREAM_ROWS or not isinstance(x.norm, RMSNorm))):
+        if self._few_rows_unfit(rows):
             return None
         frequencies = getattr(self.position, "rotary_frequencies", None)
         if frequencies is None and not getattr(self.position, "identity", False):

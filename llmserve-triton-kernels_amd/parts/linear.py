@@ -40,10 +40,16 @@ def few_rows(m: int, weight: torch.Tensor) -> bool:
     return m <= STREAM_MAX_ROWS and -(-m // 16) * weight.numel() * 2 <= STREAM_REREAD_BYTES
 
 # Whether the few-row product also does the residual sum and the norm in front of it
-# (ops.gemm_stream(norm=...)).  Off: every workgroup repeats the statistics and the rounding of its
-# rows with most lanes idle, which measured slower (TinyLlama shape, batch 1: 2.7 ms against
-# 1.4 ms a step) than the norm as a kernel of its own.
-FUSE_NORM_INTO_PRODUCT = False
+# (ops.gemm_stream(norm=...)): every workgroup norms the rows itself while its first weights are in
+# flight.  Off by default: it saves the norm kernel, but the rows in LDS leave room for one workgroup
+# per CU instead of two, and the prologue is repeated by hundreds of workgroups.  Measured on the
+# TinyLlama shape: 864 against 898 tokens a second at batch 1, 5,310 against 6,302 at batch 8.
+FUSE_NORM_INTO_PRODUCT = os.environ.get("LLMSERVE_FUSE_NORM", "0") == "1"
+
+
+def norm_fusable(m: int, k: int) -> bool:
+    """Whether ops.gemm_stream's norm prologue takes m rows of k elements (they wait in LDS)."""
+    return FUSE_NORM_INTO_PRODUCT and 0 < m <= ops.STREAM_NORM_ROWS and m * (k // 8 + 1) * 16 <= ops.STREAM_NORM_LDS_BYTES
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,

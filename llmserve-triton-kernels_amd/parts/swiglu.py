@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .linear import FUSE_NORM_INTO_PRODUCT, STREAM_ROWS, few_rows, linear
+from .linear import few_rows, linear, norm_fusable
 from .registry import DeferredNorm, FeedForward, register_feed_forward
 from .rmsnorm import RMSNorm
 from .spec import ParamInfo
@@ -44,7 +44,7 @@ class SwiGLU(FeedForward):
         few = dtype == torch.bfloat16 and few_rows(m, self.gate_up) and self.intermediate % 8 == 0
         if isinstance(x, DeferredNorm):
             norm = x.norm
-            if (FUSE_NORM_INTO_PRODUCT and few and m <= STREAM_ROWS and isinstance(norm, RMSNorm)
+            if (few and norm_fusable(m, x.residual.shape[1]) and isinstance(norm, RMSNorm)
                     and ops.gemm_bf16_supported(x.residual, self.gate_up)):
                 new_residual = torch.empty_like(x.residual) if x.delta is not None else None
                 ops.gemm_stream(act, x.residual, self.gate_up, norm=(x.delta, norm.weight, norm.eps, new_residual),
