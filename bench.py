@@ -6,8 +6,20 @@ weights, bfloat16.
 Prints one JSON line.  `value` is decoded tokens per second at the default batch: K timed
 scheduler steps (step function + sampling + the read-back of the token ids) after W untimed
 ones, with synchronisation on both sides.  `prefill` is one request of 2,048 tokens in one
-step; `roofline` prices the decode step against HBM bandwidth (every weight it uses read
-once, plus the keys and values of the live requests); `points` holds decode at batch 1 and 64.
+step (`chunked`: the same prompt in portions of 512 tokens, the scheduler cutting it);
+`roofline` prices the decode step against HBM bandwidth (every weight it uses read once, plus
+the keys and values of the live requests); `points` holds decode at batch 1 and 64;
+`measured_peaks` is what this box delivers to a plain device copy and to a large library
+matrix product, the practical ceilings beside the published ones.
+
+    python bench.py --workload serve [--model llama2-7b] [--requests 64] [--new-tokens 256]
+                    [--prompt-min 128] [--prompt-max 2048] [--pages-fraction 1.0]
+
+runs the other workload: continuous batching of requests with seeded random prompt lengths,
+all arriving at once; `value` is generated tokens per second over the whole run, with time to
+first token, inter-token latency percentiles and the number of preemptions beside it.
+`--pages-fraction` shrinks the cache pool below what the whole workload needs, so that
+requests wait and are preempted.
 """
 
 from __future__ import annotations
@@ -25,6 +37,102 @@ if ROOT not in sys.path:
 HBM_PEAK = 8.0e12  # bytes/s, MI355X
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}  # dense matrix-core peaks, MI355X
 PREFILL_TOKENS = 2048
+PREFILL_CHUNK = 512  # the portion size of the chunked prefill measurement
+
+
+def measured_peaks(torch) -> dict:
+    """What the box delivers: a device-to-device copy of 1 GiB (read + write counted) and a
+    bfloat16 library product of 8192^3."""
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    copy_s = timed(lambda: dst.copy_(src), 10)
+    a = torch.randn(8192, 8192, device="cuda").bfloat16()
+    b = torch.randn(8192, 8192, device="cuda").bfloat16()
+    mm_s = timed(lambda: torch.mm(a, b.t()), 10)
+    return {"copy_GBps": round(2 * src.numel() / copy_s / 1e9, 1), "gemm_bf16_TFLOPs": round(2 * 8192 ** 3 / mm_s / 1e12, 1)}
+
+
+def percentile(values, q):
+    values = sorted(values)
+    if not values:
+        return 0.0
+    return values[min(len(values) - 1, int(q * len(values)))]
+
+
+def serve(args) -> int:
+    """Continuous batching of --requests requests that all arrive at time 0."""
+    import torch
+
+    from llmserve import EngineConfig, SamplingParams
+    from llmserve.config import preset
+    from llmserve.engine.runner import ModelRunner
+    from llmserve.engine.scheduler import ContinuousBatchingEngine
+    from llmserve.sampling import Sampler
+
+    cfg = preset(args.model)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    layers = cfg["num_hidden_layers"]
+    vocab = cfg["vocab_size"]
+    block_size = 16
+    gen = torch.Generator().manual_seed(0)
+    lengths = torch.randint(args.prompt_min, args.prompt_max + 1, (args.requests,), generator=gen).tolist()
+    lo = min(100, vocab // 4)
+    prompts = [torch.randint(lo, vocab, (n,), generator=gen).tolist() for n in lengths]
+    longest = max(lengths) + args.new_tokens + 1
+    cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], longest)
+    need = sum(-(-(n + args.new_tokens + 1) // block_size) + 1 for n in lengths)
+    pages = max(int(need * args.pages_fraction), -(-longest // block_size) + 2) + 1
+    engine_cfg = EngineConfig(dtype=args.dtype, block_size=block_size, num_blocks=pages, max_num_seqs=args.requests,
+                              max_num_batched_tokens=args.budget, seed=0)
+    runner = ModelRunner.from_random(cfg, seed=0, engine_config=engine_cfg)
+    sampler = Sampler(runner.device)
+
+    def run(n_requests, new_tokens):
+        eng = ContinuousBatchingEngine(runner, sampler, max_num_seqs=args.requests, max_num_batched_tokens=args.budget)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ids = [eng.add_request(p, SamplingParams(max_new_tokens=new_tokens), arrival_time=t0) for p in prompts[:n_requests]]
+        steps = 0
+        while eng.has_unfinished():
+            eng.step()
+            steps += 1
+        torch.cuda.synchronize()
+        return eng, [eng.finished[i] for i in ids], time.perf_counter() - t0, steps
+
+    run(min(4, args.requests), 8)  # warm-up: kernels loaded, graphs of the small batches captured
+    eng, reqs, total_s, steps = run(args.requests, args.new_tokens)
+    generated = sum(len(r.generated) for r in reqs)
+    ttft = [r.token_times[0] - r.arrival_time for r in reqs]
+    itl = [b - a for r in reqs for a, b in zip(r.token_times, r.token_times[1:])]
+    line = {
+        "metric": "continuous batching: generated tok/s over the whole run",
+        "value": round(generated / total_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+        "ms_per_step": round(total_s / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": args.model, "requests": args.requests, "prompt_min": args.prompt_min,
+                   "prompt_max": args.prompt_max, "prompt_tokens": sum(lengths), "new_tokens": args.new_tokens,
+                   "parallelism": "single-gpu", "layers": layers, "layers_full": full_layers, "budget": args.budget,
+                   "pages": pages, "pages_needed": need, "block_size": block_size, "weights": "random"},
+        "total_s": round(total_s, 3),
+        "ttft_ms": {"p50": round(percentile(ttft, 0.5) * 1e3, 2), "p90": round(percentile(ttft, 0.9) * 1e3, 2),
+                    "max": round(max(ttft) * 1e3, 2)},
+        "itl_ms": {"p50": round(percentile(itl, 0.5) * 1e3, 3), "p90": round(percentile(itl, 0.9) * 1e3, 3),
+                   "p99": round(percentile(itl, 0.99) * 1e3, 3), "max": round(max(itl) * 1e3, 3)},
+        "preemptions": eng.stats.preemptions,
+    }
+    print(json.dumps(line))
+    return 0
 
 
 def main() -> int:
@@ -37,13 +145,23 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--model", default="tinyllama-1.1b")
-    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--no-points", action="store_true", help="skip the further batch sizes")
+    ap.add_argument("--points", default="1,64", help="further batch sizes to measure decoding at")
     ap.add_argument("--phase", choices=["all", "decode", "prefill"], default="all",
                     help="run one phase only (for profiles; the line then holds zeros for the other)")
+    ap.add_argument("--workload", choices=["steps", "serve"], default="steps")
+    ap.add_argument("--requests", type=int, default=64)
+    ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--prompt-min", type=int, default=128)
+    ap.add_argument("--prompt-max", type=int, default=2048)
+    ap.add_argument("--pages-fraction", type=float, default=1.0)
+    ap.add_argument("--budget", type=int, default=2048, help="serve: tokens per step (max_num_batched_tokens)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2
+    if args.workload == "serve":
+        return serve(args)
 
     import torch
 
@@ -63,7 +181,8 @@ def main() -> int:
     d = h // nh
     elem = 2 if args.dtype == "bfloat16" else 4
     block_size = 16
-    max_batch = 64 if not args.no_points and args.phase == "all" else args.batch
+    point_batches = [int(b) for b in args.points.split(",") if b] if not args.no_points and args.phase == "all" else []
+    max_batch = max([args.batch] + point_batches)
     budget = max(PREFILL_TOKENS, max_batch)
     # requests whose prompt went in first decode while the others' prompts still go in
     slack = -(-max_batch * args.context // budget) + 2
@@ -86,7 +205,7 @@ def main() -> int:
                                        max_num_batched_tokens=engine_cfg.max_num_batched_tokens)
         for p in prompts(batch, args.context):
             eng.add_request(p, SamplingParams(max_new_tokens=new_tokens))
-        while eng.waiting or any(len(r.all_ids) - r.num_computed_tokens > 1 for r in eng.running):
+        while eng.waiting or any(r.num_tokens - r.num_computed_tokens > 1 for r in eng.running):
             eng.step()  # prompts in
         for _ in range(args.warmup):
             eng.step()
@@ -100,24 +219,26 @@ def main() -> int:
         eng.run_until_complete()
         return batch * args.steps / dt, dt / args.steps
 
-    def prefill_time():
-        eng = ContinuousBatchingEngine(runner, sampler, max_num_seqs=1, max_num_batched_tokens=PREFILL_TOKENS)
+    def prefill_time(budget=PREFILL_TOKENS):
+        eng = ContinuousBatchingEngine(runner, sampler, max_num_seqs=1, max_num_batched_tokens=budget)
         times = []
         for i in range(4):
             eng.add_request(prompts(1, PREFILL_TOKENS)[0], SamplingParams(max_new_tokens=1))
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            eng.step()  # the whole prompt in one step, first token sampled and read back
+            while eng.has_unfinished():
+                eng.step()  # the whole prompt in one step (or in portions of `budget`), first token sampled and read back
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t0)
-            assert not eng.has_unfinished()
         return sorted(times[1:])[len(times[1:]) // 2]
 
     value, step_s = decode_rate(args.batch) if args.phase != "prefill" else (0.0, float("inf"))
     points = {}
-    if not args.no_points and args.phase == "all":
-        points = {"decode_b1": round(decode_rate(1)[0], 1), "decode_b64": round(decode_rate(64)[0], 1)}
+    for b in point_batches:
+        points[f"decode_b{b}"] = round(decode_rate(b)[0], 1)
     pre_s = prefill_time() if args.phase != "decode" else float("inf")
+    chunked_s = prefill_time(PREFILL_CHUNK) if args.phase == "all" else float("inf")
+    peaks = measured_peaks(torch) if args.phase == "all" else {}
 
     # bytes a decode step must read: every matrix and norm once, the rows of the embedding it
     # gathers, and the keys and values of the live requests at their mean length in the timed steps
@@ -144,10 +265,12 @@ def main() -> int:
                    "heads": nh, "kv_heads": nkv, "head_dim": d, "intermediate": inter, "vocab": vocab,
                    "block_size": block_size, "weights": "random", "prefill_tokens": PREFILL_TOKENS},
         "prefill": {"value": round(t / pre_s, 1), "tokens": t, "ms": ms(pre_s),
-                    "frac": round(flops / pre_s / PEAK_FLOPS[args.dtype], 4)},
+                    "frac": round(flops / pre_s / PEAK_FLOPS[args.dtype], 4),
+                    "chunked": {"budget": PREFILL_CHUNK, "ms": ms(chunked_s)}},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
+        "measured_peaks": peaks,
     }
     print(json.dumps(line))
     return 0

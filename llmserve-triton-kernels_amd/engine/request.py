@@ -36,6 +36,19 @@ class Request:
         return self.prompt_ids + self.generated
 
     @property
+    def num_tokens(self) -> int:
+        return len(self.prompt_ids) + len(self.generated)
+
+    def tokens(self, start: int, count: int) -> list[int]:
+        """`count` tokens of prompt + generated from position `start`, without building the whole list."""
+        n = len(self.prompt_ids)
+        if start >= n:
+            return self.generated[start - n: start - n + count]
+        if start + count <= n:
+            return self.prompt_ids[start: start + count]
+        return self.prompt_ids[start:] + self.generated[: start + count - n]
+
+    @property
     def first_token_time(self) -> float | None:
         return self.token_times[0] if self.token_times else None
 

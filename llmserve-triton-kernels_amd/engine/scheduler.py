@@ -127,7 +127,7 @@ class ContinuousBatchingEngine:
         plan = self._plan(admit=not preempted)
         if not plan:
             return events
-        entries = [StepEntry(r.req_id, r.all_ids[r.num_computed_tokens: r.num_computed_tokens + n],
+        entries = [StepEntry(r.req_id, r.tokens(r.num_computed_tokens, n),
                              [n - 1] if samples else []) for r, n, samples in plan]
         logits = self.runner.step(entries)
         sampling = [r for r, _, samples in plan if samples]
@@ -159,7 +159,7 @@ class ContinuousBatchingEngine:
 
     def _known_need(self, r: Request) -> int:
         """Pages `r` still has to take for the tokens it already has."""
-        return self.manager.extra_blocks_needed(r.req_id, len(r.all_ids) - self.manager.lengths[r.req_id])
+        return self.manager.extra_blocks_needed(r.req_id, r.num_tokens - self.manager.lengths[r.req_id])
 
     def _make_room(self) -> bool:
         """Preempt, newest admission first, until the running requests' known tokens fit."""
@@ -188,12 +188,12 @@ class ContinuousBatchingEngine:
         """(request, tokens it feeds, whether it samples) for this step."""
         budget = self.max_num_batched_tokens
         plan: list[tuple[Request, int, bool]] = []
-        decoding = [r for r in self.running if len(r.all_ids) - r.num_computed_tokens == 1]
-        prefilling = [r for r in self.running if len(r.all_ids) - r.num_computed_tokens > 1]
+        decoding = [r for r in self.running if r.num_tokens - r.num_computed_tokens == 1]
+        prefilling = [r for r in self.running if r.num_tokens - r.num_computed_tokens > 1]
         for r in decoding + prefilling:
             if budget <= 0:
                 break
-            remaining = len(r.all_ids) - r.num_computed_tokens
+            remaining = r.num_tokens - r.num_computed_tokens
             n = self._portion(remaining, budget)
             plan.append((r, n, n == remaining))
             budget -= n
@@ -202,7 +202,7 @@ class ContinuousBatchingEngine:
         reserved = sum(self._known_need(r) for r in self.running)
         while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
             req = self.waiting[0]
-            total = len(req.all_ids)
+            total = req.num_tokens
             need = self.manager.blocks_for(total)
             headroom = len(self.running)  # one spare page per request already live
             if self.manager.num_free_blocks - reserved - need < headroom:
