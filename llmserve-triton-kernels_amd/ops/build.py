@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -118,8 +119,9 @@ def _compile(name: str, out_dir: Path, log) -> Path:
         tmp.unlink(missing_ok=True)
         raise BuildError(f"hipcc failed on {src}:\n{output}")
     os.replace(tmp, final)  # atomic: a concurrent process sees either nothing or the whole file
-    for old in out_dir.glob(f"libllms_{name}_*.so"):
-        if old != final:
+    stale = re.compile(rf"libllms_{re.escape(name)}_[0-9a-f]{{12}}\.so")  # (not gemm_stream's when this is gemm)
+    for old in out_dir.iterdir():
+        if stale.fullmatch(old.name) and old != final:
             old.unlink(missing_ok=True)
     log(f"[llmserve build] {name}.hip -> {final.name} ({time.time() - t0:.0f} s)")
     return final
