@@ -350,8 +350,14 @@ __global__ __launch_bounds__(SPLIT_WAVES && DB <= 10 ? 512 : 256) void attn_mfma
 // rows and of the (page-transposed) value rows into LDS, double-buffered, and the waves read their matrix operands
 // from there.  Key rows are stored in the order the score product wants them (row 16u + i holds key 8*(i/4) + 4u + i%4,
 // padded by one chunk per row against bank conflicts); values keep their [dimension][key] order.
-template <int DB>
-__global__ __launch_bounds__(256) void attn_prompt_kernel(const AttnArgs a) {
+//
+// PAIRED (no window): the causal triangle gives the last tokens of a prompt the most keys, and a workgroup with
+// few keys leaves its CU idle while others still run.  A workgroup then has 8 waves and takes two blocks of
+// tokens, number x from the front and number x from the back: waves 0-3 the late block, whose keys they load
+// for all, waves 4-7 the early block, which sees a prefix of the same keys and stops when it has passed its
+// own position.  Every workgroup of a request then has the same work.
+template <int DB, bool PAIRED>
+__global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
     constexpr int KS = (D + 31) / 32;
     constexpr int KCH = D / 8;          // 16-byte chunks of a key row
@@ -369,12 +375,27 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const AttnArgs a) {
     const int b = a.seq_begin + blockIdx.z;
     const int tok0 = a.cu_seqlens[b], n_new = a.cu_seqlens[b + 1] - tok0;
     const int ctx = a.context_lens[b];
-    const int wg_first = blockIdx.x * 4 * TPG;  // first token of the workgroup within the request's new tokens
-    if (wg_first >= n_new || ctx <= 0) return;
+    // wg_first: first token (within the request's new tokens) of the block whose keys the workgroup walks;
+    // my_first: of the block this wave works for
+    int wg_first, my_first;
+    bool wave_on = true;
+    if (PAIRED) {
+        const int blocks = ((n_new + TPG - 1) / TPG + 3) / 4;
+        const int late = blocks - 1 - (int)blockIdx.x, early = blockIdx.x;
+        if (late < early || ctx <= 0) return;
+        wg_first = late * 4 * TPG;
+        my_first = (wave < 4 ? late : early) * 4 * TPG;
+        wave_on = wave < 4 || early != late;  // (the middle block of an odd number is its own partner)
+    } else {
+        wg_first = my_first = blockIdx.x * 4 * TPG;
+        if (wg_first >= n_new || ctx <= 0) return;
+    }
+    const bool loader = tid < 256;  // waves 0-3 bring the tiles in
 
-    const int t_first = wg_first + wave * TPG;
+    const int t_first = my_first + (wave % 4) * TPG;
+    wave_on = wave_on && t_first < n_new;
     const int c_tok = t_first + col / HG, c_head_in = hb * HG + col % HG;
-    const bool col_ok = col < HG * TPG && c_tok < n_new && c_head_in < G;
+    const bool col_ok = wave_on && col < HG * TPG && c_tok < n_new && c_head_in < G;
     const int head = kvh * G + c_head_in;
     const int p_col = col_ok ? ctx - n_new + c_tok : -1;
     const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
@@ -464,13 +485,16 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const AttnArgs a) {
         }
     };
 
-    load_pages(block_of(j_begin));
-    load_tile(j_begin);
-    store_tile(0, j_begin);
-    if (n_tiles > 1) load_tile(j_begin + 32);
+    if (loader) {
+        load_pages(block_of(j_begin));
+        load_tile(j_begin);
+        store_tile(0, j_begin);
+        if (n_tiles > 1) load_tile(j_begin + 32);
+    }
     __syncthreads();
     for (int t = 0; t < n_tiles; ++t) {
         const int buf = t & 1, j0 = j_begin + 32 * t;
+        if (wave_on && j0 <= w_pmax) {  // (a tile beyond the wave's last position adds nothing)
         uint4 kf[2][KS], vf[DB];
 #pragma unroll
         for (int u = 0; u < 2; ++u)
@@ -485,7 +509,8 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const AttnArgs a) {
             attend_tile<DB, KS, false>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
         else
             attend_tile<DB, KS, true>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
-        if (t + 1 < n_tiles) {
+        }
+        if (loader && t + 1 < n_tiles) {
             store_tile(buf ^ 1, j0 + 32);  // last read two tiles ago, before the previous barrier
             if (t + 2 < n_tiles) load_tile(j_begin + 32 * (t + 2));
         }
@@ -528,10 +553,11 @@ __global__ void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const 
     }
 }
 
-static int launch_prompt(int db, dim3 grid, const AttnArgs& a, hipStream_t stream) {
-#define ATT_CASE(N)                                                  \
-    case N:                                                          \
-        attn_prompt_kernel<N><<<grid, 256, 0, stream>>>(a);          \
+static int launch_prompt(int db, dim3 grid, bool paired, const AttnArgs& a, hipStream_t stream) {
+#define ATT_CASE(N)                                                                  \
+    case N:                                                                          \
+        if (paired) attn_prompt_kernel<N, true><<<grid, 512, 0, stream>>>(a);        \
+        else attn_prompt_kernel<N, false><<<grid, 256, 0, stream>>>(a);              \
         break;
     switch (db) {
         ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
@@ -611,8 +637,12 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
         dim3 grid((groups + 3) / 4, n_kv_heads * HB, n_seqs);
         if (split_waves < 0) {  // the variant that reads every operand straight from global memory
             if (int e = launch_attn<false>(head_dim / 16, grid, 256, a, stream)) return e;
+        } else if (window == 0 && head_dim <= 192) {  // early and late blocks of tokens paired in one workgroup
+            // (8 waves of wider heads would not fit the registers)
+            grid.x = (grid.x + 1) / 2;
+            if (int e = launch_prompt(head_dim / 16, grid, true, a, stream)) return e;
         } else {
-            if (int e = launch_prompt(head_dim / 16, grid, a, stream)) return e;
+            if (int e = launch_prompt(head_dim / 16, grid, false, a, stream)) return e;
         }
     }
     LLMS_LAUNCH_CHECK();
