@@ -96,8 +96,6 @@ class Attention(Mixer):
         """With few bfloat16 rows one kernel does the projection, the rotation and the cache store (and,
         if switched on, the residual sum and the norm before them): ops.gemm_stream.  Returns the rotated
         queries, or None when that kernel does not apply."""
-        if isinstance(x, DeferredNorm) and not (norm_fusable(*x.residual.shape) and isinstance(x.norm, RMSNorm)):
-            return None if self._few_rows_unfit(x.residual) else self.project_few_rows(x.materialize(), batch, cache, slots)
         deferred = isinstance(x, DeferredNorm)
         rows = x.residual if deferred else x
         m = rows.shape[0]
@@ -106,6 +104,8 @@ class Attention(Mixer):
         frequencies = getattr(self.position, "rotary_frequencies", None)
         if frequencies is None and not getattr(self.position, "identity", False):
             return None  # a position encoding this kernel does not know
+        if deferred and not (norm_fusable(*rows.shape) and isinstance(x.norm, RMSNorm)):
+            x, rows, deferred = None, x.materialize(), False  # the norm by its own kernel, the rest fused
         rope = dict(n_heads=self.num_heads, n_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                     inv_freq=frequencies() if frequencies is not None else None, positions=batch.positions,
                     slots=slots, k_pool=cache.k_pool, v_pool=cache.v_pool, block_size=cache.block_size)

@@ -237,8 +237,58 @@ class ToyConfig:
 
 def register_toy():
     from llmserve.config import register_architecture
-    from llmserve.parts import (LayerSpec, Mixer, ModelSpec, ParamInfo, PartSpec, StateCacheSpec, register_mixer)
+    from llmserve.parts import (FeedForward, LayerSpec, Mixer, ModelSpec, ParamInfo, PartSpec, PositionEncoding,
+                                StateCacheSpec, register_feed_forward, register_mixer, register_position_encoding)
     from llmserve.parts.linear import linear
+
+    @register_position_encoding("interleaved")
+    class InterleavedRotation(PositionEncoding):
+        """Rotation of the pairs (2i, 2i+1) instead of (i, i + D/2): another position encoding, which the
+        attention part takes through `rotate` alone (its fused kernels step aside)."""
+
+        def __init__(self, spec, ctx):
+            super().__init__(spec, ctx)
+            self.theta = float(spec["theta"])
+
+        def rotate(self, qkv, positions, n_heads, n_kv_heads, head_dim):
+            n, half = qkv.shape[0], head_dim // 2
+            inv = self.theta ** (-torch.arange(half, device=qkv.device, dtype=torch.float32) * 2 / head_dim)
+            ang = positions.float()[:, None] * inv
+            cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+            part = qkv[:, : (n_heads + n_kv_heads) * head_dim]
+            x = part.float().view(n, n_heads + n_kv_heads, half, 2)
+            even, odd = x[..., 0], x[..., 1]
+            rot = torch.stack([even * cos - odd * sin, odd * cos + even * sin], dim=-1)
+            part.copy_(rot.view(n, -1).to(qkv.dtype))
+
+    @register_feed_forward("soft_experts")
+    class SoftExperts(FeedForward):
+        """y = sum_e softmax(router x)_e * down_e(gelu(up_e x)): a feed-forward with a router of its own
+        (logits and softmax in 32-bit) and per-expert weights."""
+
+        def __init__(self, spec, ctx):
+            super().__init__(spec, ctx)
+            self.hidden, self.inter, self.experts = spec["hidden"], spec["intermediate"], spec["experts"]
+
+        def param_infos(self):
+            infos = {"router.weight": ParamInfo((self.experts, self.hidden))}
+            for e in range(self.experts):
+                infos[f"experts.{e}.up.weight"] = ParamInfo((self.inter, self.hidden))
+                infos[f"experts.{e}.down.weight"] = ParamInfo((self.hidden, self.inter))
+            return infos
+
+        def load(self, tensors):
+            self.router = tensors["router.weight"].float()
+            self.up = [tensors[f"experts.{e}.up.weight"].contiguous() for e in range(self.experts)]
+            self.down = [tensors[f"experts.{e}.down.weight"].contiguous() for e in range(self.experts)]
+
+        def forward(self, x):
+            gates = torch.softmax(x.float() @ self.router.t(), dim=-1)
+            y = torch.zeros_like(x, dtype=torch.float32)
+            for e in range(self.experts):
+                h = torch.nn.functional.gelu(linear(x, self.up[e]).float()).to(x.dtype)
+                y += gates[:, e: e + 1] * linear(h, self.down[e]).float()
+            return y.to(x.dtype)
 
     @register_mixer("running_mean")
     class RunningMean(Mixer):
@@ -275,8 +325,10 @@ def register_toy():
     def toy_spec(cfg: ToyConfig) -> ModelSpec:
         h = cfg.hidden_size
         norm = PartSpec("rmsnorm", {"hidden": h, "eps": cfg.eps})
+        interleaved = att_params(4, 2, 16, h)
+        interleaved["position"] = PartSpec("interleaved", {"theta": 10000.0})
         mixers = [
-            PartSpec("attention", att_params(4, 2, 16, h, theta=10000.0)),
+            PartSpec("attention", interleaved),
             PartSpec("attention", att_params(2, 1, 32, h, position="none", window=5, bias=True)),
             PartSpec("running_mean", {"hidden": h}),
             PartSpec("attention", att_params(2, 2, 16, h, theta=777.0)),  # reads the cache of layer 0
@@ -285,8 +337,10 @@ def register_toy():
         layers = []
         for i, (mixer, inter) in enumerate(zip(mixers, inters)):
             p = f"toy.{i}."
+            ffn = (PartSpec("soft_experts", {"hidden": h, "intermediate": inter, "experts": 3}) if i == 2
+                   else PartSpec("swiglu", {"hidden": h, "intermediate": inter}))
             layers.append(LayerSpec(
-                mixer=mixer, feed_forward=PartSpec("swiglu", {"hidden": h, "intermediate": inter}), mixer_norm=norm,
+                mixer=mixer, feed_forward=ffn, mixer_norm=norm,
                 feed_forward_norm=norm, cache_from=0 if i == 3 else None,
                 weights={"mixer": p + "mix.", "feed_forward": p + "ffn.", "mixer_norm": p + "n1.",
                          "feed_forward_norm": p + "n2."}))
@@ -308,12 +362,21 @@ def plain_toy_forward(w, ids, dtype):
     x = w["toy.emb.weight"][torch.tensor(ids)].to(dtype)
     kv = {}
 
-    def attention(i, hn, nh, nkv, d, theta, window, borrow=None):
+    def attention(i, hn, nh, nkv, d, theta, window, borrow=None, interleaved=False):
         p = f"toy.{i}.mix."
         q = pl.linear(hn, w[p + "q_proj.weight"], w.get(p + "q_proj.bias")).view(t, nh, d).transpose(0, 1)
         k = pl.linear(hn, w[p + "k_proj.weight"], w.get(p + "k_proj.bias")).view(t, nkv, d).transpose(0, 1)
         v = pl.linear(hn, w[p + "v_proj.weight"], w.get(p + "v_proj.bias")).view(t, nkv, d).transpose(0, 1)
-        if theta is not None:
+        if theta is not None and interleaved:
+            ang = torch.arange(t, dtype=torch.float32)[:, None] * theta ** (-torch.arange(d // 2, dtype=torch.float32) * 2 / d)
+
+            def turn(x):  # [heads, t, d], pairs (2i, 2i+1)
+                xf = x.float().view(x.shape[0], t, d // 2, 2)
+                even, odd = xf[..., 0], xf[..., 1]
+                return torch.stack([even * ang.cos() - odd * ang.sin(), odd * ang.cos() + even * ang.sin()], -1).view_as(x).to(x.dtype)
+
+            q, k = turn(q.contiguous()), turn(k.contiguous())
+        elif theta is not None:
             cos, sin = pl.rope_cos_sin(torch.arange(t), d, theta)
             q, k = pl.apply_rope(q, cos, sin), pl.apply_rope(k, cos, sin)
         if borrow is not None:
@@ -326,7 +389,7 @@ def plain_toy_forward(w, ids, dtype):
         p = f"toy.{i}."
         hn = pl.rms_norm(x, w[p + "n1.weight"], eps)
         if i == 0:
-            a = attention(0, hn, 4, 2, 16, 10000.0, None)
+            a = attention(0, hn, 4, 2, 16, 10000.0, None, interleaved=True)
         elif i == 1:
             a = attention(1, hn, 2, 1, 32, None, 5)
         elif i == 2:
@@ -335,7 +398,17 @@ def plain_toy_forward(w, ids, dtype):
         else:
             a = attention(3, hn, 2, 2, 16, 777.0, None, borrow=0)
         x = x + a
-        x = x + pl.swiglu(pl.rms_norm(x, w[p + "n2.weight"], eps), w, p + "ffn.")
+        hn2 = pl.rms_norm(x, w[p + "n2.weight"], eps)
+        if i == 2:  # the routed feed-forward
+            gates = torch.softmax(hn2.float() @ w[p + "ffn.router.weight"].float().t(), dim=-1)
+            y = torch.zeros(t, h)
+            for e in range(3):
+                up = pl.linear(hn2, w[p + f"ffn.experts.{e}.up.weight"])
+                y += gates[:, e: e + 1] * pl.linear(torch.nn.functional.gelu(up.float()).to(dtype),
+                                                    w[p + f"ffn.experts.{e}.down.weight"]).float()
+            x = x + y.to(dtype)
+        else:
+            x = x + pl.swiglu(hn2, w, p + "ffn.")
     return pl.rms_norm(x, w["toy.norm.weight"], eps).float() @ w["toy.head.weight"].float().t()
 
 
