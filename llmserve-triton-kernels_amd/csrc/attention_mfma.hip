@@ -287,61 +287,58 @@ __global__ __launch_bounds__(SPLIT_WAVES && DB <= 10 ? 512 : 256) void attn_mfma
         return;
     }
 
-    // ---- the waves' partial results meet in LDS, wave 0 first, then 1, 2, ...
-    __shared__ float sh_acc[DB][LLMS_WAVE][4];
-    __shared__ float sh_m[16], sh_l[16];
-    for (int w = 0; w < (int)(blockDim.x / LLMS_WAVE); ++w) {
-        if (wave == w) {
-            if (w == 0) {
+    // ---- the waves' partial results meet in LDS: every wave leaves its own, then the blocks of 16 dimensions
+    // are dealt to the waves, each of which adds the partial results up in the order of the waves
+    constexpr int NW = SPLIT_WAVES ? (DB <= 10 ? 8 : 4) : 1;  // (what the launch bounds allow)
+    __shared__ float sh_acc[NW][DB][LLMS_WAVE][4];
+    __shared__ float sh_m[NW][16], sh_l[NW][16];
+    const int nw = blockDim.x / LLMS_WAVE;
 #pragma unroll
-                for (int m = 0; m < DB; ++m)
+    for (int m = 0; m < DB; ++m)
+        *reinterpret_cast<float4*>(sh_acc[wave][m][lane]) = make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+    if (g == 0) {
+        sh_m[wave][col] = m_run;
+        sh_l[wave][col] = l_run;
+    }
+    __syncthreads();
+    float m_tot = -INFINITY;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) sh_acc[m][lane][r] = acc[m][r];
-                if (g == 0) {
-                    sh_m[col] = m_run;
-                    sh_l[col] = l_run;
-                }
-            } else {
-                const float m_old = sh_m[col], l_old = sh_l[col];
-                const float m_tot = fmaxf(m_old, m_run);
-                const float m_safe = (m_tot == -INFINITY) ? 0.f : m_tot;
-                const float wa = exp2_fast(m_old - m_safe), wb = exp2_fast(m_run - m_safe);
+    for (int w = 0; w < NW; ++w)
+        if (w < nw) m_tot = fmaxf(m_tot, sh_m[w][col]);
+    const float m_safe = (m_tot == -INFINITY) ? 0.f : m_tot;
+    float weight[NW], l_tot = 0.f;
 #pragma unroll
-                for (int m = 0; m < DB; ++m)
+    for (int w = 0; w < NW; ++w) {
+        weight[w] = w < nw ? exp2_fast(sh_m[w][col] - m_safe) : 0.f;  // 0 for a wave that saw no key
+        if (w < nw) l_tot += sh_l[w][col] * weight[w];
+    }
+    const size_t item = ((size_t)(tok0 + c_tok) * a.n_heads + head) * a.num_splits + split;
+    for (int m = wave; m < DB; m += nw) {
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) sh_acc[m][lane][r] = sh_acc[m][lane][r] * wa + acc[m][r] * wb;
-                __builtin_amdgcn_wave_barrier();  // all lanes have read sh_m/sh_l before lane group 0 rewrites them
-                if (g == 0) {
-                    sh_m[col] = m_tot;
-                    sh_l[col] = l_old * wa + l_run * wb;
-                }
+        for (int w = 0; w < NW; ++w) {
+            if (w < nw) {
+                const float4 p = *reinterpret_cast<const float4*>(sh_acc[w][m][lane]);
+                o.x += p.x * weight[w];
+                o.y += p.y * weight[w];
+                o.z += p.z * weight[w];
+                o.w += p.w * weight[w];
             }
         }
-        __syncthreads();
+        if (!col_ok) continue;
+        if (a.num_splits == 1) {
+            const float inv = 1.f / l_tot;
+            uint2 pk;
+            pk.x = pack_bf16(o.x * inv, o.y * inv);
+            pk.y = pack_bf16(o.z * inv, o.w * inv);
+            *reinterpret_cast<uint2*>(a.out + (size_t)(tok0 + c_tok) * a.out_stride + (size_t)head * D + 16 * m + 4 * g) = pk;
+        } else {
+            *reinterpret_cast<float4*>(a.ws_o + item * D + 16 * m + 4 * g) = o;
+        }
     }
-    if (wave != 0 || !col_ok) return;
-    const float m_tot = sh_m[col], l_tot = sh_l[col];
-    if (a.num_splits == 1) {
-        const float inv = 1.f / l_tot;
-        bf16* orow = a.out + (size_t)(tok0 + c_tok) * a.out_stride + (size_t)head * D;
-#pragma unroll
-        for (int m = 0; m < DB; ++m) {
-            uint2 w;
-            w.x = pack_bf16(sh_acc[m][lane][0] * inv, sh_acc[m][lane][1] * inv);
-            w.y = pack_bf16(sh_acc[m][lane][2] * inv, sh_acc[m][lane][3] * inv);
-            *reinterpret_cast<uint2*>(orow + 16 * m + 4 * g) = w;
-        }
-    } else {
-        const size_t item = ((size_t)(tok0 + c_tok) * a.n_heads + head) * a.num_splits + split;
-        float* wo = a.ws_o + item * D;
-#pragma unroll
-        for (int m = 0; m < DB; ++m)
-            *reinterpret_cast<float4*>(wo + 16 * m + 4 * g) =
-                make_float4(sh_acc[m][lane][0], sh_acc[m][lane][1], sh_acc[m][lane][2], sh_acc[m][lane][3]);
-        if (g == 0) {
-            a.ws_ml[item * 2] = m_tot;
-            a.ws_ml[item * 2 + 1] = l_tot;
-        }
+    if (a.num_splits > 1 && wave == 0 && g == 0 && col_ok) {
+        a.ws_ml[item * 2] = m_tot;
+        a.ws_ml[item * 2 + 1] = l_tot;
     }
 }
 
