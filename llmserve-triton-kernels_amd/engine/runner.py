@@ -117,12 +117,28 @@ class ModelRunner:
 
     # ---- the step ---------------------------------------------------------------------------
     @torch.inference_mode()
-    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+    @property
+    def takes_device_tokens(self) -> bool:
+        """Whether `step(..., device_tokens=...)` is available (decode-only steps are replayed graphs)."""
+        return self._use_graphs
+
+    def step(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None) -> torch.Tensor:
         """Run the entries' tokens as one batch; float32 logits [sum(len(want)), vocab] in the
         order of the entries and of their `want`.  Raises `OutOfBlocks` (nothing changed) when
-        the pages do not suffice."""
+        the pages do not suffice.
+
+        `device_tokens` (int32, one per entry, on the device): every entry brings one token, and
+        its value is taken from this tensor instead of the entry (whose token is a placeholder):
+        the ids the sampler chose for the previous step, which the host need not have seen yet."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        if device_tokens is not None:
+            if not self.takes_device_tokens:
+                raise ValueError("this runner does not replay decode steps, so it takes tokens from the host only")
+            if (device_tokens.dtype != torch.int32 or device_tokens.device != self.device or
+                    tuple(device_tokens.shape) != (len(entries),) or any(len(e.tokens) != 1 for e in entries)):
+                raise ValueError("device_tokens must be an int32 tensor on the runner's device, one id per entry, "
+                                 "and every entry must bring exactly one token")
         for e in entries:
             if not e.tokens:
                 raise ValueError(f"request {e.seq_id!r} brings no tokens")
@@ -150,7 +166,7 @@ class ModelRunner:
         logit_rows = [first_row[id(e)] + w for e in entries for w in e.want]
         self.storage.clear_state(layout.fresh_slots)
         if self._use_graphs and all(len(e.tokens) == 1 for e in ordered):
-            logits = self._replay_decode(layout, [e.tokens[0] for e in ordered], logit_rows)
+            logits = self._replay_decode(layout, [e.tokens[0] for e in ordered], logit_rows, device_tokens)
         else:
             batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
             logits = self.model.forward(batch, self.storage)
@@ -158,7 +174,8 @@ class ModelRunner:
         return logits
 
     # ---- decode-only steps as HIP graphs --------------------------------------------------------
-    def _replay_decode(self, layout, tokens: list[int], logit_rows: list[int]) -> torch.Tensor:
+    def _replay_decode(self, layout, tokens: list[int], logit_rows: list[int],
+                       device_tokens: torch.Tensor | None = None) -> torch.Tensor:
         """A step of single tokens: replay the graph captured for this batch size and context range
         (capture it at first use).  The logits it returns live in the graph's own memory and are
         overwritten by the next replay of the same graph."""
@@ -176,6 +193,8 @@ class ModelRunner:
             graph = _DecodeGraph(self, capacity, reach)
             self._graphs[key] = graph
         graph.static.fill(layout, tokens)
+        if device_tokens is not None:  # (all entries bring one token, so their order is the caller's)
+            graph.static.batch.token_ids[:n].copy_(device_tokens)
         graph.graph.replay()
         if logit_rows == list(range(n)):
             return graph.logits[:n]

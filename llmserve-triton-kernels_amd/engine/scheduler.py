@@ -20,6 +20,15 @@ One `step()` is one call of the step function with everything that is scheduled:
 A request samples when its portion reaches the end of `prompt + generated`.  The reference
 prefills a prompt whole and runs two forwards per iteration; portions under a token budget
 and the single mixed batch are this engine's own.
+
+Reading tokens back one step late.  With a sampler that can leave its ids on the device
+(`sample_async`) a step does not wait for them: they are read at the start of the next `step()`.
+And when that next step is a plain continuation (the same requests, all decoding, nothing
+waiting, aborted or about to reach its length, pages at hand) it is started first, on the ids
+still on the device, and the ids of the step before are read while it runs, so the GPU never
+waits for the host's bookkeeping.  A request that turns out to have stopped (its end-of-sequence
+token) has then one more row in the step already started; that row's token is dropped.  Events
+and `token_times` therefore lag a step behind the GPU; which tokens are produced does not change.
 """
 
 from __future__ import annotations
@@ -55,6 +64,9 @@ class ContinuousBatchingEngine:
         self._next_id = 0
         self._aborts: set[int] = set()
         self._lock = threading.Lock()
+        # the requests (in row order) and the token ids of a step that has been started but not read yet
+        self._pending: tuple[list[Request], object] | None = None
+        self._lagged = hasattr(sampler, "sample_async")
 
     # ------------------------------------------------------------------ public
     def validate_request(self, prompt_len: int, max_new_tokens: int) -> None:
@@ -94,6 +106,7 @@ class ContinuousBatchingEngine:
 
     def reset(self) -> None:
         """Drop every request in flight and give back what they hold."""
+        self._pending = None
         for r in self.running:
             self.manager.free_sequence(r.req_id)
         self.running.clear()
@@ -122,6 +135,11 @@ class ContinuousBatchingEngine:
     def step(self) -> list[TokenEvent]:
         events: list[TokenEvent] = []
         self.stats.steps += 1
+        if self._pending is not None:
+            if self._can_continue():
+                self._continue(events)
+                return events
+            self._read_pending(events)
         self._process_aborts(events)
         preempted = self._make_room()
         plan = self._plan(admit=not preempted)
@@ -131,15 +149,51 @@ class ContinuousBatchingEngine:
                              [n - 1] if samples else []) for r, n, samples in plan]
         logits = self.runner.step(entries)
         sampling = [r for r, _, samples in plan if samples]
-        tokens = self.sampler.sample(logits, [(r.params, r.seed, len(r.generated)) for r in sampling])
+        items = [(r.params, r.seed, len(r.generated)) for r in sampling]
         for r, n, _ in plan:
             if n == 1 and r.num_computed_tokens > 0 and r.generated:
                 self.stats.decode_tokens += 1
             else:
                 self.stats.prefill_tokens += n
             r.num_computed_tokens += n
-        self._append_tokens(sampling, tokens, events)
+        if self._lagged:
+            self._pending = (sampling, self.sampler.sample_async(logits, items))  # read at the next step
+        else:
+            self._append_tokens(sampling, self.sampler.sample(logits, items), events)
         return events
+
+    # ------------------------------------------------- a step whose tokens are read later
+    def _read_pending(self, events: list[TokenEvent]) -> None:
+        reqs, pending = self._pending
+        self._pending = None
+        self._append_tokens(reqs, pending.result(), events)
+
+    def _can_continue(self) -> bool:
+        """Whether the next step is the pending one's requests again, each with the one token
+        that is still on the device."""
+        reqs, pending = self._pending
+        if (self.waiting or self._aborts or not reqs or len(reqs) != len(self.running)
+                or not getattr(self.runner, "takes_device_tokens", False)):
+            return False
+        need = 0
+        for r, q in zip(reqs, self.running):
+            # the same requests in the same order, none stopped meanwhile, none at its last token
+            if r is not q or r.status is not Status.RUNNING or len(r.generated) + 2 > r.params.max_new_tokens:
+                return False
+            if r.num_computed_tokens != r.num_tokens:  # (every token it has is in the cache: it is decoding)
+                return False
+            need += self.manager.extra_blocks_needed(r.req_id, 1)
+        return need <= self.manager.num_free_blocks
+
+    def _continue(self, events: list[TokenEvent]) -> None:
+        reqs, pending = self._pending
+        logits = self.runner.step([StepEntry(r.req_id, [0], [0]) for r in reqs], device_tokens=pending.device)
+        following = self.sampler.sample_async(logits, [(r.params, r.seed, len(r.generated) + 1) for r in reqs])
+        for r in reqs:
+            r.num_computed_tokens += 1
+        self.stats.decode_tokens += len(reqs)
+        self._read_pending(events)  # the step before; a request that stopped there is skipped from now on
+        self._pending = (reqs, following)
 
     # --------------------------------------------------------------- internals
     def _process_aborts(self, events: list[TokenEvent]) -> None:
@@ -223,6 +277,8 @@ class ContinuousBatchingEngine:
     def _append_tokens(self, reqs: list[Request], tokens: list[int], events: list[TokenEvent]) -> None:
         now = perf_counter()
         for r, tok in zip(reqs, tokens):
+            if r.status is not Status.RUNNING:
+                continue  # it stopped a step earlier; this row was computed for nothing
             r.generated.append(tok)
             r.token_times.append(now)
             self.stats.tokens_generated += 1

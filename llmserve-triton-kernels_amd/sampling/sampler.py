@@ -39,17 +39,44 @@ def request_seed(params: SamplingParams, engine_seed: int, request_id: int) -> i
     return _splitmix64((engine_seed << 32) ^ (request_id & 0xFFFFFFFF))
 
 
+class PendingTokens:
+    """Token ids that were chosen on the device and are on their way to the host: `device` is the
+    int32 tensor the sampling kernel wrote (the next step can read it there), `result()` waits for
+    the copy and returns the ids."""
+
+    def __init__(self, device: torch.Tensor | None):
+        self.device = device
+        self._host = None
+        self._event = None
+        if device is not None:
+            self._host = torch.empty(device.shape, dtype=torch.int32, pin_memory=True)
+            self._host.copy_(device, non_blocking=True)
+            self._event = torch.cuda.Event()
+            self._event.record(torch.cuda.current_stream(device.device))
+
+    def result(self) -> list[int]:
+        if self._host is None:
+            return []
+        self._event.synchronize()
+        return self._host.tolist()  # the step's one read-back
+
+
 class Sampler:
     def __init__(self, device: torch.device):
         self.device = device
 
     def sample(self, logits: torch.Tensor, items: list[tuple[SamplingParams, int, int]]) -> list[int]:
         """logits float32 [R, V]; items[r] = (params, seed, index of the token being generated)."""
+        return self.sample_async(logits, items).result()
+
+    def sample_async(self, logits: torch.Tensor, items: list[tuple[SamplingParams, int, int]]) -> PendingTokens:
+        """As `sample`, but returns at once: the ids stay on the device for the next step and come
+        to the host when `result()` is asked."""
         r = logits.shape[0]
         if r != len(items):
             raise ValueError(f"{r} rows of logits for {len(items)} requests")
         if r == 0:
-            return []
+            return PendingTokens(None)
         out = torch.empty(r, dtype=torch.int32, device=logits.device)
         if all(p.temperature <= 0 for p, _, _ in items):
             ops.sample_rows(out, logits)
@@ -59,4 +86,4 @@ class Sampler:
                 dtype=torch.float32).t().contiguous().to(logits.device)
             top_k = torch.tensor([p.top_k for p, _, _ in items], dtype=torch.int32).to(logits.device)
             ops.sample_rows(out, logits, temperature=host[0], top_k=top_k, top_p=host[1], uniform=host[2])
-        return out.tolist()  # the step's one read-back
+        return PendingTokens(out)

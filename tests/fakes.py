@@ -39,3 +39,37 @@ class PlainSampler:
     def sample(self, logits, items):
         return [plain_llama.sample(logits[i], p.temperature, p.top_k, p.top_p, uniform(seed, index))
                 for i, (p, seed, index) in enumerate(items)]
+
+
+class LaggedRunner(PlainRunner):
+    """The same, taking a step's tokens from the sampler's pending ids (here a list stands in for
+    the tensor on the device), as the GPU runner does when decode steps are replayed graphs."""
+
+    takes_device_tokens = True
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.continuations = 0
+
+    def step(self, entries, device_tokens=None):
+        if device_tokens is not None:
+            assert len(device_tokens) == len(entries) and all(e.tokens == [0] for e in entries)
+            entries = [type(e)(e.seq_id, [int(t)], e.want) for e, t in zip(entries, device_tokens)]
+            self.continuations += 1
+        return super().step(entries)
+
+
+class FakePending:
+    def __init__(self, tokens):
+        self.device = list(tokens)
+        self.reads = 0
+
+    def result(self):
+        self.reads += 1
+        assert self.reads == 1, "a step's tokens are read once"
+        return list(self.device)
+
+
+class LaggedSampler(PlainSampler):
+    def sample_async(self, logits, items):
+        return FakePending(self.sample(logits, items))

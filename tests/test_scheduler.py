@@ -7,7 +7,7 @@ import torch
 
 import plain_llama
 from conftest import TINY_A
-from fakes import PlainRunner, PlainSampler
+from fakes import LaggedRunner, LaggedSampler, PlainRunner, PlainSampler
 from llmserve.engine.scheduler import ContinuousBatchingEngine
 from llmserve.sampling import SamplingParams
 from llmserve.weights import random_tensors
@@ -28,10 +28,15 @@ def prompt(n, seed):
     return torch.randint(0, TINY_A["vocab_size"], (n,), generator=torch.Generator().manual_seed(seed)).tolist()
 
 
-def engine(weights, *, num_blocks=64, block_size=4, max_batch=4, budget=2048, chunk=None):
-    runner = PlainRunner(TINY_A, weights, num_blocks, block_size)
-    return ContinuousBatchingEngine(runner, PlainSampler(), max_num_seqs=max_batch, max_num_batched_tokens=budget,
-                                    max_prefill_chunk=chunk)
+def engine(weights, *, num_blocks=64, block_size=4, max_batch=4, budget=2048, chunk=None, lagged=False):
+    """`lagged`: runner and sampler that let the scheduler read a step's tokens one step late and start
+    the next step on the ids the sampler left behind, as on the GPU."""
+    runner = (LaggedRunner if lagged else PlainRunner)(TINY_A, weights, num_blocks, block_size)
+    return ContinuousBatchingEngine(runner, LaggedSampler() if lagged else PlainSampler(), max_num_seqs=max_batch,
+                                    max_num_batched_tokens=budget, max_prefill_chunk=chunk)
+
+
+LAGGED = pytest.mark.parametrize("lagged", [False, True], ids=["immediate", "lagged"])
 
 
 _REFERENCE = {}
@@ -47,9 +52,10 @@ def reference(weights, p, max_new):
 WORKLOAD = [(5, 9), (13, 4), (8, 12), (3, 7), (17, 5), (6, 10)]  # (prompt_len, max_new)
 
 
+@LAGGED
 @pytest.mark.parametrize("budget,chunk", [(2048, None), (16, None), (8, 5), (4, 2)])
-def test_batched_outputs_equal_independent_generation(weights, budget, chunk):
-    eng = engine(weights, max_batch=3, budget=budget, chunk=chunk)
+def test_batched_outputs_equal_independent_generation(weights, budget, chunk, lagged):
+    eng = engine(weights, max_batch=3, budget=budget, chunk=chunk, lagged=lagged)
     prompts = [prompt(n, 100 + i) for i, (n, _) in enumerate(WORKLOAD)]
     ids = [eng.add_request(p, SamplingParams(max_new_tokens=m)) for p, (_, m) in zip(prompts, WORKLOAD)]
     done = eng.run_until_complete()
@@ -61,6 +67,8 @@ def test_batched_outputs_equal_independent_generation(weights, budget, chunk):
     if chunk:
         assert all(n <= chunk for sizes in eng.runner.step_sizes for n in sizes)
     assert eng.stats.tokens_generated == sum(m for _, m in WORKLOAD)
+    if lagged:
+        assert eng.runner.continuations > 0, "some steps must have started on tokens not yet read"
 
 
 def test_portions_run_beside_decoding(weights):
@@ -104,9 +112,10 @@ def test_admission_is_in_order_and_keeps_headroom(weights):
     assert done[small].generated == reference(weights, prompt(2, 3), 2)
 
 
-def test_preemption_recompute_preserves_greedy_outputs(weights):
+@LAGGED
+def test_preemption_recompute_preserves_greedy_outputs(weights, lagged):
     # 14 pages of 4 and four (6, 14) requests cannot all grow (tests/test_scheduler.py:69-82 there)
-    eng = engine(weights, num_blocks=14, block_size=4, max_batch=4)
+    eng = engine(weights, num_blocks=14, block_size=4, max_batch=4, lagged=lagged)
     work = [(6, 14)] * 4
     prompts = [prompt(n, 50 + i) for i, (n, _) in enumerate(work)]
     ids = [eng.add_request(p, SamplingParams(max_new_tokens=m)) for p, (_, m) in zip(prompts, work)]
@@ -131,10 +140,11 @@ def test_preemption_takes_the_newest_and_requeues_it_first(weights):
     assert eng.manager.num_free_blocks == 6
 
 
-def test_eos_finishes_early_and_frees_blocks(weights):
+@LAGGED
+def test_eos_finishes_early_and_frees_blocks(weights, lagged):
     p = prompt(7, 9)
     first = reference(weights, p, 1)[0]
-    eng = engine(weights)
+    eng = engine(weights, lagged=lagged)
     rid = eng.add_request(p, SamplingParams(max_new_tokens=20, eos_token_id=first))
     done = eng.run_until_complete()
     assert done[rid].generated == [first] and done[rid].finish_reason == "stop"
@@ -203,3 +213,72 @@ def test_snapshot_and_events(weights):
     eng.step()
     eng.reset()
     assert not eng.has_unfinished() and eng.manager.num_free_blocks == eng.manager.num_blocks
+
+
+# ------------------------------------------------------- tokens read one step late (as on the GPU)
+def test_lagged_sampling_draws_the_same_tokens(weights):
+    """Reading tokens a step late must not shift which uniform number a token is drawn with."""
+    work = [(6, 12, 0.9, 11), (9, 10, 0.6, 12), (4, 14, 1.2, 13)]
+    outs = []
+    for lagged in (False, True):
+        eng = engine(weights, max_batch=3, lagged=lagged)
+        ids = [eng.add_request(prompt(n, 30 + i), SamplingParams(temperature=t, top_k=20, seed=sd, max_new_tokens=m))
+               for i, (n, m, t, sd) in enumerate(work)]
+        done = eng.run_until_complete()
+        outs.append([done[r].generated for r in ids])
+        if lagged:
+            assert eng.runner.continuations > 0
+    assert outs[0] == outs[1]
+
+
+def test_lagged_late_stop_drops_the_row_computed_for_nothing(weights):
+    """A request whose end-of-sequence token is seen a step late has a row in the step already started:
+    its token is dropped, its pages are freed, and the other request goes on as if alone."""
+    a, b = prompt(7, 9), prompt(5, 12)
+    ref_a, ref_b = reference(weights, a, 12), reference(weights, b, 12)
+    stop_at = 4
+    eos = ref_a[stop_at]
+    assert eos not in ref_a[:stop_at] and eos not in ref_b
+    eng = engine(weights, lagged=True)
+    ra = eng.add_request(a, SamplingParams(max_new_tokens=12, eos_token_id=eos))
+    rb = eng.add_request(b, SamplingParams(max_new_tokens=12, eos_token_id=eos))
+    done = eng.run_until_complete()
+    assert done[ra].generated == ref_a[: stop_at + 1] and done[ra].finish_reason == "stop"
+    assert done[rb].generated == ref_b and done[rb].finish_reason == "length"
+    assert eng.runner.continuations > 0
+    assert eng.stats.tokens_generated == stop_at + 1 + 12
+    assert eng.manager.num_free_blocks == eng.manager.num_blocks and eng.manager.num_free_slots == eng.manager.max_seqs
+    eng.manager.check_invariants()
+
+
+def test_lagged_abort_and_late_arrival(weights):
+    eng = engine(weights, max_batch=3, lagged=True)
+    r0 = eng.add_request(prompt(5, 40), SamplingParams(max_new_tokens=16))
+    r1 = eng.add_request(prompt(6, 41), SamplingParams(max_new_tokens=16))
+    for _ in range(5):
+        eng.step()
+    assert eng.runner.continuations > 0
+    eng.abort(r1)
+    late = eng.add_request(prompt(4, 42), SamplingParams(max_new_tokens=6))  # ends the run of continuations
+    done = eng.run_until_complete()
+    assert done[r1].finish_reason == "abort" and len(done[r1].generated) < 16
+    assert done[r1].generated == reference(weights, prompt(6, 41), 16)[: len(done[r1].generated)]
+    assert done[r0].generated == reference(weights, prompt(5, 40), 16)
+    assert done[late].generated == reference(weights, prompt(4, 42), 6)
+    assert eng.manager.num_free_blocks == eng.manager.num_blocks
+
+
+def test_lagged_events_arrive_one_step_later_and_reset_forgets_them(weights):
+    eng = engine(weights, lagged=True)
+    rid = eng.add_request(prompt(5, 4), SamplingParams(max_new_tokens=3))
+    assert eng.step() == []  # the prompt went in; its token has not been read
+    assert eng.has_unfinished()
+    events = eng.step()
+    assert [(e.req_id, e.finished) for e in events] == [(rid, False)]
+    events = eng.step() + eng.step() + eng.step()
+    assert [e.finished for e in events] == [False, True] and not eng.has_unfinished()
+    eng.add_request(prompt(5, 5), SamplingParams(max_new_tokens=3))
+    eng.step()
+    eng.reset()
+    assert not eng.has_unfinished() and eng.manager.num_free_blocks == eng.manager.num_blocks
+    assert eng.step() == []
