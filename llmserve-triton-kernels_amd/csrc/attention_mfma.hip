@@ -73,6 +73,26 @@ __device__ __forceinline__ const bf16* page_ptr(const bf16* base, int page, uint
     return base + (uint64_t)(uint32_t)page * page_stride;  // one 32 x 32 -> 64 bit multiply-add
 }
 
+// Maximum and sum over the four lanes l, l^16, l^32, l^48 that share a column, with gfx950's row swaps
+// (v_permlane32_swap, v_permlane16_swap: the upper half / the odd rows of 16 lanes of one operand change
+// places with the lower half / the even rows of the other), which stay in the vector unit; a lane shuffle
+// would go through LDS four times per tile.
+__device__ __forceinline__ float column_max(float x) {
+    const unsigned xi = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+    const unsigned mi = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+    const auto b = __builtin_amdgcn_permlane16_swap(mi, mi, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+__device__ __forceinline__ float column_sum(float x) {
+    const unsigned xi = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+    const unsigned si = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane16_swap(si, si, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // One tile of 32 keys for a wave's 16 columns: scores, online softmax, weighted values.
 //   kf[u][s]: key rows of score tile u (row i = key 8*(i/4) + 4u + i%4), k-step s;  vf[m]: the lane's 8 keys
 //   (jk .. jk+7) of value dimensions 16m + col, already zero where the key is outside the group's range;
@@ -104,8 +124,7 @@ __device__ __forceinline__ void attend_tile(f32x4 (&acc)[DB], float& m_run, floa
         }
         tmax = fmaxf(tmax, sc[e]);
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, LLMS_WAVE));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, LLMS_WAVE));
+    tmax = column_max(tmax);
     const float m_new = fmaxf(m_run, tmax * scale_log2);  // (scale > 0)
     const float m_safe = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
     if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
@@ -123,9 +142,7 @@ __device__ __forceinline__ void attend_tile(f32x4 (&acc)[DB], float& m_run, floa
         sc[e] = exp2_fast(fmaf(sc[e], scale_log2, -m_safe));
         psum += sc[e];
     }
-    psum += __shfl_xor(psum, 16, LLMS_WAVE);
-    psum += __shfl_xor(psum, 32, LLMS_WAVE);
-    l_run += psum;
+    l_run += column_sum(psum);
     const uint4 pf = make_uint4(pack_bf16(sc[0], sc[1]), pack_bf16(sc[2], sc[3]), pack_bf16(sc[4], sc[5]),
                                 pack_bf16(sc[6], sc[7]));
 #pragma unroll
