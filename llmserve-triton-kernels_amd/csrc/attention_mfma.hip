@@ -367,9 +367,9 @@ __global__ __launch_bounds__(SPLIT_WAVES && DB <= 10 ? 512 : 256) void attn_mfma
 //
 // PAIRED (no window): the causal triangle gives the last tokens of a prompt the most keys, and a workgroup with
 // few keys leaves its CU idle while others still run.  A workgroup then has 8 waves and takes two blocks of
-// tokens, number x from the front and number x from the back: waves 0-3 the late block, whose keys they load
-// for all, waves 4-7 the early block, which sees a prefix of the same keys and stops when it has passed its
-// own position.  Every workgroup of a request then has the same work.
+// tokens, number x from the front and number x from the back: waves 0-3 the late block, waves 4-7 the early
+// block, which sees a prefix of the same keys, stops multiplying when it has passed its own position, and
+// loads the tiles for all.  Every workgroup of a request then has the same work.
 template <int DB, bool PAIRED>
 __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
@@ -404,7 +404,10 @@ __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const A
         wg_first = my_first = blockIdx.x * 4 * TPG;
         if (wg_first >= n_new || ctx <= 0) return;
     }
-    const bool loader = tid < 256;  // waves 0-3 bring the tiles in
+    // The tiles are brought in by the waves that have time for it: those of the early block, which stop
+    // multiplying half way on average (without pairing, by everyone).
+    const bool loader = !PAIRED || tid >= 256;
+    const int ltid = PAIRED ? tid - 256 : tid;
 
     const int t_first = my_first + (wave % 4) * TPG;
     wave_on = wave_on && t_first < n_new;
@@ -462,7 +465,7 @@ __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const A
         if (blk_first < blk_base || block_of(min(j0 + 31, p_max)) >= blk_base + LLMS_WAVE) load_pages(blk_first);
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
-            const int c = tid + 256 * i;
+            const int c = ltid + 256 * i;
             const bool piece_ok = c < PIECES;  // (D < 64: the upper threads have no piece)
             {
                 const int key = min(j0 + (piece_ok ? c / KCH : 0), p_max), ch = piece_ok ? c % KCH : 0;
@@ -485,7 +488,7 @@ __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const A
         const bool inside = j0 >= lo_min && j0 + 31 <= p_max;  // (uniform)
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
-            const int c = tid + 256 * i;
+            const int c = ltid + 256 * i;
             if (c < PIECES) {
                 if (!inside) {
                     const int jk = j0 + 8 * (c % 4);
