@@ -9,16 +9,15 @@
 //   online softmax per column in 32-bit        (max, sum, rescale), masked by position and window
 //   O^T[d, col] += V^T[d, key] . P^T[key, col] A = values, which the cache stores transposed inside
 //                                              a page, so 8 keys of one dimension are one 16-byte load
-// Nothing goes through LDS on the way to the matrix instruction.  The row-to-key assignment of
-// the two S^T tiles is chosen so that each lane ends up with 8 consecutive keys, which is what
-// the B operand of the second product wants: no exchange between lanes.
+// The row-to-key assignment of the two S^T tiles is chosen so that each lane ends up with 8 consecutive
+// keys, which is what the B operand of the second product wants: no exchange between lanes.
 //
-// Arrangements of the waves of a workgroup:
-//   attn_prompt_kernel (prompts): 4 consecutive column groups of one request share each tile of keys through
-//     LDS (the exception to "nothing goes through LDS": 4 waves want the same bytes).
-//   SPLIT_WAVES = false: the same 4 column groups, every wave loading for itself (kept for comparison).
-//   SPLIT_WAVES = true  (decoding): one column group; the key tiles are dealt to the 4 or 8 waves, and
-//     optionally to `num_splits` workgroups whose partial results a second kernel merges.
+// Two kernels, two arrangements of the waves of a workgroup:
+//   attn_mfma_kernel (decoding): one column group; its key tiles are dealt to the 4 or 8 waves, which load
+//     their operands straight from the cache (nothing goes through LDS on the way to the matrix instruction),
+//     and optionally to `num_splits` workgroups whose partial results a second kernel merges.
+//   attn_prompt_kernel (prompts): 4 consecutive column groups of one request want the same keys and share
+//     each tile through LDS; without a window, a block of late tokens and a block of early ones are paired.
 // All merges run in a fixed order, so a token's result does not depend on the batch around it.
 //
 // Needs block_size % 8 == 0, head_dim % 16 == 0 and <= 256, 16-byte aligned rows.
@@ -150,8 +149,8 @@ __device__ __forceinline__ void attend_tile(f32x4 (&acc)[DB], float& m_run, floa
         acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[m]), as_bf16x8(pf), acc[m], 0, 0, 0);
 }
 
-template <int DB, bool SPLIT_WAVES>
-__global__ __launch_bounds__(SPLIT_WAVES && DB <= 10 ? 512 : 256) void attn_mfma_kernel(const AttnArgs a) {
+template <int DB>
+__global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
     constexpr int KS = (D + 31) / 32;  // k-steps of the score product
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
@@ -166,15 +165,9 @@ __global__ __launch_bounds__(SPLIT_WAVES && DB <= 10 ? 512 : 256) void attn_mfma
     const int tok0 = a.cu_seqlens[b], n_new = a.cu_seqlens[b + 1] - tok0;
     const int ctx = a.context_lens[b];
 
-    int tile, split = 0;
-    if (SPLIT_WAVES) {
-        tile = blockIdx.x / a.num_splits;
-        split = blockIdx.x % a.num_splits;
-    } else {
-        tile = blockIdx.x * 4 + wave;
-    }
+    const int tile = blockIdx.x / a.num_splits, split = blockIdx.x % a.num_splits;
     const int t_first = tile * TPG;  // first token (within the request's new tokens) of this group
-    if (t_first >= n_new || ctx <= 0) return;  // (uniform over the workgroup when SPLIT_WAVES)
+    if (t_first >= n_new || ctx <= 0) return;  // (uniform over the workgroup)
 
     // this lane's column
     const int c_tok = t_first + col / HG, c_head_in = hb * HG + col % HG;
@@ -214,13 +207,11 @@ __global__ __launch_bounds__(SPLIT_WAVES && DB <= 10 ? 512 : 256) void attn_mfma
     // first and last tile whose 32 keys every column of the group sees
     const int lo_max = (a.window > 0 && p_max - a.window + 1 > 0) ? p_max - a.window + 1 : 0;
 
-    int t_begin = 0, t_end = n_tiles, t_step = 1;
-    if (SPLIT_WAVES) {
-        const int per_split = (n_tiles + a.num_splits - 1) / a.num_splits;
-        t_begin = split * per_split + wave;
-        t_end = min(n_tiles, (split + 1) * per_split);
-        t_step = blockDim.x / LLMS_WAVE;  // 4 or 8 waves share the keys
-    }
+    // this workgroup's share of the tiles, dealt to its waves
+    const int per_split = (n_tiles + a.num_splits - 1) / a.num_splits;
+    const int t_begin = split * per_split + wave;
+    const int t_end = min(n_tiles, (split + 1) * per_split);
+    const int t_step = blockDim.x / LLMS_WAVE;  // 4 or 8 waves share the keys
     // The request's page ids are held in registers, 64 blocks at a time (lane l: block blk_base + l), and
     // handed around with lane shuffles, so finding a key's page costs no memory access in the loop.
     const int bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
@@ -289,24 +280,9 @@ __global__ __launch_bounds__(SPLIT_WAVES && DB <= 10 ? 512 : 256) void attn_mfma
     }
 
     // acc[m][r] = O^T[d = 16m + 4g + r][col]
-    if (!SPLIT_WAVES) {
-        if (col_ok) {
-            const float inv = 1.f / l_run;
-            bf16* orow = a.out + (size_t)(tok0 + c_tok) * a.out_stride + (size_t)head * D;
-#pragma unroll
-            for (int m = 0; m < DB; ++m) {
-                uint2 w;
-                w.x = pack_bf16(acc[m][0] * inv, acc[m][1] * inv);
-                w.y = pack_bf16(acc[m][2] * inv, acc[m][3] * inv);
-                *reinterpret_cast<uint2*>(orow + 16 * m + 4 * g) = w;
-            }
-        }
-        return;
-    }
-
     // ---- the waves' partial results meet in LDS: every wave leaves its own, then the blocks of 16 dimensions
     // are dealt to the waves, each of which adds the partial results up in the order of the waves
-    constexpr int NW = SPLIT_WAVES ? (DB <= 10 ? 8 : 4) : 1;  // (what the launch bounds allow)
+    constexpr int NW = DB <= 10 ? 8 : 4;  // (what the launch bounds allow)
     __shared__ float sh_acc[NW][DB][LLMS_WAVE][4];
     __shared__ float sh_m[NW][16], sh_l[NW][16];
     const int nw = blockDim.x / LLMS_WAVE;
@@ -586,11 +562,10 @@ static int launch_prompt(int db, dim3 grid, bool paired, const AttnArgs& a, hipS
     return LLMS_OK;
 }
 
-template <bool SPLIT_WAVES>
 static int launch_attn(int db, dim3 grid, int threads, const AttnArgs& a, hipStream_t stream) {
-#define ATT_CASE(N)                                                          \
-    case N:                                                                  \
-        attn_mfma_kernel<N, SPLIT_WAVES><<<grid, threads, 0, stream>>>(a);   \
+#define ATT_CASE(N)                                             \
+    case N:                                                     \
+        attn_mfma_kernel<N><<<grid, threads, 0, stream>>>(a);   \
         break;
     switch (db) {
         ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
@@ -605,7 +580,7 @@ static int launch_attn(int db, dim3 grid, int threads, const AttnArgs& a, hipStr
 extern "C" {
 
 // Attention for the requests [seq_begin, seq_begin + n_seqs) of a step.  max_new: most new tokens any of
-// them brings.  split_waves = 0: prompt portions (keys shared through LDS); -1: the same without LDS;
+// them brings.  split_waves = 0: prompt portions (attn_prompt_kernel);
 // split_waves = 1 deals the keys of each column group to `waves` (4 or 8) waves and
 // `num_splits` workgroups (decoding); with num_splits > 1 the caller provides ws_o [tokens * heads * splits * D] and
 // ws_ml [tokens * heads * splits * 2] floats, indexed by absolute token row.
@@ -627,6 +602,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     LLMS_REQUIRE(num_splits >= 1, "attention_mfma: num_splits must be >= 1");
     LLMS_REQUIRE(scale > 0.f, "attention_mfma: scale must be positive");
     LLMS_REQUIRE((long long)n_kv_heads * block_size * head_dim < (1ll << 31), "attention_mfma: a page is too large");
+    LLMS_REQUIRE(split_waves == 0 || split_waves == 1, "attention_mfma: split_waves is 0 or 1");
     LLMS_REQUIRE(waves == 4 || (split_waves > 0 && waves == 8), "attention_mfma: 4 waves, or 8 when the waves share the keys");
     LLMS_REQUIRE(waves == 4 || head_dim <= 160, "attention_mfma: 8 waves take head_dim up to 160");
     LLMS_REQUIRE(split_waves > 0 || num_splits == 1, "attention_mfma: splits need split_waves");
@@ -640,7 +616,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
     if (split_waves > 0) {
         dim3 grid(groups * num_splits, n_kv_heads * HB, n_seqs);
-        if (int e = launch_attn<true>(head_dim / 16, grid, waves * LLMS_WAVE, a, stream)) return e;
+        if (int e = launch_attn(head_dim / 16, grid, waves * LLMS_WAVE, a, stream)) return e;
         if (num_splits > 1) {
             hipError_t e1 = hipGetLastError();
             if (e1 != hipSuccess) {
@@ -652,9 +628,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
         }
     } else {
         dim3 grid((groups + 3) / 4, n_kv_heads * HB, n_seqs);
-        if (split_waves < 0) {  // the variant that reads every operand straight from global memory
-            if (int e = launch_attn<false>(head_dim / 16, grid, 256, a, stream)) return e;
-        } else if (window == 0 && head_dim <= 192) {  // early and late blocks of tokens paired in one workgroup
+        if (window == 0 && head_dim <= 192) {  // early and late blocks of tokens paired in one workgroup
             // (8 waves of wider heads would not fit the registers)
             grid.x = (grid.x + 1) / 2;
             if (int e = launch_prompt(head_dim / 16, grid, true, a, stream)) return e;

@@ -455,13 +455,12 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
                    seq_begin: int, n_seqs: int, max_new: int, token_begin: int, n_tokens: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, block_size: int, window: int = 0,
                    scale: float | None = None, split_waves: bool = False, num_splits: int = 1,
-                   table_rows: torch.Tensor | None = None, waves: int = 4, through_lds: bool = True) -> torch.Tensor:
+                   table_rows: torch.Tensor | None = None, waves: int = 4) -> torch.Tensor:
     """bfloat16 causal attention on the matrix cores for requests [seq_begin, seq_begin + n_seqs) of a
     step, whose new tokens are rows [token_begin, token_begin + n_tokens) of q and out and bring at most
     `max_new` tokens each.  `split_waves` (with `waves` = 4 or 8 and `num_splits`) spreads each request's keys
     over the waves of a workgroup and over workgroups: the arrangement for single decoded tokens.  Without
-    it the 4 waves of a workgroup take neighbouring tokens and share each tile of keys through LDS
-    (`through_lds=False`: every wave loads for itself)."""
+    it the 4 waves of a workgroup take neighbouring tokens and share each tile of keys through LDS."""
     dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, table_rows)
     _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
     if not attention_mfma_supported(q.dtype, head_dim, block_size):
@@ -499,7 +498,7 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
         c_int(seq_begin),
         c_int(n_seqs), c_int(max_new), c_int(token_begin), c_int(n_tokens), c_int(n_heads), c_int(n_kv_heads),
         c_int(head_dim), c_int(block_size), c_int(window), c_float(scale),
-        c_int(1 if split_waves else 0 if through_lds else -1),
+        c_int(1 if split_waves else 0),
         c_int(num_splits), c_int(waves), _ptr(ws_o), _ptr(ws_ml), _stream(dev)), "attention_mfma")
     return out
 

@@ -438,8 +438,8 @@ def run_attention_mfma(nh, nkv, d, bs, lens, new, window=0, seed=0, craft=None, 
     out = torch.empty(cu[-1], nh * d, dtype=dtype, device=DEV)
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)  # noqa: E731
     ops().attention_mfma(out, q, k_pool.to(DEV), v_pool.to(DEV), tables.to(DEV), i32(cu), i32(lens), 0, len(lens),
-                         max(new), 0, cu[-1], nh, nkv, d, bs, window, None, split_waves=split_waves is True,
-                         num_splits=num_splits, waves=waves, through_lds=split_waves is not None)
+                         max(new), 0, cu[-1], nh, nkv, d, bs, window, None, split_waves=split_waves,
+                         num_splits=num_splits, waves=waves)
     got = out.float().cpu()
     assert torch.isfinite(got).all(), "read a slot that was never written"
     return got, torch.cat(refs)
@@ -463,10 +463,9 @@ MFMA_CASES = [  # nh, nkv, d, bs, lens, new, window
 ]
 
 
-# split_waves: False = prompt arrangement through LDS, None = the same with every wave loading for itself,
-# True = the waves (4 or 8) share the keys, optionally split over workgroups
-@pytest.mark.parametrize("arrangement", [(False, 1, 4), (None, 1, 4), (True, 1, 4), (True, 2, 4), (True, 5, 4), (True, 1, 8),
-                                         (True, 3, 8)])
+# split_waves: False = the prompt kernel (tiles shared through LDS, early and late blocks paired when there is
+# no window), True = the waves (4 or 8) share the keys, optionally split over workgroups
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 4), (True, 2, 4), (True, 5, 4), (True, 1, 8), (True, 3, 8)])
 @pytest.mark.parametrize("case", MFMA_CASES)
 def test_attention_mfma(case, arrangement):
     nh, nkv, d, bs, lens, new, window = case
@@ -481,7 +480,7 @@ def test_attention_mfma(case, arrangement):
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
 
 
-@pytest.mark.parametrize("arrangement", [(False, 1, 4), (None, 1, 4), (True, 1, 4), (True, 3, 4), (True, 1, 8)])
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 4), (True, 3, 4), (True, 1, 8)])
 @pytest.mark.parametrize("needle", [0, 15, 16, 31, 32, 299, 300 - 17, 141])
 def test_attention_mfma_finds_one_far_key(needle, arrangement):
     def craft(qs, ks, vs):
@@ -505,7 +504,7 @@ def test_attention_mfma_window_edge():
             ks[0][needle, :, 1] = 10.0
             vs[0][needle] = 5.0
 
-        for split_waves in (False, None, True):
+        for split_waves in (False, True):
             got, ref = run_attention_mfma(2, 1, 32, 8, [101], [1], 8, seed=61, craft=craft, split_waves=split_waves)
             assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
             assert (got.mean() > 4.0) == inside
