@@ -222,3 +222,128 @@ class StaticDecodeBatch:
         self.dev.copy_(self.host, non_blocking=True)
         self._event = torch.cuda.Event()
         self._event.record(torch.cuda.current_stream(self.dev.device))
+
+
+class StaticStepBatch:
+    """Fixed device buffers for steps of any mixture, so that such steps can be captured as HIP graphs and
+    replayed: up to `decode` requests that bring one token (rows 0 .. decode-1), then up to `prefill`
+    requests that bring portions, `tokens` rows in all, and `logits` wanted rows.  What a step does not
+    use belongs to dummy requests without keys (context length 0, no cache slot), which every kernel
+    leaves alone or computes harmlessly, rows never mixing: the unused decode rows are requests of one
+    token each, the unused prefill requests bring no token, and one last dummy request owns the rows
+    after the last real token."""
+
+    def __init__(self, decode: int, prefill: int, tokens: int, logits: int, storage, group_ids: list[int],
+                 device: torch.device):
+        self.decode, self.prefill, self.tokens, self.logits = decode, prefill, tokens, logits
+        self.storage = storage
+        self.group_ids = list(group_ids)
+        n, b = decode + tokens, decode + prefill + 1
+        self.num_rows, self.num_seqs = n, b
+        self.updates = decode + prefill + -(-tokens // storage.block_size) + 1  # new pages a step can take
+        sizes = [n, n, n, b + 1, b, b, logits]
+        for _ in group_ids:
+            sizes += [n, self.updates, self.updates]
+        self._offsets, total = [], 0
+        for size in sizes:
+            self._offsets.append(total)
+            total += size + (-size % 4)
+        self._sizes = sizes
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(total, dtype=torch.int32, device=device)
+        self._event = None
+        v = self._view
+        groups = {g: GroupView(storage.tables[g], v(7 + 3 * j)) for j, g in enumerate(group_ids)}
+        self.batch = StepBatch(
+            num_tokens=n, num_seqs=b, token_ids=v(0), positions=v(1), token_seq=v(2), cu_seqlens=v(3),
+            context_lens=v(4), state_slots=v(5), logit_rows=v(6), groups=groups,
+            counts=[1] * decode + [0] * prefill + [tokens], starts=[0] * b, state_slot_list=[0] * b,
+            num_decode=decode, max_count=max(tokens, 1), max_context=1, max_decode_context=1)
+        h = self._host_view
+        for j in range(len(group_ids)):
+            h(7 + 3 * j)[:] = -1  # until a step is filled in, no row stores anything
+            h(8 + 3 * j)[:] = -1  # and no block table entry is written
+        h(2)[:decode] = range(decode)
+        h(2)[decode:] = b - 1
+        h(3)[: decode + 1] = range(decode + 1)
+        h(3)[decode + 1: b] = decode
+        h(3)[b] = n
+        self.dev.copy_(self.host)
+
+    def _view(self, i: int) -> torch.Tensor:
+        return self.dev[self._offsets[i]: self._offsets[i] + self._sizes[i]]
+
+    def _host_view(self, i: int):
+        return self.host_np[self._offsets[i]: self._offsets[i] + self._sizes[i]]
+
+    def apply_table_updates(self) -> None:
+        """Write the step's new pages into the device block tables (part of the captured graph)."""
+        from ..ops import library as ops
+
+        for j, g in enumerate(self.group_ids):
+            ops.scatter_i32(self.storage.tables[g], self._view(8 + 3 * j), self._view(9 + 3 * j))
+
+    def fits(self, n_decode: int, n_prefill: int, n_prefill_tokens: int, n_logits: int) -> bool:
+        return (n_decode <= self.decode and n_prefill <= self.prefill and n_prefill_tokens <= self.tokens
+                and n_logits <= self.logits)
+
+    def fill(self, layout: StepLayout, tokens: list[list[int]], logit_rows: list[int]) -> None:
+        """Write a step into the buffers: `layout` lists the requests that bring one token first."""
+        import numpy as np
+
+        counts, starts = layout.counts, layout.starts
+        n_dec = 0
+        while n_dec < len(counts) and counts[n_dec] == 1:
+            n_dec += 1
+        n_pre = len(counts) - n_dec
+        d, b, n = self.decode, self.num_seqs, self.num_rows
+        if self._event is not None:
+            self._event.synchronize()  # the previous copy out of the pinned buffer has finished
+        h = self._host_view
+        tok, pos, seq, cu, ctx, state, rows = (h(i) for i in range(7))
+        tok[:] = 0
+        pos[:] = 0
+        ctx[:] = 0  # dummy requests: no keys, nothing to attend to
+        state[:] = 0
+        # requests of one token
+        tok[:n_dec] = [t[0] for t in tokens[:n_dec]]
+        pos[:n_dec] = starts[:n_dec]
+        ctx[:n_dec] = starts[:n_dec]
+        ctx[:n_dec] += 1
+        state[:n_dec] = layout.state_slots[:n_dec]
+        # portions, end to end from row d; the rows behind them go to the last dummy request
+        row = d
+        for j in range(n_pre):
+            i = n_dec + j
+            c = counts[i]
+            tok[row: row + c] = tokens[i]
+            pos[row: row + c] = np.arange(starts[i], starts[i] + c)
+            seq[row: row + c] = d + j
+            ctx[d + j] = starts[i] + c
+            state[d + j] = layout.state_slots[i]
+            row += c
+            cu[d + j + 1] = row
+        seq[row:] = b - 1
+        cu[d + n_pre + 1: b] = row
+        used = row - d
+        rows[:] = 0
+        shift = d - n_dec  # a row of the step's own numbering that lies behind the decode rows moves by this
+        rows[: len(logit_rows)] = [r if r < n_dec else r + shift for r in logit_rows]
+        for j, g in enumerate(self.group_ids):
+            slots = h(7 + 3 * j)
+            slots[:] = -1  # dummy tokens store nothing
+            own = layout.slots[g]
+            slots[:n_dec] = own[:n_dec]
+            slots[d: d + used] = own[n_dec:]
+            index, value = _update_arrays(layout.table_updates[g], self.storage.table_width, self.storage.max_seqs)
+            k = len(index)
+            if k > self.updates:
+                raise ValueError("more new pages than this batch has room for")
+            ui, uv = h(8 + 3 * j), h(9 + 3 * j)
+            ui[:k] = index
+            ui[k:] = -1
+            uv[:k] = value
+        self.dev.copy_(self.host, non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record(torch.cuda.current_stream(self.dev.device))

@@ -23,7 +23,7 @@ from ..parts.model import Model
 from ..parts.registry import BuildContext
 from ..weights.loader import load_tensors
 from ..weights.random import random_tensors
-from .batch import BatchUploader, StaticDecodeBatch, build_batch
+from .batch import StaticStepBatch, BatchUploader, StaticDecodeBatch, build_batch
 
 _TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
@@ -67,6 +67,12 @@ class ModelRunner:
         self._uploader = BatchUploader(device)
         self._graphs: dict[tuple[int, int], "_DecodeGraph"] = {}
         self._use_graphs = engine_config.use_graphs and model.graph_safe()
+        # graphs of steps that bring portions of prompts, by the sizes they were captured for (most
+        # recently used last); a shape is captured when it comes again after a run that the host could
+        # not keep up with (`_step_shapes`: what was measured when the shape ran kernel by kernel)
+        self._step_graphs: dict[tuple, "_StepGraph"] = {}
+        self._step_shapes: dict[tuple, dict] = {}
+        self._step_graph_pool = None
 
     # ---- construction ---------------------------------------------------------------------
     @staticmethod
@@ -168,8 +174,13 @@ class ModelRunner:
         if self._use_graphs and all(len(e.tokens) == 1 for e in ordered):
             logits = self._replay_decode(layout, [e.tokens[0] for e in ordered], logit_rows, device_tokens)
         else:
-            batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
-            logits = self.model.forward(batch, self.storage)
+            logits = self._replay_step(layout, [e.tokens for e in ordered], logit_rows) if self._use_graphs else None
+            if logits is None:
+                watch = self._watch_eager_step(layout, len(logit_rows)) if self._use_graphs else None
+                batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
+                logits = self.model.forward(batch, self.storage)
+                if watch is not None:
+                    watch()
         self.manager.release_passed(layout.seq_ids)
         return logits
 
@@ -199,6 +210,97 @@ class ModelRunner:
         if logit_rows == list(range(n)):
             return graph.logits[:n]
         return graph.logits[torch.tensor(logit_rows, dtype=torch.long, device=self.device)]
+
+
+    # ---- steps with portions of prompts as HIP graphs ----------------------------------------------
+    MAX_STEP_GRAPHS = 32
+
+    @staticmethod
+    def _step_shape(n_decode: int, n_prefill: int, n_prefill_tokens: int, n_logits: int, context: int) -> tuple:
+        """The sizes a step is padded to: powers of two for the requests, the wanted rows and the reach of
+        the contexts, multiples of 64 (up to 512) or 256 for the rows of the portions."""
+        def pow2(x, least=1):
+            p = least
+            while p < x:
+                p *= 2
+            return p
+        step = 64 if n_prefill_tokens <= 512 else 256
+        return (pow2(n_decode) if n_decode else 0, pow2(n_prefill), -(-n_prefill_tokens // step) * step,
+                pow2(max(n_logits, 1)), pow2(context, 256) if n_decode else 256)  # (the reach matters to decoding only)
+
+    def _shape_of(self, layout, n_logits: int) -> tuple:
+        n_dec = 0
+        while n_dec < len(layout.counts) and layout.counts[n_dec] == 1:
+            n_dec += 1
+        context = max(s + c for s, c in zip(layout.starts, layout.counts))
+        return self._step_shape(n_dec, len(layout.counts) - n_dec, sum(layout.counts[n_dec:]), n_logits, context)
+
+    def _watch_eager_step(self, layout, n_logits: int):
+        """Time a step that is launched kernel by kernel, on the host and on the device; returns the
+        function to call when everything has been launched."""
+        from time import perf_counter
+
+        record = self._step_shapes.setdefault(self._shape_of(layout, n_logits), {})
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(torch.cuda.current_stream(self.device))
+        t0 = perf_counter()
+
+        def done():
+            end.record(torch.cuda.current_stream(self.device))
+            record.update(host_ms=(perf_counter() - t0) * 1e3, start=start, end=end)
+        return done
+
+    def _host_bound(self, record: dict) -> bool:
+        """Whether the last kernel-by-kernel run of this shape kept the device waiting for launches: the
+        device was done about when the host was (a step that keeps the device busy for longer gains nothing
+        from a graph, and capturing one costs two runs)."""
+        end = record.get("end")
+        if end is None or not end.query():
+            return False
+        return record["start"].elapsed_time(end) < 1.5 * record["host_ms"]
+
+    def _replay_step(self, layout, tokens: list[list[int]], logit_rows: list[int]) -> torch.Tensor | None:
+        """A step with portions of prompts, replayed from the graph captured for its padded sizes; None
+        when this shape has no graph (the caller then runs it kernel by kernel).  Launching the ~160
+        kernels of a step one by one costs the host milliseconds; a replay costs microseconds."""
+        shape = self._shape_of(layout, len(logit_rows))
+        graph = self._step_graphs.pop(shape, None)
+        if graph is None:
+            record = self._step_shapes.get(shape)
+            if record is None or not self._host_bound(record):
+                return None
+            if len(self._step_graphs) >= self.MAX_STEP_GRAPHS:
+                self._step_graphs.pop(next(iter(self._step_graphs)))  # the least recently used
+            if self._step_graph_pool is None:
+                self._step_graph_pool = torch.cuda.graph_pool_handle()
+            graph = _StepGraph(self, shape, self._step_graph_pool)
+        self._step_graphs[shape] = graph
+        graph.static.fill(layout, tokens, logit_rows)
+        graph.graph.replay()
+        return graph.logits[: len(logit_rows)]
+
+
+class _StepGraph:
+    """One captured step for up to `decode` single tokens, `prefill` portions of `tokens` rows in all and
+    `logits` wanted rows, contexts up to `reach` (which only sets how decode attention spreads its work).
+    All such graphs share one memory pool: they never run at the same time, and a step's logits are
+    consumed before the next step is replayed."""
+
+    def __init__(self, runner: "ModelRunner", shape: tuple, pool):
+        decode, prefill, tokens, logits, reach = shape
+        group_ids = [g.group_id for g in runner.manager.paged_groups]
+        self.static = StaticStepBatch(decode, prefill, tokens, logits, runner.storage, group_ids, runner.device)
+        batch = self.static.batch
+        batch.max_context = batch.max_decode_context = reach
+        # a first run outside the capture: libraries load, memory pools warm up (the buffers describe
+        # dummy requests only, so nothing is stored or attended to)
+        self.static.apply_table_updates()
+        runner.model.forward(batch, runner.storage)
+        torch.cuda.synchronize(runner.device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, pool=pool):
+            self.static.apply_table_updates()
+            self.logits = runner.model.forward(batch, runner.storage)
 
 
 class _DecodeGraph:

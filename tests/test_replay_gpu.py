@@ -88,6 +88,39 @@ def test_replay_without_graphs(model_dirs, dtype_name, mode):
     check_against_plain(model_dirs["b"], dtype_name, seqs, steps, outputs)
 
 
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_steps_with_portions_are_replayed_from_graphs(model_dirs, dtype_name):
+    """A step shape that comes a second time is captured as a graph (padded to its bucket with dummy
+    requests and rows) and replayed from then on: the mixed and the portioned trace, run twice through one
+    runner, must hit such graphs and still agree with the plain implementation, whatever the padding
+    holds (the cache is poisoned) and whichever pages are used again."""
+    from llmserve.config import EngineConfig
+    from llmserve.engine.replay import Replayer
+    from llmserve.engine.runner import ModelRunner
+
+    name = "a"
+    seqs = sequences(name)
+    block_size = TINY[name][1]
+    for mode in ("mixed", "portions"):
+        steps = MODES[mode](seqs)
+        num_blocks = traces.tokens_needed(steps, round_to=block_size) // block_size
+        runner = ModelRunner.from_folder(model_dirs[name], EngineConfig(dtype=dtype_name, block_size=block_size,
+                                                                        num_blocks=num_blocks, max_num_seqs=4))
+        runner.storage.poison()
+        for _ in range(2):
+            rep = Replayer(runner)
+            outputs = {}
+            for rec in steps:
+                logits = rep.run(rec)
+                runner.manager.check_invariants()
+                if logits.shape[0]:
+                    outputs[rec["step"]] = logits.float().cpu()
+            check_against_plain(model_dirs[name], dtype_name, seqs, steps, outputs)
+            assert runner.manager.num_free_blocks == num_blocks
+        assert runner._step_graphs, f"{mode}: no step with portions was replayed from a graph"
+        assert len(runner._step_graphs) <= runner.MAX_STEP_GRAPHS
+
+
 def test_mixed_trace_reuses_pages(model_dirs):
     """The mixed trace is only a test of reuse if it hands out more pages than the pool has."""
     seqs = sequences("a")
