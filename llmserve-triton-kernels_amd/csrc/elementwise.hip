@@ -30,17 +30,26 @@ __global__ void embed_gather_kernel(T* __restrict__ out, const T* __restrict__ t
 template <typename T>
 __global__ void rmsnorm_kernel(T* __restrict__ out, const T* x, const T* __restrict__ delta, T* resid_out,
                                const T* __restrict__ weight, const int* __restrict__ rows, float eps,
-                               int hidden) {
+                               int hidden, const float* __restrict__ parts, int n_parts, size_t part_stride) {
     __shared__ float red[16];
     const int r = blockIdx.x;
     const int s = rows ? rows[r] : r;
     const T* xs = x + (size_t)s * hidden;
     const T* ds = delta ? delta + (size_t)s * hidden : nullptr;
     T* rs = resid_out ? resid_out + (size_t)s * hidden : nullptr;
+    // delta as partial sums in 32-bit (a product whose K was split): added up in order, rounded as the product
+    // would have rounded its result
+    const float* ps = parts ? parts + (size_t)s * hidden : nullptr;
+    auto delta_at = [&](int i) -> float {
+        if (ds) return to_f32(ds[i]);
+        float d = 0.f;
+        for (int p = 0; p < n_parts; ++p) d += ps[(size_t)p * part_stride + i];
+        return round_to<T>(d);
+    };
     float ss = 0.f;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = to_f32(xs[i]);
-        if (ds) v = round_to<T>(v + to_f32(ds[i]));
+        if (ds || ps) v = round_to<T>(v + delta_at(i));
         if (rs) rs[i] = from_f32<T>(v);
         ss += v * v;
     }
@@ -53,7 +62,7 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, const T* x, const T* __restr
             v = to_f32(rs[i]);  // written by this same thread above
         } else {
             v = to_f32(xs[i]);
-            if (ds) v = round_to<T>(v + to_f32(ds[i]));
+            if (ds || ps) v = round_to<T>(v + delta_at(i));
         }
         o[i] = from_f32<T>(to_f32(weight[i]) * round_to<T>(v * inv));
     }
@@ -64,7 +73,8 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, const T* x, const T* __restr
 #define RV_CHUNKS 4
 __global__ void rmsnorm_bf16_vec_kernel(bf16* __restrict__ out, const bf16* x, const bf16* __restrict__ delta,
                                         bf16* resid_out, const bf16* __restrict__ weight,
-                                        const int* __restrict__ rows, float eps, int hidden) {
+                                        const int* __restrict__ rows, float eps, int hidden,
+                                        const float* __restrict__ parts, int n_parts, size_t part_stride) {
     __shared__ float red[16];
     const int r = blockIdx.x;
     const int s = rows ? rows[r] : r;
@@ -84,12 +94,23 @@ __global__ void rmsnorm_bf16_vec_kernel(bf16* __restrict__ out, const bf16* x, c
             if (ds) {
                 const uint4 dv = ds[i];
                 dw[0] = dv.x; dw[1] = dv.y; dw[2] = dv.z; dw[3] = dv.w;
+            } else if (parts) {  // partial sums in 32-bit, added up in order and rounded as the product would have
+                float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                const float* ps = parts + (size_t)s * hidden + 8 * i;
+                for (int p = 0; p < n_parts; ++p) {
+                    const float4 a = *reinterpret_cast<const float4*>(ps + (size_t)p * part_stride);
+                    const float4 b = *reinterpret_cast<const float4*>(ps + (size_t)p * part_stride + 4);
+                    d[0] += a.x; d[1] += a.y; d[2] += a.z; d[3] += a.w;
+                    d[4] += b.x; d[5] += b.y; d[6] += b.z; d[7] += b.w;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) dw[j] = pack_bf16x2(d[2 * j], d[2 * j + 1]);
             }
             uint32_t ow[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 float lo = bf16_bits_to_f32((uint16_t)(xw[j] & 0xffffu)), hi = bf16_bits_to_f32((uint16_t)(xw[j] >> 16));
-                if (ds) {
+                if (ds || parts) {
                     lo = bf16_bits_to_f32(f32_to_bf16_bits(lo + bf16_bits_to_f32((uint16_t)(dw[j] & 0xffffu))));
                     hi = bf16_bits_to_f32(f32_to_bf16_bits(hi + bf16_bits_to_f32((uint16_t)(dw[j] >> 16))));
                 }
@@ -251,24 +272,29 @@ int llms_embed_gather(int dtype, void* out, const void* table, const int* ids, i
     LLMS_LAUNCH_CHECK();
 }
 
+// parts (nullable, instead of delta): n_parts arrays of 32-bit partial sums, part_stride elements apart, each laid
+// out like x; the delta is their sum, rounded to the dtype of x.
 int llms_rmsnorm(int dtype, void* out, const void* x, const void* delta, void* resid_out, const void* weight,
-                 const int* rows, float eps, int n_rows, int hidden, hipStream_t stream) {
+                 const int* rows, float eps, int n_rows, int hidden, const float* parts, int n_parts,
+                 size_t part_stride, hipStream_t stream) {
     LLMS_REQUIRE(n_rows > 0 && hidden > 0, "rmsnorm: sizes must be positive");
     LLMS_REQUIRE(!(rows && resid_out), "rmsnorm: a row gather cannot also write the residual back");
+    LLMS_REQUIRE(!(parts && delta) && (!parts || n_parts > 0), "rmsnorm: delta or its partial sums, not both");
     if (dtype == 1 && hidden % 8 == 0 && hidden <= 8 * RV_CHUNKS * 256 && ((uintptr_t)x % 16) == 0 &&
         ((uintptr_t)out % 16) == 0 && ((uintptr_t)weight % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0) &&
+        (!parts || (((uintptr_t)parts % 16) == 0 && part_stride % 4 == 0)) &&
         (!resid_out || ((uintptr_t)resid_out % 16) == 0)) {
         const int chunks = hidden / 8;
         const int threads = chunks <= 64 ? 64 : chunks <= 128 ? 128 : 256;
         rmsnorm_bf16_vec_kernel<<<n_rows, threads, 0, stream>>>((bf16*)out, (const bf16*)x, (const bf16*)delta,
                                                                 (bf16*)resid_out, (const bf16*)weight, rows, eps,
-                                                                hidden);
+                                                                hidden, parts, n_parts, part_stride);
         LLMS_LAUNCH_CHECK();
     }
     const int threads = hidden >= 2048 ? 512 : 256;
     DISPATCH_DTYPE(dtype, rmsnorm_kernel<T><<<n_rows, threads, 0, stream>>>(
                               (T*)out, (const T*)x, (const T*)delta, (T*)resid_out, (const T*)weight, rows,
-                              eps, hidden);)
+                              eps, hidden, parts, n_parts, part_stride);)
     LLMS_LAUNCH_CHECK();
 }
 

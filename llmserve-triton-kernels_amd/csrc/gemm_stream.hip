@@ -61,6 +61,7 @@ struct StreamArgs {
     const bf16* bias;
     int M, N, K;
     int num_tiles;  // tiles of 16 weight rows (8 features for the gated and rotary epilogues)
+    int k_splits;   // workgroups that share a tile's K (blockIdx.y); each stores its partial sums, 32-bit, in C[split]
     // NORM
     const bf16* delta;
     const bf16* norm_w;
@@ -132,7 +133,11 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     };
 
     uint4* tile = lds + wave * 16 * (ST_KC / 8);
-    const int chunks = (K + ST_KC - 1) / ST_KC;
+    // this workgroup's chunks of K: all of them, or its share when K is split over workgroups
+    const int all_chunks = (K + ST_KC - 1) / ST_KC;
+    const int per_split = (all_chunks + a.k_splits - 1) / a.k_splits;
+    const int split = blockIdx.y, c_begin = split * per_split;
+    const int chunks = min(all_chunks, c_begin + per_split);
     uint4 wreg[16];
     auto load_weights = [&](int c) {
         const int kl = c * ST_KC + 8 * lane;
@@ -142,7 +147,7 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
             wreg[i] = (n >= 0 && kl < K) ? load_streaming(a.W + (size_t)n * K + kl) : zero;
         }
     };
-    if (wave < chunks) load_weights(wave);  // in flight while the row statistics are computed
+    if (c_begin + wave < chunks) load_weights(c_begin + wave);  // in flight while the row statistics are computed
 
     const bool m_ok = m0 + r16 < M;
     const bf16* xrow = a.X + (size_t)(m_ok ? m0 + r16 : 0) * a.ldx;
@@ -210,7 +215,7 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     }
 
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
-    for (int c = wave; c < chunks; c += ST_WAVES) {
+    for (int c = c_begin + wave; c < chunks; c += ST_WAVES) {
         const int k0 = c * ST_KC;
         uint4 xreg[16];
 #pragma unroll
@@ -244,13 +249,13 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
         return s;
     };
     const int idx = threadIdx.x;
-    TOut* C = reinterpret_cast<TOut*>(a.C);
+    TOut* C = reinterpret_cast<TOut*>(a.C) + (size_t)split * M * a.ldc;  // (one result, or one array of partial sums per split)
 
     if (EPI == EPI_PLAIN) {
         const int i = idx % 16, ml = idx / 16, m = m0 + ml, n = tile_id * 16 + i;  // consecutive threads: consecutive features
         if (m < M && n < N) {
             float s = total_of(i, ml);
-            if (a.bias) s += bf16_bits_to_f32(a.bias[n].bits);
+            if (a.bias && split == 0) s += bf16_bits_to_f32(a.bias[n].bits);
             store_out<TOut>(C + (size_t)m * a.ldc + n, s);
         }
     } else if (EPI == EPI_SWIGLU) {
@@ -309,7 +314,8 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
 #define ST_NORM_LDS_MAX (96 * 1024)  // beside the 64 KB of weight tiles, of the 160 KB a workgroup may hold
 
 template <typename TOut, int EPI>
-static int launch_stream(bool norm, unsigned grid, const StreamArgs& a, hipStream_t stream) {
+static int launch_stream(bool norm, unsigned tiles, const StreamArgs& a, hipStream_t stream) {
+    const dim3 grid(tiles, a.k_splits);
     if (norm) {
         static bool raised = false;  // (per instantiation) allow more dynamic LDS than the default limit
         if (!raised) {
@@ -331,11 +337,13 @@ extern "C" {
 // 2 rotary q/k/v (W = [q; k; v], C = q [M, n_heads*head_dim], k and v stored at `slots` when given).
 // norm_w != null: X is the residual stream, `delta` (nullable) is added to it, the sum goes to resid_out
 // (nullable) and its RMSNorm with norm_w and eps is what is multiplied.  out_dtype: 0 float32, 1 bfloat16.
+// k_splits > 1 (plain epilogue, float32): K is shared out to k_splits workgroups per tile, a short wide matrix
+// then fills the chip; C is [k_splits][M][ldc], partial sums that the caller adds up (bias in the first).
 int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* X, int ldx, const void* W,
                      const void* bias, int M, int N, int K, const void* delta, const void* norm_w, float eps,
                      void* resid_out, int inter, int n_heads, int n_kv_heads, int head_dim, int block_size,
                      const float* inv_freq, const int* positions, const int* slots, void* k_pool, void* v_pool,
-                     hipStream_t stream) {
+                     int k_splits, hipStream_t stream) {
     LLMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_stream: needs 1 <= M <= 64 and positive sizes");
     LLMS_REQUIRE(norm_w == nullptr || (M <= 16 && (size_t)M * (K / 8 + 1) * 16 <= ST_NORM_LDS_MAX),
                  "gemm_stream: the norm prologue takes at most 16 rows and rows * (K + 8) * 2 bytes up to 96 KB");
@@ -350,7 +358,10 @@ int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* 
     } else {
         LLMS_REQUIRE(!delta && !resid_out, "gemm_stream: delta and resid_out need norm_w");
     }
-    StreamArgs a = {C, ldc, (const bf16*)X, ldx, (const bf16*)W, (const bf16*)bias, M, N, K, 0, (const bf16*)delta,
+    LLMS_REQUIRE(k_splits >= 1 && k_splits <= 16, "gemm_stream: k_splits must be in 1..16");
+    LLMS_REQUIRE(k_splits == 1 || (epilogue == EPI_PLAIN && out_dtype == 0 && norm_w == nullptr),
+                 "gemm_stream: K is split for plain 32-bit partial sums only");
+    StreamArgs a = {C, ldc, (const bf16*)X, ldx, (const bf16*)W, (const bf16*)bias, M, N, K, 0, k_splits, (const bf16*)delta,
                     (const bf16*)norm_w, eps, (bf16*)resid_out, inter, n_heads, n_kv_heads, head_dim, block_size,
                     inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool};
     unsigned grid;

@@ -148,10 +148,17 @@ def embed_gather(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> t
 def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, *,
             delta: torch.Tensor | None = None, resid_out: torch.Tensor | None = None,
             rows: torch.Tensor | None = None) -> torch.Tensor:
-    """out[r] = weight * norm(x[s] + delta[s]), s = rows[r] or r; resid_out[s] = x[s] + delta[s]."""
+    """out[r] = weight * norm(x[s] + delta[s]), s = rows[r] or r; resid_out[s] = x[s] + delta[s].
+    `delta` may be a float32 [S, N, hidden] tensor of partial sums (ops.gemm_stream(k_splits=S)): it then
+    stands for their sum in order, rounded to the dtype of x."""
     dev = _dev(out, x, weight, delta, resid_out, rows)
     _rows(x, "x")
     hidden = x.shape[1]
+    parts, n_parts, part_stride = None, 0, 0
+    if delta is not None and delta.dim() == 3:
+        if delta.dtype != torch.float32 or tuple(delta.shape[1:]) != tuple(x.shape) or not delta.is_contiguous():
+            raise ValueError("partial sums must be a contiguous float32 [S, rows, hidden] tensor matching x")
+        parts, n_parts, part_stride, delta = delta, delta.shape[0], delta.stride(0), None
     _rows(out, "out", hidden)
     n_out = out.shape[0]
     if weight.dim() != 1 or weight.numel() != hidden or not weight.is_contiguous():
@@ -173,7 +180,8 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
         return out
     _check(load("elementwise").llms_rmsnorm(
         c_int(_code(x)), _ptr(out), _ptr(x), _ptr(delta), _ptr(resid_out), _ptr(weight), _ptr(rows),
-        c_float(eps), c_int(n_out), c_int(hidden), _stream(dev)), "rmsnorm")
+        c_float(eps), c_int(n_out), c_int(hidden), _ptr(parts), c_int(n_parts), ctypes.c_size_t(part_stride),
+        _stream(dev)), "rmsnorm")
     return out
 
 
@@ -311,7 +319,8 @@ STREAM_NORM_LDS_BYTES = 96 * 1024
 
 
 def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, *,
-                norm: tuple | None = None, swiglu: bool = False, rope: dict | None = None) -> torch.Tensor:
+                norm: tuple | None = None, swiglu: bool = False, rope: dict | None = None,
+                k_splits: int = 1) -> torch.Tensor:
     """The product for up to 64 bfloat16 rows (built for up to 16), with what surrounds it fused in.
 
     plain:   out[M, N] = x w^T (+ bias).
@@ -321,8 +330,16 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
     swiglu:  w = [gate; up] ([2I, K]); out[M, I] = silu(gate) * up.
     rope = dict(n_heads, n_kv_heads, head_dim, inv_freq | None, positions, slots | None, k_pool, v_pool,
              block_size): w = [q; k; v]; out[M, n_heads * head_dim] = rotated q; rotated k and v are stored at
-             the tokens' cache slots."""
+             the tokens' cache slots.
+    k_splits > 1 (plain, float32): out is [k_splits, M, N], partial sums over shares of K (a short, wide
+             matrix then fills the chip); their sum in order is the product, the bias is in the first."""
     dev = _dev(out, x, w, bias)
+    if k_splits != 1:
+        if not 1 < k_splits <= 16 or norm is not None or swiglu or rope is not None:
+            raise ValueError("k_splits is 1..16 and goes with the plain epilogue only")
+        if out.dim() != 3 or out.shape[0] != k_splits or out.dtype != torch.float32 or not out.is_contiguous():
+            raise ValueError("with k_splits the output is a contiguous float32 [k_splits, M, N] tensor")
+        parts, out = out, out[0]
     if x.dim() != 2 or x.stride(1) != 1 or out.dim() != 2 or out.stride(1) != 1:
         raise ValueError("x and out must be 2-d with unit inner stride")
     _rows(w, "w", x.shape[1])
@@ -384,8 +401,8 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
         _ptr(bias), c_int(m), c_int(n), c_int(k), _ptr(delta), _ptr(norm_w), c_float(eps), _ptr(resid_out),
         c_int(inter), c_int(r["n_heads"]), c_int(r["n_kv_heads"]), c_int(r["head_dim"]), c_int(r["block_size"]),
         _ptr(r["inv_freq"]), _ptr(r["positions"]), _ptr(r["slots"]), _ptr(r["k_pool"]), _ptr(r["v_pool"]),
-        _stream(dev)), "gemm_stream")
-    return out
+        c_int(k_splits), _stream(dev)), "gemm_stream")
+    return parts if k_splits != 1 else out
 
 
 # ------------------------------------------------------------------------------ attention

@@ -16,8 +16,8 @@ import math
 import torch
 
 from ..ops import library as ops
-from .linear import few_rows, linear, norm_fusable
-from .registry import POSITION_ENCODINGS, DeferredNorm, Mixer, register_mixer
+from .linear import few_rows, linear, linear_partial_sums, norm_fusable
+from .registry import POSITION_ENCODINGS, DeferredNorm, Mixer, as_tensor, register_mixer
 from .rmsnorm import RMSNorm
 from .spec import PagedCacheSpec, ParamInfo
 
@@ -71,6 +71,7 @@ class Attention(Mixer):
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         view = batch.groups[cache.group_id]
         slots = view.slots if cache.store else None
+        to_a_norm = isinstance(x, DeferredNorm)  # the caller hands the result to a norm, which takes partial sums
         q = self.project_few_rows(x, batch, cache, slots)
         if q is None:
             if isinstance(x, DeferredNorm):
@@ -86,7 +87,7 @@ class Attention(Mixer):
                                    cache.block_size)
         out = torch.empty((q.shape[0], nh * d), dtype=q.dtype, device=q.device)
         self.attend(out, q, cache, view, batch)
-        return linear(out, self.o_weight)
+        return (linear_partial_sums(out, self.o_weight) if to_a_norm else None) or linear(out, self.o_weight)
 
     def _few_rows_unfit(self, rows) -> bool:
         return (rows.dtype != torch.bfloat16 or not few_rows(rows.shape[0], self.qkv_weight) or self.head_dim % 16 != 0
@@ -113,7 +114,7 @@ class Attention(Mixer):
         if deferred:
             new_residual = torch.empty_like(rows) if x.delta is not None else None
             ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias,
-                            norm=(x.delta, x.norm.weight, x.norm.eps, new_residual), rope=rope)
+                            norm=(as_tensor(x.delta), x.norm.weight, x.norm.eps, new_residual), rope=rope)
             x.resolve(new_residual)
         else:
             ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias, rope=rope)

@@ -18,7 +18,9 @@ Interfaces (x is always the flat batch of new tokens, [N, hidden], in the model 
   Block             forward(x, delta, batch, cache) -> (x, delta)   hidden state is x + delta
 
 A mixer or feed-forward that sets `accepts_deferred_norm` is handed a `DeferredNorm` instead of the
-normed tensor and may fold the residual sum and the norm into its own first kernel.
+normed tensor and may fold the residual sum and the norm into its own first kernel.  To such a caller
+it may also return `PartialSums` instead of y: 32-bit partial sums of its last product, which the next
+norm's kernel adds up as it adds the residual.
 """
 
 from __future__ import annotations
@@ -63,16 +65,39 @@ class Norm(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
-    def add_norm(self, residual: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
+    def add_norm(self, residual: torch.Tensor, delta: "torch.Tensor | PartialSums | None") -> torch.Tensor:
+        delta = as_tensor(delta)
         if delta is not None:
             residual.copy_((residual.float() + delta.float()).to(residual.dtype))
         return self.forward(residual)
 
-    def norm_rows(self, x: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
+    def norm_rows(self, x: torch.Tensor, delta: "torch.Tensor | PartialSums | None", rows: torch.Tensor) -> torch.Tensor:
+        delta = as_tensor(delta)
         picked = x[rows.long()]
         if delta is not None:
             picked = (picked.float() + delta[rows.long()].float()).to(x.dtype)
         return self.forward(picked)
+
+
+@dataclass
+class PartialSums:
+    """A part's result y as 32-bit partial sums `parts` [S, N, hidden] of a product whose K was shared out
+    to several workgroups (ops.gemm_stream(k_splits=S)): y is their sum in the order of S, rounded to
+    `dtype`.  Norms take it in the place of `delta`."""
+
+    parts: torch.Tensor
+    dtype: torch.dtype
+
+    def total(self) -> torch.Tensor:
+        acc = self.parts[0].clone()
+        for i in range(1, self.parts.shape[0]):
+            acc += self.parts[i]
+        return acc.to(self.dtype)
+
+
+def as_tensor(delta):
+    """`delta` as a tensor in the model's dtype (None stays None)."""
+    return delta.total() if isinstance(delta, PartialSums) else delta
 
 
 class DeferredNorm:

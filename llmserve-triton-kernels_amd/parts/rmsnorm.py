@@ -6,7 +6,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .registry import Norm, register_norm
+from .registry import PartialSums, Norm, register_norm
 from .spec import ParamInfo
 
 
@@ -32,9 +32,13 @@ class RMSNorm(Norm):
     def add_norm(self, residual, delta):
         if delta is None:
             return self.forward(residual)
+        if isinstance(delta, PartialSums):  # the kernel adds the partial sums up itself
+            delta = delta.parts
         return ops.rmsnorm(torch.empty_like(residual), residual, self.weight, self.eps, delta=delta,
                            resid_out=residual)
 
     def norm_rows(self, x, delta, rows):
         out = torch.empty((rows.numel(), self.hidden), dtype=x.dtype, device=x.device)
+        if isinstance(delta, PartialSums):
+            delta = delta.parts
         return ops.rmsnorm(out, x, self.weight, self.eps, delta=delta, rows=rows)

@@ -10,8 +10,8 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .linear import few_rows, linear, norm_fusable
-from .registry import DeferredNorm, FeedForward, register_feed_forward
+from .linear import few_rows, linear, linear_partial_sums, norm_fusable
+from .registry import DeferredNorm, FeedForward, as_tensor, register_feed_forward
 from .rmsnorm import RMSNorm
 from .spec import ParamInfo
 
@@ -42,18 +42,22 @@ class SwiGLU(FeedForward):
         dtype, device = self.gate_up.dtype, self.gate_up.device
         act = torch.empty((m, self.intermediate), dtype=dtype, device=device)
         few = dtype == torch.bfloat16 and few_rows(m, self.gate_up) and self.intermediate % 8 == 0
+        to_a_norm = isinstance(x, DeferredNorm)  # the caller hands the result to a norm, which takes partial sums
         if isinstance(x, DeferredNorm):
             norm = x.norm
             if (few and norm_fusable(m, x.residual.shape[1]) and isinstance(norm, RMSNorm)
                     and ops.gemm_bf16_supported(x.residual, self.gate_up)):
                 new_residual = torch.empty_like(x.residual) if x.delta is not None else None
-                ops.gemm_stream(act, x.residual, self.gate_up, norm=(x.delta, norm.weight, norm.eps, new_residual),
-                                swiglu=True)
+                ops.gemm_stream(act, x.residual, self.gate_up,
+                                norm=(as_tensor(x.delta), norm.weight, norm.eps, new_residual), swiglu=True)
                 x.resolve(new_residual)
-                return linear(act, self.down)
+                return self._down(act, to_a_norm)
             x = x.materialize()
         if few and ops.gemm_bf16_supported(x, self.gate_up):
             ops.gemm_stream(act, x, self.gate_up, swiglu=True)  # activation in the product's epilogue
         else:
             ops.silu_mul(act, linear(x, self.gate_up))
-        return linear(act, self.down)
+        return self._down(act, to_a_norm)
+
+    def _down(self, act, to_a_norm):
+        return (linear_partial_sums(act, self.down) if to_a_norm else None) or linear(act, self.down)

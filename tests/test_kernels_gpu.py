@@ -72,6 +72,30 @@ def test_rmsnorm(dtype, hidden, eps):
     assert torch.equal(resid.cpu(), x)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,parts", [(64, 2), (96, 3), (2048, 2), (333, 4), (5000, 2)])
+def test_rmsnorm_takes_the_delta_as_partial_sums(dtype, hidden, parts):
+    """The delta as 32-bit partial sums of a product whose K was split: the same bits as the delta they add
+    up to, rounded to the model's dtype, would give."""
+    x = rnd(9, hidden, seed=2, scale=3.0).to(dtype)
+    p = rnd(parts * 9, hidden, seed=3).view(parts, 9, hidden)
+    total = torch.zeros(9, hidden)
+    for i in range(parts):
+        total += p[i]  # the kernel adds in this order
+    delta = total.to(dtype)
+    w = (1 + 0.1 * rnd(hidden, seed=4)).to(dtype)
+    want_resid = x.clone().to(DEV)
+    want = ops().rmsnorm(torch.empty_like(want_resid), want_resid, w.to(DEV), 1e-5, delta=delta.to(DEV), resid_out=want_resid)
+    resid = x.clone().to(DEV)
+    got = ops().rmsnorm(torch.empty_like(resid), resid, w.to(DEV), 1e-5, delta=p.to(DEV), resid_out=resid)
+    assert torch.equal(resid, want_resid) and torch.equal(got, want)
+    rows = torch.tensor([8, 0, 3], dtype=torch.int32, device=DEV)
+    got = ops().rmsnorm(torch.empty(3, hidden, dtype=dtype, device=DEV), x.to(DEV), w.to(DEV), 1e-5, delta=p.to(DEV), rows=rows)
+    assert torch.equal(got, want[rows.long()])
+    with pytest.raises(ValueError, match="partial sums"):
+        ops().rmsnorm(torch.empty_like(resid), resid, w.to(DEV), 1e-5, delta=p[:, :8].contiguous().to(DEV))
+
+
 def test_rmsnorm_tiny_inputs_feel_eps():
     x = rnd(2, 96, seed=5, scale=1e-3)
     w = torch.ones(96)
@@ -169,6 +193,28 @@ def test_gemm_stream_plain(m, n, k):
     ref = x.double() @ w.double().t() + b.double()
     out = ops().gemm_stream(torch.empty(m, n, device=DEV), x.to(DEV), w.to(DEV), b.to(DEV))
     assert (out.cpu().double() - ref).abs().max() <= 2e-6 * math.sqrt(k) * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("m,n,k,splits", [(1, 16, 64, 2), (8, 2048, 2048, 2), (5, 2048, 5632, 4), (16, 100, 5632 + 96, 3),
+                                          (40, 320, 2048, 2), (3, 48, 1024, 16)])
+def test_gemm_stream_k_split_over_workgroups(m, n, k, splits):
+    """K shared out to several workgroups per tile: partial sums whose total is the product (a share may be
+    empty when there are fewer chunks of 512 than splits); the bias is in the first."""
+    x, w, b = rnd(m, k, seed=11).bfloat16(), rnd(n, k, seed=12).bfloat16(), rnd(n, seed=13).bfloat16()
+    ref = x.double() @ w.double().t() + b.double()
+    parts = ops().gemm_stream(torch.full((splits, m, n), 9.0, device=DEV), x.to(DEV), w.to(DEV), b.to(DEV), k_splits=splits)
+    assert parts.shape == (splits, m, n)
+    assert (parts.cpu().double().sum(0) - ref).abs().max() <= 2e-6 * math.sqrt(k) * float(ref.abs().max())
+    chunks = -(-k // 512)
+    per = -(-chunks // splits)
+    for s_ in range(splits):  # each share holds exactly its columns of K
+        lo, hi = min(k, s_ * per * 512), min(k, (s_ + 1) * per * 512)
+        want = x[:, lo:hi].double() @ w[:, lo:hi].double().t() + (b.double() if s_ == 0 else 0)
+        assert (parts[s_].cpu().double() - want).abs().max() <= 2e-6 * math.sqrt(k) * float(ref.abs().max())
+    with pytest.raises(ValueError, match="k_splits"):
+        ops().gemm_stream(torch.empty(splits, m, n, device=DEV), x.to(DEV), w.to(DEV), k_splits=splits, swiglu=True)
+    with pytest.raises(ValueError, match="float32"):
+        ops().gemm_stream(torch.empty(splits, m, n, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV), k_splits=splits)
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96), (37, 5632, 2048), (64, 256, 1024)])
