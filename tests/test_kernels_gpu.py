@@ -541,6 +541,44 @@ def test_attention_mfma_finds_one_far_key(needle, arrangement):
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max()) and got.mean() > 2.9
 
 
+# The kernels keep 64 page ids of a request in registers and fetch the next 64 when a tile leaves them: contexts
+# of more than 64 pages (once and twice over), where random weights would hide a wrong page among hundreds.
+LONG_CASES = [  # nh, nkv, d, bs, lens, new
+    (8, 2, 64, 8, [700], [1]),           # 88 pages: decoding across one refill
+    (4, 1, 32, 8, [1100], [1]),          # 138 pages: two refills
+    (8, 2, 64, 16, [2300], [1]),         # 144 pages of 16
+    (4, 2, 64, 8, [900], [300]),         # a portion of a long prompt: early and late blocks, refills on the way
+    (4, 4, 128, 8, [640, 530], [640, 2]),  # a whole prompt of 80 pages beside the end of another
+]
+
+
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 4), (True, 1, 8), (True, 4, 8), (True, 7, 4)])
+@pytest.mark.parametrize("case", LONG_CASES)
+def test_attention_mfma_long_contexts(case, arrangement):
+    nh, nkv, d, bs, lens, new = case
+    split_waves, num_splits, waves = arrangement
+    got, ref = run_attention_mfma(nh, nkv, d, bs, lens, new, 0, seed=70, split_waves=split_waves,
+                                  num_splits=num_splits, waves=waves)
+    assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 8), (True, 3, 8)])
+@pytest.mark.parametrize("needle", [0, 511, 512, 519, 520, 1023, 1024, 1090])
+def test_attention_mfma_finds_one_key_beyond_the_first_pages(needle, arrangement):
+    """1,100 keys in pages of 8: the one key that matters lies before, at and after the places where the
+    page ids in registers are exchanged (keys 512 and 1024)."""
+    def craft(qs, ks, vs):
+        qs[0][-1] = 0
+        qs[0][-1, :, 0] = 12.0
+        ks[0][:, :, 0] = 0
+        ks[0][needle, :, 0] = 12.0
+        vs[0][needle] = 3.0
+
+    got, ref = run_attention_mfma(4, 1, 32, 8, [1100], [1], 0, seed=71, craft=craft, split_waves=arrangement[0],
+                                  num_splits=arrangement[1], waves=arrangement[2])
+    assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max()) and got.mean() > 2.9
+
+
 def test_attention_mfma_window_edge():
     for needle, inside in ((100 - 8, False), (100 - 7, True)):
         def craft(qs, ks, vs):

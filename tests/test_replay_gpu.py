@@ -171,6 +171,47 @@ def test_long_decoding(model_dirs, dtype_name):
 
 
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_contexts_of_many_pages(tmp_path_factory, dtype_name):
+    """1,300 tokens in pages of 8 (163 pages: the attention kernels hold 64 page ids at a time): the prompt in
+    portions of 512, 300 and what is left, then tokens one by one, beside a second request that is decoding
+    all the while; wanted are the last rows of each portion and every decoded token."""
+    from llmserve.weights import write_random_model
+
+    cfg = dict(TINY["a"][0], max_position_embeddings=2048)
+    model_dir = tmp_path_factory.mktemp(f"long_{dtype_name}")
+    write_random_model(model_dir, cfg, seed=77)
+    vocab = cfg["vocab_size"]
+    seqs = {"long": traces.random_ids(vocab, 1300, 5), "side": traces.random_ids(vocab, 29, 6)}
+    long_ids, side_ids = seqs["long"], seqs["side"]
+    steps, pos, side = [], 0, 8
+    steps.append({"step": 0, "entries": [{"id": "side", "tokens": side_ids[:side], "want": list(range(side))}], "end": []})
+    for n in (512, 300, 470):
+        entries = [{"id": "long", "tokens": long_ids[pos:pos + n], "want": list(range(n - 4, n))},
+                   {"id": "side", "tokens": [side_ids[side]], "want": [0]}]
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+        pos, side = pos + n, side + 1
+    while pos < len(long_ids):
+        entries = [{"id": "long", "tokens": [long_ids[pos]], "want": [0]}]
+        if side < len(side_ids):
+            entries.append({"id": "side", "tokens": [side_ids[side]], "want": [0]})
+            side += 1
+        pos += 1
+        steps.append({"step": len(steps), "entries": entries,
+                      "end": (["long"] if pos == len(long_ids) else []) + (["side"] if side == len(side_ids) and "side" in
+                              [e["id"] for e in entries] else [])})
+    assert side == len(side_ids)
+    outputs = replay_in_process(model_dir, dtype_name, steps, 8, 163 + 5)
+    per_request = traces.collect(steps, outputs, partial=True)
+    dtype = DTYPES[dtype_name]
+    for rid, ids in seqs.items():
+        ref = traces.plain_logits(model_dir, ids, dtype)
+        places = sorted(per_request[rid])
+        got = torch.stack([per_request[rid][p] for p in places])
+        traces.assert_close(got, ref[places], dtype, f"{rid} ({dtype_name})")
+    assert len(per_request["long"]) == 12 + 18 and len(per_request["side"]) == 29
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
 @pytest.mark.parametrize("name", list(TINY))
 def test_first_tokens(model_dirs, name, dtype_name):
     """The first tokens of a sequence: prompts of one, two and three tokens, whole and token by token

@@ -98,8 +98,9 @@ def tokens_needed(steps: list[dict], round_to: int = 64) -> int:
     return most
 
 
-def collect(steps: list[dict], outputs: dict[int, torch.Tensor]) -> dict[str, torch.Tensor]:
-    """Per request the [len, vocab] logits, assembled from per-step outputs."""
+def collect(steps: list[dict], outputs: dict[int, torch.Tensor], partial: bool = False):
+    """Per request the [len, vocab] logits, assembled from per-step outputs (`partial`: only some places
+    were wanted; per request a dict from place to its logits)."""
     rows: dict[str, dict[int, torch.Tensor]] = {}
     length: dict[str, int] = {}
     for rec in steps:
@@ -112,6 +113,8 @@ def collect(steps: list[dict], outputs: dict[int, torch.Tensor]) -> dict[str, to
                 r += 1
             length[e["id"]] = start + len(e["tokens"])
         assert out is None or r == out.shape[0]
+    if partial:
+        return rows
     return {rid: torch.stack([d[i] for i in sorted(d)]) for rid, d in rows.items()}
 
 
