@@ -53,11 +53,6 @@ def ensure_built(dtype_name: str, verbose: bool = True) -> None:
         load(n)
 
 
-def has_mfma() -> bool:
-    """Whether the matrix-core kernels for bfloat16 are part of this build."""
-    return "gemm_mfma" in _build.all_sources()
-
-
 def loaded_libraries() -> dict[str, str]:
     return {k: v._name for k, v in _libs.items()}
 
