@@ -25,7 +25,7 @@ class EngineConfig:
     max_prefill_chunk: int | None = None  # longest portion of one prompt in one step
     max_model_len: int | None = None  # defaults to the model's max_position_embeddings
     seed: int = 0
-    use_graphs: bool = True  # replay decode-only steps from captured HIP graphs
+    use_graphs: bool = True  # replay steps from captured HIP graphs (decode-only steps; others when the host was their limit)
 
     def validate(self) -> None:
         if self.dtype not in DTYPE_NAMES:

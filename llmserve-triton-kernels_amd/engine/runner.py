@@ -4,7 +4,9 @@ the cache that earlier steps left, and returns the logits at the wanted places.
 The reference has no single step function: its scheduler runs one padded forward for new
 prompts and one for decoding requests (src/llmserve/scheduler/engine.py:186-193,236-246).
 Here one call runs everything a step holds as one flat batch: portions of prompts beside
-single decoded tokens, cut anywhere.
+single decoded tokens, cut anywhere.  Steps of single tokens are replayed from HIP graphs (one per
+batch size and context range); so are other steps whose shape comes again after a run in which the
+device waited for the host's launches.
 """
 
 from __future__ import annotations
@@ -23,7 +25,7 @@ from ..parts.model import Model
 from ..parts.registry import BuildContext
 from ..weights.loader import load_tensors
 from ..weights.random import random_tensors
-from .batch import StaticStepBatch, BatchUploader, StaticDecodeBatch, build_batch
+from .batch import BatchUploader, StaticDecodeBatch, StaticStepBatch, build_batch
 
 _TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
