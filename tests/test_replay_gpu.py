@@ -121,6 +121,33 @@ def test_steps_with_portions_are_replayed_from_graphs(model_dirs, dtype_name):
         assert len(runner._step_graphs) <= runner.MAX_STEP_GRAPHS
 
 
+@pytest.fixture(scope="module")
+def wide_model_dir(tmp_path_factory):
+    """Two layers with the sizes of TinyLlama 1.1B (hidden 2048, 32 heads on 4 KV heads, intermediate 5632,
+    vocabulary 32000), random weights."""
+    from llmserve.config import preset
+    from llmserve.weights import write_random_model
+
+    cfg = dict(preset("tinyllama-1.1b"), num_hidden_layers=2)
+    d = tmp_path_factory.mktemp("wide")
+    write_random_model(d, cfg, seed=23)
+    return d, cfg
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_replay_at_full_layer_sizes(wide_model_dir, dtype_name, mode):
+    """The tiny configurations never reach the paths that the sizes of a real model choose: products whose
+    K is shared out to several workgroups and summed by the norm, the library's product for many rows, 8 waves
+    per decoded token, a vocabulary of 2,000 tiles."""
+    model_dir, cfg = wide_model_dir
+    seqs = {f"w{i}": traces.random_ids(cfg["vocab_size"], n, 2000 + i) for i, n in enumerate([40, 150, 300])}
+    steps = MODES[mode](seqs)
+    num_blocks = traces.tokens_needed(steps, round_to=16) // 16
+    outputs = replay_in_process(model_dir, dtype_name, steps, 16, num_blocks)
+    check_against_plain(model_dir, dtype_name, seqs, steps, outputs)
+
+
 def test_mixed_trace_reuses_pages(model_dirs):
     """The mixed trace is only a test of reuse if it hands out more pages than the pool has."""
     seqs = sequences("a")
