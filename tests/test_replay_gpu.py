@@ -121,14 +121,18 @@ def test_steps_with_portions_are_replayed_from_graphs(model_dirs, dtype_name):
         assert len(runner._step_graphs) <= runner.MAX_STEP_GRAPHS
 
 
-@pytest.fixture(scope="module")
-def wide_model_dir(tmp_path_factory):
-    """Two layers with the sizes of TinyLlama 1.1B (hidden 2048, 32 heads on 4 KV heads, intermediate 5632,
-    vocabulary 32000), random weights."""
+WIDE = {  # layer sizes of real models, few layers
+    "tinyllama-1.1b": dict(num_hidden_layers=2),               # hidden 2048, 32 heads on 4 KV heads of 64, 5632, 32000
+    "llama2-7b": dict(num_hidden_layers=1, vocab_size=4000),   # hidden 4096, 32 heads of 128, 11008 (no multiple of 512)
+}
+
+
+@pytest.fixture(scope="module", params=list(WIDE))
+def wide_model_dir(request, tmp_path_factory):
     from llmserve.config import preset
     from llmserve.weights import write_random_model
 
-    cfg = dict(preset("tinyllama-1.1b"), num_hidden_layers=2)
+    cfg = dict(preset(request.param), **WIDE[request.param])
     d = tmp_path_factory.mktemp("wide")
     write_random_model(d, cfg, seed=23)
     return d, cfg
