@@ -311,6 +311,78 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     }
 }
 
+// 17 to 64 rows against a short, wide weight (o_proj, down_proj): K is cut into slices of 512 and a workgroup
+// (blockIdx.y = slice) keeps that slice of all rows of X in LDS, where its 4 waves, each with 16 weight rows of its
+// own, read it as the second operand; with one workgroup per block of 16 rows (above) every workgroup would pull
+// its weights through L2 again.  The weights come straight from memory in the matrix instruction's layout (a lane
+// reads 16 bytes of row l%16 at element 8*(l/16) of each k-step: 64 bytes per row and instruction, and the 16
+// instructions of a wave use every byte of the 1 KB it touches per row), all 16 loads in flight before the first
+// product.  Every slice leaves 32-bit partial sums P[slice][M][N]; the norm kernel that follows adds them up.
+#define SL_KC 512
+#define SL_PITCH (SL_KC * 2 + 16)  // bytes per row of X in LDS: the 16 rows of an operand fall into different banks
+
+template <int MB>  // blocks of 16 rows of X
+__global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_slices_kernel(const bf16* __restrict__ X, int ldx,
+                                                                         const bf16* __restrict__ W,
+                                                                         float* __restrict__ P, int M, int N, int K) {
+    __shared__ __attribute__((aligned(16))) char x_lds[MB * 16 * SL_PITCH];
+    constexpr int THREADS = ST_WAVES * LLMS_WAVE;
+    constexpr int PIECES = MB * 16 * (SL_KC / 8) / THREADS;  // 16-byte pieces of the slice per thread
+    const int tid = threadIdx.x, wave = tid / LLMS_WAVE, lane = tid % LLMS_WAVE, r16 = lane % 16, g = lane / 16;
+    const int slice = blockIdx.y, k0 = slice * SL_KC;
+    // the slice of X (addresses clamped, what lies outside is zeroed when it is stored)
+    uint4 xr[PIECES];
+#pragma unroll
+    for (int p = 0; p < PIECES; ++p) {
+        const int idx = p * THREADS + tid, row = idx / (SL_KC / 8), k = k0 + (idx % (SL_KC / 8)) * 8;
+        const bool ok = row < M && k < K;
+        xr[p] = *reinterpret_cast<const uint4*>(X + (size_t)(ok ? row : 0) * ldx + (ok ? k : 0));
+    }
+    // this wave's 16 weight rows x 512 (clamped likewise: what they meet in X is zero)
+    const int tile = blockIdx.x * ST_WAVES + wave, n = tile * 16 + r16;
+    const bf16* wrow = W + (size_t)(n < N ? n : N - 1) * K;
+    uint4 wr[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        const int k = k0 + 32 * s + 8 * g;
+        wr[s] = load_streaming(wrow + (k < K ? k : 0));
+    }
+    __builtin_amdgcn_sched_barrier(0);  // all loads are issued before anything waits for the first
+#pragma unroll
+    for (int p = 0; p < PIECES; ++p) {
+        const int idx = p * THREADS + tid, row = idx / (SL_KC / 8), piece = idx % (SL_KC / 8);
+        if (!(row < M && k0 + piece * 8 < K)) xr[p] = make_uint4(0, 0, 0, 0);
+        *reinterpret_cast<uint4*>(x_lds + row * SL_PITCH + piece * 16) = xr[p];
+    }
+    __syncthreads();
+    f32x4 acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            const uint4 xv = *reinterpret_cast<const uint4*>(x_lds + (16 * b + r16) * SL_PITCH + 64 * s + 16 * g);
+            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(wr[s]), as_bf16x8(xv), acc[b], 0, 0, 0);
+        }
+    }
+    // acc[b][r] = D[weight row 4g + r][row 16b + r16 of X]
+    float* out = P + (size_t)slice * M * N;
+    const int n0 = tile * 16 + 4 * g;
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+        const int m = 16 * b + r16;
+        if (m >= M || n0 >= N) continue;
+        if (n0 + 3 < N && N % 4 == 0) {
+            *reinterpret_cast<f32x4*>(out + (size_t)m * N + n0) = acc[b];
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n0 + r < N) out[(size_t)m * N + n0 + r] = acc[b][r];
+        }
+    }
+}
+
 #define ST_NORM_LDS_MAX (96 * 1024)  // beside the 64 KB of weight tiles, of the 160 KB a workgroup may hold
 
 template <typename TOut, int EPI>
@@ -391,6 +463,27 @@ int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* 
     else if (epilogue == EPI_SWIGLU) { ST_EPI(EPI_SWIGLU) }
     else { ST_EPI(EPI_ROPE_QKV) }
 #undef ST_EPI
+    LLMS_LAUNCH_CHECK();
+}
+
+// P[slice][M][N] (float32, contiguous) = X[:, slice] * W[:, slice]^T for the ceil(K / 512) slices of K; their sum in
+// order is X * W^T.  For 17 to 64 rows (fewer are taken too) against a weight that is short and wide.
+int llms_gemm_slices(void* P, const void* X, int ldx, const void* W, int M, int N, int K, hipStream_t stream) {
+    LLMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_slices: needs 1 <= M <= 64 and positive sizes");
+    LLMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "gemm_slices: K and the row stride of X must be multiples of 8");
+    LLMS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)P % 16) == 0,
+                 "gemm_slices: X, W and P must be 16-byte aligned");
+    const int slices = (K + SL_KC - 1) / SL_KC, tiles = (N + 15) / 16;
+    LLMS_REQUIRE(slices <= 65535, "gemm_slices: K too large");
+    const dim3 grid((tiles + ST_WAVES - 1) / ST_WAVES, slices);
+    const bf16* x = (const bf16*)X;
+    const bf16* w = (const bf16*)W;
+    switch ((M + 15) / 16) {
+        case 1: gemm_slices_kernel<1><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(x, ldx, w, (float*)P, M, N, K); break;
+        case 2: gemm_slices_kernel<2><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(x, ldx, w, (float*)P, M, N, K); break;
+        case 3: gemm_slices_kernel<3><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(x, ldx, w, (float*)P, M, N, K); break;
+        default: gemm_slices_kernel<4><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(x, ldx, w, (float*)P, M, N, K); break;
+    }
     LLMS_LAUNCH_CHECK();
 }
 

@@ -400,6 +400,34 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
     return parts if k_splits != 1 else out
 
 
+SLICE_K = 512  # what one workgroup of gemm_slices takes of K
+
+
+def gemm_slices(parts: torch.Tensor, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """parts[s] = x[:, 512 s : 512 (s+1)] w[:, likewise]^T for the ceil(K / 512) slices of K: float32
+    [slices, M, N], whose sum in order is x w^T.  For 17 to 64 bfloat16 rows (fewer are taken too) against a
+    short, wide weight: every workgroup keeps its slice of all rows in LDS and reads its weights once."""
+    dev = _dev(parts, x, w)
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise ValueError("x must be 2-d with unit inner stride")
+    _rows(w, "w", x.shape[1])
+    m, k = x.shape
+    n = w.shape[0]
+    if not 0 < m <= 64:
+        raise ValueError("gemm_slices takes 1..64 rows")
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise ValueError("gemm_slices takes bfloat16 operands")
+    if not gemm_bf16_supported(x, w):
+        raise ValueError(f"gemm_slices needs K ({k}) and the row stride of x ({x.stride(0)}) to be multiples of 8 "
+                         "and 16-byte aligned operands")
+    slices = -(-k // SLICE_K)
+    if parts.dtype != torch.float32 or tuple(parts.shape) != (slices, m, n) or not parts.is_contiguous():
+        raise ValueError(f"parts must be a contiguous float32 tensor of shape {(slices, m, n)}")
+    _check(load("gemm_stream").llms_gemm_slices(_ptr(parts), _ptr(x), c_int(x.stride(0)), _ptr(w), c_int(m),
+                                                c_int(n), c_int(k), _stream(dev)), "gemm_slices")
+    return parts
+
+
 # ------------------------------------------------------------------------------ attention
 
 

@@ -68,13 +68,25 @@ def k_splits_for(m: int, weight: torch.Tensor) -> int:
     return max(1, min(SPLIT_K_MAX, SPLIT_K_WORKGROUPS // workgroups, chunks // 2))
 
 
+# 17 to 64 rows against a weight of up to this many bytes: ops.gemm_slices (a slice of all rows in LDS, one
+# array of partial sums per 512 of K).  Measured at 64 rows on 2048 x 2048 and 2048 x 5632: 6.3 and 11.5
+# microseconds against the library's 11.6 and 18.0; the partial sums are a quarter of the weight's bytes at 64
+# rows, written here and read by the norm, which is what a larger weight does not earn back.
+SLICES_MAX_WEIGHT_BYTES = 24e6
+
+
 def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor):
     """x W^T as `PartialSums` (K shared out to several workgroups per tile), or None where that does not
     pay or does not apply; for callers whose result goes to a norm next."""
     from .registry import PartialSums
 
     m = x.shape[0]
-    if not (SPLIT_K and x.dtype == torch.bfloat16 and few_rows(m, weight) and ops.gemm_bf16_supported(x, weight)):
+    if not (SPLIT_K and x.dtype == torch.bfloat16 and ops.gemm_bf16_supported(x, weight)):
+        return None
+    if STREAM_ROWS < m <= STREAM_MAX_ROWS and weight.numel() * 2 <= SLICES_MAX_WEIGHT_BYTES:
+        parts = torch.empty((-(-weight.shape[1] // ops.SLICE_K), m, weight.shape[0]), dtype=torch.float32, device=x.device)
+        return PartialSums(ops.gemm_slices(parts, x, weight), x.dtype)
+    if not few_rows(m, weight):
         return None
     splits = k_splits_for(m, weight)
     if splits < 2:

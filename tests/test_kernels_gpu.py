@@ -217,6 +217,33 @@ def test_gemm_stream_k_split_over_workgroups(m, n, k, splits):
         ops().gemm_stream(torch.empty(splits, m, n, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV), k_splits=splits)
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 2048, 2048), (33, 2048, 5632), (17, 333, 1048), (50, 1002, 520), (24, 64, 176),
+                                   (48, 96, 96), (1, 17, 8), (64, 40, 4096 + 40)])
+def test_gemm_slices(m, n, k):
+    """A slice of all rows in LDS, one array of partial sums per 512 of K: each array holds exactly its columns
+    of K (rows and k-steps that do not exist add nothing, whatever the clamped loads brought), their sum is the
+    product, and what lies around the arrays is not written."""
+    x, w = rnd(m, k, seed=31).bfloat16(), rnd(n, k, seed=32).bfloat16()
+    ref = x.double() @ w.double().t()
+    slices = -(-k // 512)
+    buf = torch.full((slices * m * n + 64,), 7.0, device=DEV)
+    parts = ops().gemm_slices(buf[32:-32].view(slices, m, n), x.to(DEV), w.to(DEV))
+    assert torch.all(buf[:32] == 7.0) and torch.all(buf[-32:] == 7.0)
+    tol = 2e-6 * math.sqrt(k) * float(ref.abs().max())
+    assert (parts.cpu().double().sum(0) - ref).abs().max() <= tol
+    for s_ in range(slices):
+        lo, hi = 512 * s_, min(k, 512 * (s_ + 1))
+        assert (parts[s_].cpu().double() - x[:, lo:hi].double() @ w[:, lo:hi].double().t()).abs().max() <= tol
+    # rows of a larger tensor: the stride of x is not K
+    wide = torch.cat([x, rnd(m, 8, seed=33).bfloat16()], dim=1).to(DEV)
+    again = ops().gemm_slices(torch.empty(slices, m, n, device=DEV), wide[:, :k], w.to(DEV))
+    assert torch.equal(again, parts)
+    with pytest.raises(ValueError, match="shape"):
+        ops().gemm_slices(torch.empty(slices + 1, m, n, device=DEV), x.to(DEV), w.to(DEV))
+    with pytest.raises(ValueError, match="1..64"):
+        ops().gemm_slices(torch.empty(slices, 65, n, device=DEV), rnd(65, k).bfloat16().to(DEV), w.to(DEV))
+
+
 @pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96), (37, 5632, 2048), (64, 256, 1024)])
 def test_gemm_stream_gated_epilogue(m, inter, k):
     """gate and up of the feed-forward in one product over [gate; up], silu(gate) * up in the epilogue:
