@@ -4,6 +4,9 @@ float32: the 32-bit multiply-add kernel, always (no reduced-precision matrix mod
 bfloat16, few rows (decoding): the hand-written kernel that streams the weight once
   (ops.gemm_stream); it takes up to 64 rows, one workgroup per 16 rows and 16 weight rows, so
   beyond 16 rows the weights are re-read from L2 and it only pays for the smaller matrices.
+  A product whose result goes to a norm may be left as 32-bit partial sums over shares of K, which
+  the norm kernel adds up (linear_partial_sums): that fills the chip for a short, wide weight, and
+  for 17 to 64 rows it is ops.gemm_slices, which keeps a slice of all rows in LDS.
 bfloat16, more rows: the library's matrix product (hipBLASLt through torch.mm), which is
   where the reference's engine uses a library too (nn.Linear, src/llmserve/model/llama.py:64-67);
   sums are 32-bit, the result bfloat16 or, for logits, float32.
