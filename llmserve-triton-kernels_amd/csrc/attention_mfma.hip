@@ -16,8 +16,9 @@
 //   attn_mfma_kernel (decoding): one column group; its key tiles are dealt to the 4 or 8 waves, which load
 //     their operands straight from the cache (nothing goes through LDS on the way to the matrix instruction),
 //     and optionally to `num_splits` workgroups whose partial results a second kernel merges.
-//   attn_prompt_kernel (prompts): 4 consecutive column groups of one request want the same keys and share
-//     each tile through LDS; without a window, a block of late tokens and a block of early ones are paired.
+//   attn_prompt_kernel (prompts): consecutive column groups of one request want the same keys and share
+//     each tile through LDS, one or two groups per wave; without a window, a block of late tokens and a block of
+//     early ones are paired.
 // All merges run in a fixed order, so a token's result does not depend on the batch around it.
 //
 // Needs block_size % 8 == 0, head_dim % 16 == 0 and <= 256, 16-byte aligned rows.
@@ -335,25 +336,29 @@ __global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const A
     }
 }
 
-// Prompt portions, 4 consecutive column groups of one request and KV head per workgroup.  The 4 waves walk the
-// same keys, so each tile of 32 keys is fetched once per workgroup: every thread brings a 16-byte piece of the key
-// rows and of the (page-transposed) value rows into LDS, double-buffered, and the waves read their matrix operands
-// from there.  Key rows are stored in the order the score product wants them (row 16u + i holds key 8*(i/4) + 4u + i%4,
-// padded by one chunk per row against bank conflicts); values keep their [dimension][key] order.
+// Prompt portions: a block of WB * CG consecutive column groups of one request and KV head per workgroup, CG per
+// wave.  The WB waves walk the same keys, so each tile of 32 keys is fetched once per workgroup: every thread brings
+// 16-byte pieces of the key rows and of the (page-transposed) value rows into LDS, double-buffered, and the waves
+// read their matrix operands from there.  Key rows are stored in the order the score product wants them (row
+// 16u + i holds key 8*(i/4) + 4u + i%4, padded by one chunk per row against bank conflicts); values keep their
+// [dimension][key] order.  With CG = 2 every key and value fragment that a wave reads from LDS serves 32 columns
+// instead of 16: with head_dim 128 the LDS reads were what the loop waited for (twice the matrix instructions'
+// time), with head_dim 64 it was instruction issue, of which the reads and the loop's own work are a third.
 //
 // PAIRED (no window): the causal triangle gives the last tokens of a prompt the most keys, and a workgroup with
-// few keys leaves its CU idle while others still run.  A workgroup then has 8 waves and takes two blocks of
-// tokens, number x from the front and number x from the back: waves 0-3 the late block, waves 4-7 the early
+// few keys leaves its CU idle while others still run.  A workgroup then has 2 WB waves and takes two blocks of
+// tokens, number x from the front and number x from the back: the first WB waves the late block, the others the early
 // block, which sees a prefix of the same keys, stops multiplying when it has passed its own position, and
 // loads the tiles for all.  Every workgroup of a request then has the same work.
-template <int DB, bool PAIRED>
-__global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const AttnArgs a) {
+template <int DB, bool PAIRED, int CG, int WB>
+__global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
     constexpr int KS = (D + 31) / 32;
     constexpr int KCH = D / 8;          // 16-byte chunks of a key row
     constexpr int KROW = KCH + 1;       // padded row stride in chunks
     constexpr int PIECES = 4 * D;       // chunks of the key tile (32 x KCH) = chunks of the value tile (D x 4)
-    constexpr int PER_THREAD = (PIECES + 255) / 256;
+    constexpr int LT = WB * LLMS_WAVE;  // threads that bring the tiles in
+    constexpr int PER_THREAD = (PIECES + LT - 1) / LT;
     __shared__ uint4 k_lds[2][32 * KROW];
     __shared__ uint4 v_lds[2][D * 4];
     const int tid = threadIdx.x, wave = tid / LLMS_WAVE, lane = tid % LLMS_WAVE;
@@ -369,49 +374,61 @@ __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const A
     // my_first: of the block this wave works for
     int wg_first, my_first;
     bool wave_on = true;
+    const int BLK = WB * CG * TPG;  // tokens of a block: WB waves with CG column groups each
     if (PAIRED) {
-        const int blocks = ((n_new + TPG - 1) / TPG + 3) / 4;
+        const int blocks = (n_new + BLK - 1) / BLK;
         const int late = blocks - 1 - (int)blockIdx.x, early = blockIdx.x;
         if (late < early || ctx <= 0) return;
-        wg_first = late * 4 * TPG;
-        my_first = (wave < 4 ? late : early) * 4 * TPG;
-        wave_on = wave < 4 || early != late;  // (the middle block of an odd number is its own partner)
+        wg_first = late * BLK;
+        my_first = (wave < WB ? late : early) * BLK;
+        wave_on = wave < WB || early != late;  // (the middle block of an odd number is its own partner)
     } else {
-        wg_first = my_first = blockIdx.x * 4 * TPG;
+        wg_first = my_first = blockIdx.x * BLK;
         if (wg_first >= n_new || ctx <= 0) return;
     }
     // The tiles are brought in by the waves that have time for it: those of the early block, which stop
     // multiplying half way on average (without pairing, by everyone).
-    const bool loader = !PAIRED || tid >= 256;
-    const int ltid = PAIRED ? tid - 256 : tid;
+    const bool loader = !PAIRED || tid >= LT;
+    const int ltid = PAIRED ? tid - LT : tid;
 
-    const int t_first = my_first + (wave % 4) * TPG;
-    wave_on = wave_on && t_first < n_new;
-    const int c_tok = t_first + col / HG, c_head_in = hb * HG + col % HG;
-    const bool col_ok = wave_on && col < HG * TPG && c_tok < n_new && c_head_in < G;
-    const int head = kvh * G + c_head_in;
-    const int p_col = col_ok ? ctx - n_new + c_tok : -1;
-    const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
+    // this wave's CG column groups: consecutive tokens, the same heads
+    const int w_first = my_first + (wave % WB) * CG * TPG;
+    wave_on = wave_on && w_first < n_new;
+    const int c_head_in = hb * HG + col % HG, head = kvh * G + c_head_in;
+    int c_tok[CG], p_col[CG], lo_col[CG];
+    bool col_ok[CG];
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg) {
+        c_tok[cg] = w_first + cg * TPG + col / HG;
+        col_ok[cg] = wave_on && col < HG * TPG && c_tok[cg] < n_new && c_head_in < G;
+        p_col[cg] = col_ok[cg] ? ctx - n_new + c_tok[cg] : -1;
+        lo_col[cg] = (a.window > 0 && p_col[cg] - a.window + 1 > 0) ? p_col[cg] - a.window + 1 : 0;
+    }
     // key range of the whole workgroup
-    const int p_max = ctx - n_new + min(wg_first + 4 * TPG, n_new) - 1;
+    const int p_max = ctx - n_new + min(wg_first + BLK, n_new) - 1;
     const int p_min = ctx - n_new + wg_first;
     const int lo_min = (a.window > 0 && p_min - a.window + 1 > 0) ? p_min - a.window + 1 : 0;
     const int j_begin = lo_min & ~31;
     const int n_tiles = (p_max - j_begin) / 32 + 1;
 
     const uint4 zero = make_uint4(0, 0, 0, 0);
-    uint4 qf[KS];
+    uint4 qf[CG][KS];
+    f32x4 acc[CG][DB];
+    float m_run[CG], l_run[CG];
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        const int d = 32 * s + 8 * g;
-        qf[s] = (col_ok && d < D)
-                    ? *reinterpret_cast<const uint4*>(a.q + (size_t)(tok0 + c_tok) * a.q_stride + (size_t)head * D + d)
-                    : zero;
+    for (int cg = 0; cg < CG; ++cg) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const int d = 32 * s + 8 * g;
+            qf[cg][s] = (col_ok[cg] && d < D) ? *reinterpret_cast<const uint4*>(a.q + (size_t)(tok0 + c_tok[cg]) * a.q_stride +
+                                                                                (size_t)head * D + d)
+                                              : zero;
+        }
+#pragma unroll
+        for (int m = 0; m < DB; ++m) acc[cg][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        m_run[cg] = -INFINITY;
+        l_run[cg] = 0.f;
     }
-    f32x4 acc[DB];
-#pragma unroll
-    for (int m = 0; m < DB; ++m) acc[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;
 
     const int* table = a.block_tables + (size_t)(a.table_rows ? a.table_rows[b] : b) * a.max_blocks;
     const uint32_t page_stride = (uint32_t)a.n_kv_heads * a.block_size * D;
@@ -420,8 +437,8 @@ __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const A
     const float scale_log2 = a.scale * 1.44269504088896341f;
     // the tiles whose 32 keys every column of this wave sees: up to the wave's first token, from the window's
     // start of its last one
-    const int w_last = min(t_first + TPG, n_new) - 1;
-    const int w_pmin = ctx - n_new + t_first, w_pmax = ctx - n_new + w_last;
+    const int w_last = min(w_first + CG * TPG, n_new) - 1;
+    const int w_pmin = ctx - n_new + w_first, w_pmax = ctx - n_new + w_last;
     const int w_lo_max = (a.window > 0 && w_pmax - a.window + 1 > 0) ? w_pmax - a.window + 1 : 0;
     const int bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
     auto block_of = [&](int key) { return bs_shift >= 0 ? key >> bs_shift : key / a.block_size; };
@@ -441,7 +458,7 @@ __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const A
         if (blk_first < blk_base || block_of(min(j0 + 31, p_max)) >= blk_base + LLMS_WAVE) load_pages(blk_first);
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
-            const int c = ltid + 256 * i;
+            const int c = ltid + LT * i;
             const bool piece_ok = c < PIECES;  // (D < 64: the upper threads have no piece)
             {
                 const int key = min(j0 + (piece_ok ? c / KCH : 0), p_max), ch = piece_ok ? c % KCH : 0;
@@ -464,7 +481,7 @@ __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const A
         const bool inside = j0 >= lo_min && j0 + 31 <= p_max;  // (uniform)
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
-            const int c = ltid + 256 * i;
+            const int c = ltid + LT * i;
             if (c < PIECES) {
                 if (!inside) {
                     const int jk = j0 + 8 * (c % 4);
@@ -498,10 +515,14 @@ __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const A
             }
 #pragma unroll
         for (int m = 0; m < DB; ++m) vf[m] = v_lds[buf][(16 * m + col) * 4 + g];
-        if (j0 >= w_lo_max && j0 + 31 <= w_pmin)  // (uniform over the wave; columns without a token are discarded)
-            attend_tile<DB, KS, false>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
-        else
-            attend_tile<DB, KS, true>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
+        const bool all_seen = j0 >= w_lo_max && j0 + 31 <= w_pmin;  // (uniform over the wave; columns without a token are discarded)
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg) {  // the same keys and values for each of the wave's column groups
+            if (all_seen)
+                attend_tile<DB, KS, false>(acc[cg], m_run[cg], l_run[cg], kf, vf, qf[cg], j0 + 8 * g, lo_col[cg], p_col[cg], scale_log2);
+            else
+                attend_tile<DB, KS, true>(acc[cg], m_run[cg], l_run[cg], kf, vf, qf[cg], j0 + 8 * g, lo_col[cg], p_col[cg], scale_log2);
+        }
         }
         if (loader && t + 1 < n_tiles) {
             store_tile(buf ^ 1, j0 + 32);  // last read two tiles ago, before the previous barrier
@@ -509,14 +530,16 @@ __global__ __launch_bounds__(PAIRED ? 512 : 256) void attn_prompt_kernel(const A
         }
         __syncthreads();
     }
-    if (col_ok) {
-        const float inv = 1.f / l_run;
-        bf16* orow = a.out + (size_t)(tok0 + c_tok) * a.out_stride + (size_t)head * D;
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg) {
+        if (!col_ok[cg]) continue;
+        const float inv = 1.f / l_run[cg];
+        bf16* orow = a.out + (size_t)(tok0 + c_tok[cg]) * a.out_stride + (size_t)head * D;
 #pragma unroll
         for (int m = 0; m < DB; ++m) {
             uint2 w;
-            w.x = pack_bf16(acc[m][0] * inv, acc[m][1] * inv);
-            w.y = pack_bf16(acc[m][2] * inv, acc[m][3] * inv);
+            w.x = pack_bf16(acc[cg][m][0] * inv, acc[cg][m][1] * inv);
+            w.y = pack_bf16(acc[cg][m][2] * inv, acc[cg][m][3] * inv);
             *reinterpret_cast<uint2*>(orow + 16 * m + 4 * g) = w;
         }
     }
@@ -546,11 +569,16 @@ __global__ void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const 
     }
 }
 
+// Column groups per wave of the prompt kernel: two share every key and value fragment a wave reads from LDS
+// (half the LDS reads and loop overhead per column), as long as the accumulators of both fit the registers.
+#define PROMPT_CG(N) ((N) <= 8 ? 2 : 1)
+#define PROMPT_WB 4  // waves per block of tokens (2 was tried with 2 column groups each: slower)
+
 static int launch_prompt(int db, dim3 grid, bool paired, const AttnArgs& a, hipStream_t stream) {
-#define ATT_CASE(N)                                                                  \
-    case N:                                                                          \
-        if (paired) attn_prompt_kernel<N, true><<<grid, 512, 0, stream>>>(a);        \
-        else attn_prompt_kernel<N, false><<<grid, 256, 0, stream>>>(a);              \
+#define ATT_CASE(N)                                                                                                   \
+    case N:                                                                                                           \
+        if (paired) attn_prompt_kernel<N, true, PROMPT_CG(N), PROMPT_WB><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a); \
+        else attn_prompt_kernel<N, false, PROMPT_CG(N), PROMPT_WB><<<grid, PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);    \
         break;
     switch (db) {
         ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
@@ -627,7 +655,8 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                                                                           token_begin, n_heads, head_dim, num_splits);
         }
     } else {
-        dim3 grid((groups + 3) / 4, n_kv_heads * HB, n_seqs);
+        const int per_block = PROMPT_WB * PROMPT_CG(head_dim / 16);  // column groups of a block of tokens
+        dim3 grid((groups + per_block - 1) / per_block, n_kv_heads * HB, n_seqs);
         if (window == 0 && head_dim <= 192) {  // early and late blocks of tokens paired in one workgroup
             // (8 waves of wider heads would not fit the registers)
             grid.x = (grid.x + 1) / 2;
