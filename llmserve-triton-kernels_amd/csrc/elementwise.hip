@@ -199,6 +199,87 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const float* __restrict__
     }
 }
 
+// bfloat16, head_dim % 16 == 0: the token's head_dim/2 sines and cosines are computed once per workgroup (the angle
+// depends on the token and on i only; computed per element they cost more than the kernel's memory traffic); a
+// thread takes 8 consecutive pairs (i .. i+7 and their partners at + head_dim/2) of one head with 16-byte loads and
+// stores; values leave in 16-byte reads and single stores (transposed in the page).
+__global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restrict__ qkv, const float* __restrict__ inv_freq,
+                                                                  const int* __restrict__ positions,
+                                                                  const int* __restrict__ slots, bf16* __restrict__ k_pool,
+                                                                  bf16* __restrict__ v_pool, int n_tokens, int n_heads,
+                                                                  int n_kv_heads, int head_dim, int block_size) {
+    // Workgroups go round the 8 XCDs; 16 consecutive tokens (whose values are neighbours in a page's rows, 2 bytes
+    // each) go to one XCD, so that its L2 collects them into whole pieces before they are written back.
+    const int xcd = blockIdx.x % 8, place = blockIdx.x / 8;
+    const int n = (place / 16) * 128 + xcd * 16 + place % 16;
+    if (n >= n_tokens) return;
+    const int half = head_dim / 2, chunks = half / 8;
+    const int row_width = (n_heads + 2 * n_kv_heads) * head_dim;
+    bf16* row = qkv + (size_t)n * row_width;
+    const int slot = slots ? slots[n] : -1;
+    const int page = slot >= 0 ? slot / block_size : 0;
+    const int off = slot >= 0 ? slot % block_size : 0;
+    const int c = threadIdx.x % chunks, h0 = threadIdx.x / chunks, h_step = blockDim.x / chunks;
+    // the token's head_dim/2 angles once per workgroup (their sines and cosines are most of this kernel's arithmetic)
+    extern __shared__ float angles[];  // [half] sines, [half] cosines
+    if (inv_freq) {
+        const float pos = (float)positions[n];
+        for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &angles[i], &angles[half + i]);
+        __syncthreads();
+    }
+    if (h0 < h_step) {
+        float sn[8], cs[8];
+        if (inv_freq) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                sn[e] = angles[8 * c + e];
+                cs[e] = angles[half + 8 * c + e];
+            }
+        }
+        const int rot_heads = n_heads + n_kv_heads;
+        for (int h = h0; h < rot_heads; h += h_step) {
+            bf16* x = row + (size_t)h * head_dim + 8 * c;
+            const uint4 av = *reinterpret_cast<const uint4*>(x), bv = *reinterpret_cast<const uint4*>(x + half);
+            const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
+            uint32_t ra[4] = {aw[0], aw[1], aw[2], aw[3]}, rb[4] = {bw[0], bw[1], bw[2], bw[3]};
+            if (inv_freq) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float lo_a[2], lo_b[2];
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const float a = bf16_bits_to_f32((uint16_t)(u ? aw[j] >> 16 : aw[j] & 0xffffu));
+                        const float b = bf16_bits_to_f32((uint16_t)(u ? bw[j] >> 16 : bw[j] & 0xffffu));
+                        lo_a[u] = a * cs[2 * j + u] - b * sn[2 * j + u];
+                        lo_b[u] = b * cs[2 * j + u] + a * sn[2 * j + u];
+                    }
+                    ra[j] = pack_bf16x2(lo_a[0], lo_a[1]);
+                    rb[j] = pack_bf16x2(lo_b[0], lo_b[1]);
+                }
+            }
+            bf16* dst = x;
+            if (h >= n_heads && k_pool != nullptr) {
+                if (slot < 0) continue;
+                dst = k_pool + (((size_t)page * n_kv_heads + (h - n_heads)) * block_size + off) * head_dim + 8 * c;
+            }
+            *reinterpret_cast<uint4*>(dst) = make_uint4(ra[0], ra[1], ra[2], ra[3]);
+            *reinterpret_cast<uint4*>(dst + half) = make_uint4(rb[0], rb[1], rb[2], rb[3]);
+        }
+    }
+    if (slot >= 0) {
+        const bf16* v = row + (size_t)(n_heads + n_kv_heads) * head_dim;
+        for (int t = threadIdx.x; t < n_kv_heads * head_dim / 8; t += blockDim.x) {
+            const uint4 vv = *reinterpret_cast<const uint4*>(v + 8 * t);
+            const uint32_t vw[4] = {vv.x, vv.y, vv.z, vv.w};
+            const int kvh = (8 * t) / head_dim, d = (8 * t) % head_dim;
+            bf16* dst = v_pool + (((size_t)page * n_kv_heads + kvh) * head_dim + d) * block_size + off;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                dst[(size_t)e * block_size].bits = (uint16_t)(e & 1 ? vw[e / 2] >> 16 : vw[e / 2] & 0xffffu);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ SiLU(gate) * up
 // gate_up row = [gate (inter) | up (inter)]; out = T(T(silu(gate)) * up), the reference's
 // rounding points (src/llmserve/model/llama.py:120).
@@ -305,6 +386,14 @@ int llms_rope_store(int dtype, void* qkv, const float* inv_freq, const int* posi
     LLMS_REQUIRE(head_dim > 0 && head_dim % 2 == 0, "rope_store: head_dim must be even");
     LLMS_REQUIRE(block_size > 0, "rope_store: block_size must be positive");
     LLMS_REQUIRE(slots == nullptr || (k_pool && v_pool), "rope_store: slots given without pools");
+    if (dtype == 1 && head_dim % 16 == 0 && head_dim <= 4096 && ((uintptr_t)qkv % 16) == 0 &&
+        (k_pool == nullptr || ((uintptr_t)k_pool % 16) == 0)) {
+        const unsigned grid = (unsigned)((n_tokens + 127) / 128 * 128);
+        rope_store_bf16_vec_kernel<<<grid, 256, head_dim * sizeof(float), stream>>>(
+            (bf16*)qkv, inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool, n_tokens, n_heads, n_kv_heads, head_dim,
+            block_size);
+        LLMS_LAUNCH_CHECK();
+    }
     DISPATCH_DTYPE(dtype, rope_store_kernel<T><<<n_tokens, 256, 0, stream>>>(
                               (T*)qkv, inv_freq, positions, slots, (T*)k_pool, (T*)v_pool, n_heads,
                               n_kv_heads, head_dim, block_size);)
