@@ -78,6 +78,18 @@ def k_splits_for(m: int, weight: torch.Tensor) -> int:
 SLICES_MAX_WEIGHT_BYTES = 24e6
 
 
+# Where the sums need a kernel of their own (the projection to q, k, v: sum, rotation, store), from this many rows on;
+# below, the streaming kernel with its epilogue is faster (32 rows: 8.6 against 5.0 + 5 microseconds).
+SLICES_MIN_ROWS_OWN_SUM = 33
+
+
+def slices_pay(m: int, weight: torch.Tensor, sum_is_free: bool = True) -> bool:
+    """Whether `m` bfloat16 rows against `weight` are best left as partial sums per slice of K (ops.gemm_slices).
+    `sum_is_free`: a kernel that runs anyway (the norm) adds them up."""
+    least = STREAM_ROWS + 1 if sum_is_free else SLICES_MIN_ROWS_OWN_SUM
+    return SPLIT_K and least <= m <= STREAM_MAX_ROWS and weight.numel() * 2 <= SLICES_MAX_WEIGHT_BYTES
+
+
 def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor):
     """x W^T as `PartialSums` (K shared out to several workgroups per tile), or None where that does not
     pay or does not apply; for callers whose result goes to a norm next."""
@@ -86,7 +98,7 @@ def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor):
     m = x.shape[0]
     if not (SPLIT_K and x.dtype == torch.bfloat16 and ops.gemm_bf16_supported(x, weight)):
         return None
-    if STREAM_ROWS < m <= STREAM_MAX_ROWS and weight.numel() * 2 <= SLICES_MAX_WEIGHT_BYTES:
+    if slices_pay(m, weight):
         parts = torch.empty((-(-weight.shape[1] // ops.SLICE_K), m, weight.shape[0]), dtype=torch.float32, device=x.device)
         return PartialSums(ops.gemm_slices(parts, x, weight), x.dtype)
     if not few_rows(m, weight):
