@@ -570,15 +570,23 @@ __global__ void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const 
 }
 
 // Column groups per wave of the prompt kernel: two share every key and value fragment a wave reads from LDS
-// (half the LDS reads and loop overhead per column), as long as the accumulators of both fit the registers.
-#define PROMPT_CG(N) ((N) <= 8 ? 2 : 1)
+// (half the LDS reads and loop overhead per column), as long as the accumulators of both fit the registers and
+// the launch still has a workgroup for every CU.
+#define PROMPT_CG_MAX(N) ((N) <= 8 ? 2 : 1)
 #define PROMPT_WB 4  // waves per block of tokens (2 was tried with 2 column groups each: slower)
+#define PROMPT_FULL_CHIP 256  // workgroups below which one column group per wave is kept
 
-static int launch_prompt(int db, dim3 grid, bool paired, const AttnArgs& a, hipStream_t stream) {
-#define ATT_CASE(N)                                                                                                   \
-    case N:                                                                                                           \
-        if (paired) attn_prompt_kernel<N, true, PROMPT_CG(N), PROMPT_WB><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a); \
-        else attn_prompt_kernel<N, false, PROMPT_CG(N), PROMPT_WB><<<grid, PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);    \
+template <int DB, int CG>
+static void launch_prompt_cg(dim3 grid, bool paired, const AttnArgs& a, hipStream_t stream) {
+    if (paired) attn_prompt_kernel<DB, true, CG, PROMPT_WB><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
+    else attn_prompt_kernel<DB, false, CG, PROMPT_WB><<<grid, PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
+}
+
+static int launch_prompt(int db, int cg, dim3 grid, bool paired, const AttnArgs& a, hipStream_t stream) {
+#define ATT_CASE(N)                                                                       \
+    case N:                                                                               \
+        if (cg == 2 && PROMPT_CG_MAX(N) == 2) launch_prompt_cg<N, PROMPT_CG_MAX(N)>(grid, paired, a, stream); \
+        else launch_prompt_cg<N, 1>(grid, paired, a, stream);                             \
         break;
     switch (db) {
         ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
@@ -655,15 +663,18 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                                                                           token_begin, n_heads, head_dim, num_splits);
         }
     } else {
-        const int per_block = PROMPT_WB * PROMPT_CG(head_dim / 16);  // column groups of a block of tokens
-        dim3 grid((groups + per_block - 1) / per_block, n_kv_heads * HB, n_seqs);
-        if (window == 0 && head_dim <= 192) {  // early and late blocks of tokens paired in one workgroup
-            // (8 waves of wider heads would not fit the registers)
-            grid.x = (grid.x + 1) / 2;
-            if (int e = launch_prompt(head_dim / 16, grid, true, a, stream)) return e;
-        } else {
-            if (int e = launch_prompt(head_dim / 16, grid, false, a, stream)) return e;
-        }
+        const bool paired = window == 0 && head_dim <= 192;  // early and late blocks of tokens in one workgroup
+        // (8 waves of wider heads would not fit the registers)
+        auto grid_for = [&](int cg) {
+            const int per_block = PROMPT_WB * cg;  // column groups of a block of tokens
+            dim3 grid((groups + per_block - 1) / per_block, n_kv_heads * HB, n_seqs);
+            if (paired) grid.x = (grid.x + 1) / 2;
+            return grid;
+        };
+        int cg = PROMPT_CG_MAX(head_dim / 16);
+        dim3 grid = grid_for(cg);
+        if (cg == 2 && (long long)grid.x * grid.y * grid.z < PROMPT_FULL_CHIP) grid = grid_for(cg = 1);
+        if (int e = launch_prompt(head_dim / 16, cg, grid, paired, a, stream)) return e;
     }
     LLMS_LAUNCH_CHECK();
 }
