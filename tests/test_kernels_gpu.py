@@ -6,10 +6,9 @@ import math
 
 import pytest
 import torch
-import torch.nn.functional as F
 
 import plain_llama
-from kernel_helpers import attention_reference, bf16_round, make_paged
+from kernel_helpers import attention_reference, make_paged
 
 pytestmark = pytest.mark.gpu
 

@@ -5,7 +5,6 @@ with so few pages that they are used again.  32-bit and bfloat16, both tiny conf
 import json
 import os
 import subprocess
-import sys
 
 import numpy as np
 import pytest
