@@ -68,6 +68,27 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, const T* x, const T* __restr
     }
 }
 
+// d[0..7] += the 8 consecutive floats at `ps` of each of n_parts arrays, part_stride elements apart, in the order of
+// the arrays; the loads of four arrays are in flight together (one after the other, each would wait for memory).
+__device__ __forceinline__ void sum_parts8(float (&d)[8], const float* __restrict__ ps, int n_parts, size_t part_stride) {
+    for (int p0 = 0; p0 < n_parts; p0 += 4) {
+        float4 a[4], b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float* src = ps + (size_t)min(p0 + j, n_parts - 1) * part_stride;  // (clamped: loaded, not added)
+            a[j] = *reinterpret_cast<const float4*>(src);
+            b[j] = *reinterpret_cast<const float4*>(src + 4);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (p0 + j < n_parts) {
+                d[0] += a[j].x; d[1] += a[j].y; d[2] += a[j].z; d[3] += a[j].w;
+                d[4] += b[j].x; d[5] += b[j].y; d[6] += b[j].z; d[7] += b[j].w;
+            }
+        }
+    }
+}
+
 // The same for bfloat16 rows of hidden % 8 == 0 and hidden <= 8 * RV_CHUNKS * blockDim: every thread keeps
 // its elements in registers (16-byte loads and stores), so the row is read once.
 #define RV_CHUNKS 4
@@ -97,12 +118,7 @@ __global__ void rmsnorm_bf16_vec_kernel(bf16* __restrict__ out, const bf16* x, c
             } else if (parts) {  // partial sums in 32-bit, added up in order and rounded as the product would have
                 float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 const float* ps = parts + (size_t)s * hidden + 8 * i;
-                for (int p = 0; p < n_parts; ++p) {
-                    const float4 a = *reinterpret_cast<const float4*>(ps + (size_t)p * part_stride);
-                    const float4 b = *reinterpret_cast<const float4*>(ps + (size_t)p * part_stride + 4);
-                    d[0] += a.x; d[1] += a.y; d[2] += a.z; d[3] += a.w;
-                    d[4] += b.x; d[5] += b.y; d[6] += b.z; d[7] += b.w;
-                }
+                sum_parts8(d, ps, n_parts, part_stride);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) dw[j] = pack_bf16x2(d[2 * j], d[2 * j + 1]);
             }
@@ -234,11 +250,7 @@ __global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restri
     auto load8 = [&](int col) -> uint4 {
         if (!PARTS) return *reinterpret_cast<const uint4*>(row + col);
         float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int p = 0; p < src.n_parts; ++p) {
-            const float4* ps = reinterpret_cast<const float4*>(src.parts + p * src.part_stride + (size_t)n * row_width + col);
-            const float4 lo = ps[0], hi = ps[1];
-            f[0] += lo.x, f[1] += lo.y, f[2] += lo.z, f[3] += lo.w, f[4] += hi.x, f[5] += hi.y, f[6] += hi.z, f[7] += hi.w;
-        }
+        sum_parts8(f, src.parts + (size_t)n * row_width + col, src.n_parts, src.part_stride);
         if (src.bias) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) f[e] += bf16_bits_to_f32(src.bias[col + e].bits);
