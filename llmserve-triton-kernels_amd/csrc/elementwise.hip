@@ -138,15 +138,22 @@ __global__ void rmsnorm_bf16_vec_kernel(bf16* __restrict__ out, const bf16* x, c
             if (rs) rs[i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
         }
     }
+    // the norm's weight is asked for before the barriers of the sum, behind which it would cost a trip to memory
+    const uint4* ws = reinterpret_cast<const uint4*>(weight);
+    uint4 wreg[RV_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < RV_CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nchunks) wreg[c] = ws[i];
+    }
     ss = block_sum(ss, red);
     const float inv = rsqrtf(ss / (float)hidden + eps);
-    const uint4* ws = reinterpret_cast<const uint4*>(weight);
     uint4* o = reinterpret_cast<uint4*>(out + (size_t)r * hidden);
 #pragma unroll
     for (int c = 0; c < RV_CHUNKS; ++c) {
         const int i = threadIdx.x + c * blockDim.x;
         if (i < nchunks) {
-            const uint4 wv = ws[i];
+            const uint4 wv = wreg[c];
             const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
             uint32_t ow[4];
 #pragma unroll

@@ -152,6 +152,20 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     const bool m_ok = m0 + r16 < M;
     const bf16* xrow = a.X + (size_t)(m_ok ? m0 + r16 : 0) * a.ldx;
 
+    // what the rotary epilogue needs of its token (thread -> row idx / 8 or idx / 16 of X) is asked for now: after
+    // the last barrier it would cost a trip to memory at the end of the kernel
+    int epi_pos = 0, epi_slot = -1, epi_slot_v = -1;
+    float epi_freq = 0.f;
+    if (EPI == EPI_ROPE_QKV) {
+        const int m8 = m0 + (int)threadIdx.x / 8, m16 = m0 + (int)threadIdx.x / 16;
+        if (threadIdx.x < 128 && m8 < M) {
+            if (a.inv_freq) epi_pos = a.positions[m8];
+            if (a.slots) epi_slot = a.slots[m8];
+            if (a.inv_freq && tile_id < rot_tiles) epi_freq = a.inv_freq[8 * (tile_id % spt) + (int)threadIdx.x % 8];
+        }
+        if (a.slots && m16 < M) epi_slot_v = a.slots[m16];
+    }
+
     // ---- NORM: summed residual, statistics and normed rows, kept in LDS as h[row][K/8 + 1] chunks of 8
     extern __shared__ uint4 h_lds[];
     const int hstride = K / 8 + 1;  // (one chunk of padding: the 16 rows of a matrix operand fall into different banks)
@@ -280,7 +294,7 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
                 float ra = lo, rb = hi;
                 if (a.inv_freq) {
                     float sn, cs;
-                    sincosf((float)a.positions[m] * a.inv_freq[d], &sn, &cs);
+                    sincosf((float)epi_pos * epi_freq, &sn, &cs);
                     ra = lo * cs - hi * sn;
                     rb = hi * cs + lo * sn;
                 }
@@ -288,7 +302,7 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
                     store_out<TOut>(C + (size_t)m * a.ldc + h * D + d, ra);
                     store_out<TOut>(C + (size_t)m * a.ldc + h * D + d + D / 2, rb);
                 } else {
-                    const int slot = a.slots ? a.slots[m] : -1;
+                    const int slot = epi_slot;
                     if (slot >= 0) {
                         const int page = slot / bs, off = slot % bs;
                         bf16* dst = a.k_pool + (((size_t)page * nkv + (h - nh)) * bs + off) * D;
@@ -299,7 +313,7 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
             }
         } else {
             const int i = idx % 16, ml = idx / 16, m = m0 + ml;
-            const int slot = (a.slots && m < M) ? a.slots[m] : -1;
+            const int slot = epi_slot_v;
             if (m < M && slot >= 0) {
                 const int f = (tile_id - rot_tiles) * 16 + i;  // feature among the value heads
                 float v = total_of(i, ml);
