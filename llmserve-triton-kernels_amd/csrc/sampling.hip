@@ -36,11 +36,18 @@ __device__ __forceinline__ int block_argmax(const float* __restrict__ row, int v
                                             float* max_out) {
     float best = -INFINITY;
     int besti = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-        const float v = row[i];
-        if (v > best || (v == best && i < besti)) {
-            best = v;
-            besti = i;
+    // eight loads of a thread are in flight together (one after the other, each would wait for memory)
+    for (int base = threadIdx.x; base < vocab; base += 8 * SAMPLE_THREADS) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = row[min(base + j * SAMPLE_THREADS, vocab - 1)];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = base + j * SAMPLE_THREADS;
+            if (i < vocab && (v[j] > best || (v[j] == best && i < besti))) {
+                best = v[j];
+                besti = i;
+            }
         }
     }
 #pragma unroll
