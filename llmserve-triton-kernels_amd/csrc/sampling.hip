@@ -31,23 +31,19 @@ __device__ __forceinline__ uint32_t block_sum_u32(uint32_t v, uint32_t* lds) {
     return t;
 }
 
-// argmax over a row; returns the same (value, index) to every thread.
-__device__ __forceinline__ int block_argmax(const float* __restrict__ row, int vocab, float* fl, int* il,
-                                            float* max_out) {
+// argmax over a row; returns the same (value, index) to every thread.  `value(j)` is the thread's j-th logit (element
+// threadIdx.x + j * SAMPLE_THREADS of the row), for j < nj.
+template <typename F>
+__device__ __forceinline__ int block_argmax(F value, int nj, int vocab, float* fl, int* il, float* max_out) {
     float best = -INFINITY;
     int besti = 0x7fffffff;
-    // eight loads of a thread are in flight together (one after the other, each would wait for memory)
-    for (int base = threadIdx.x; base < vocab; base += 8 * SAMPLE_THREADS) {
-        float v[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = row[min(base + j * SAMPLE_THREADS, vocab - 1)];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int i = base + j * SAMPLE_THREADS;
-            if (i < vocab && (v[j] > best || (v[j] == best && i < besti))) {
-                best = v[j];
-                besti = i;
-            }
+    for (int j = 0; j < nj; ++j) {
+        const int i = threadIdx.x + j * SAMPLE_THREADS;
+        const float v = value(j);
+        if (i < vocab && (v > best || (v == best && i < besti))) {
+            best = v;
+            besti = i;
         }
     }
 #pragma unroll
@@ -79,6 +75,10 @@ __device__ __forceinline__ int block_argmax(const float* __restrict__ row, int v
     return besti;
 }
 
+// VPT > 0: the row (vocab <= VPT * SAMPLE_THREADS) is read once and kept in registers, VPT logits per thread, for
+// the up to 70 passes that follow (a pass over memory waits for every load in turn).  VPT = 0: any vocabulary, every
+// pass reads the row again.
+template <int VPT>
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
     int* __restrict__ out, const float* __restrict__ logits, int ld, int vocab,
     const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
@@ -89,8 +89,19 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
     __shared__ int found;
     const int r = blockIdx.x;
     const float* row = logits + (size_t)r * ld;
+    const int nj = VPT > 0 ? VPT : (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+    float held[VPT > 0 ? VPT : 1];
+    if (VPT > 0) {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) held[j] = row[min((int)threadIdx.x + j * SAMPLE_THREADS, vocab - 1)];
+    }
+    // the thread's j-th logit (callers check that its index is below vocab)
+    auto raw = [&](int j) -> float {
+        if (VPT > 0) return held[j];
+        return row[min((int)threadIdx.x + j * SAMPLE_THREADS, vocab - 1)];
+    };
     float zmax_raw;
-    const int amax = block_argmax(row, vocab, fl, il, &zmax_raw);
+    const int amax = block_argmax(raw, nj, vocab, fl, il, &zmax_raw);
     const float T = temperature ? temperature[r] : 0.f;
     if (!(T > 0.f)) {
         if (threadIdx.x == 0) out[r] = amax;
@@ -106,7 +117,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
         for (int bit = 31; bit >= 0; --bit) {
             const uint32_t cand = t | (1u << bit);
             uint32_t c = 0;
-            for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) c += order_key(row[i] * inv_t) >= cand;
+#pragma unroll
+            for (int j = 0; j < nj; ++j)
+                if ((int)threadIdx.x + j * SAMPLE_THREADS < vocab) c += order_key(raw(j) * inv_t) >= cand;
             if (block_sum_u32(c, ul) >= (uint32_t)k) t = cand;
         }
         thr = t;  // key of the k-th largest
@@ -114,9 +127,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
     const float p = top_p ? top_p[r] : 1.f;
     if (p < 1.f) {
         float e = 0.f;
-        for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-            const float z = row[i] * inv_t;
-            if (order_key(z) >= thr) e += expf(z - zmax);
+#pragma unroll
+        for (int j = 0; j < nj; ++j) {
+            const float z = raw(j) * inv_t;
+            if ((int)threadIdx.x + j * SAMPLE_THREADS < vocab && order_key(z) >= thr) e += expf(z - zmax);
         }
         const float limit = p * block_sum(e, fl);
         // largest t whose mass strictly above it still exceeds the limit; survivors are > t
@@ -126,10 +140,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
             const uint32_t cand = bit >= 0 ? (t | (1u << bit)) : 0u;
             if (bit < 0 && any) break;
             float above = 0.f;
-            for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-                const float z = row[i] * inv_t;
+#pragma unroll
+            for (int j = 0; j < nj; ++j) {
+                const float z = raw(j) * inv_t;
                 const uint32_t key = order_key(z);
-                if (key >= thr && key > cand) above += expf(z - zmax);
+                if ((int)threadIdx.x + j * SAMPLE_THREADS < vocab && key >= thr && key > cand) above += expf(z - zmax);
             }
             if (block_sum(above, fl) > limit) {
                 t = cand;
@@ -140,45 +155,80 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
     }
     // total mass of the survivors, then the first index whose running sum passes u * total
     float e = 0.f;
-    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-        const float z = row[i] * inv_t;
-        if (order_key(z) >= thr) e += expf(z - zmax);
+#pragma unroll
+    for (int j = 0; j < nj; ++j) {
+        const float z = raw(j) * inv_t;
+        if ((int)threadIdx.x + j * SAMPLE_THREADS < vocab && order_key(z) >= thr) e += expf(z - zmax);
     }
     const float target = uniform[r] * block_sum(e, fl);
     if (threadIdx.x == 0) found = 0x7fffffff;
     __syncthreads();
     const int lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
-    float running = 0.f;
+    constexpr int NWAVES = SAMPLE_THREADS / LLMS_WAVE;
     int last_kept = -1;
-    for (int base = 0; base < vocab; base += SAMPLE_THREADS) {
-        const int i = base + threadIdx.x;
-        float v = 0.f;
-        bool kept = false;
-        if (i < vocab) {
-            const float z = row[i] * inv_t;
-            kept = order_key(z) >= thr;
-            if (kept) v = expf(z - zmax);
-        }
-        float scan = v;  // inclusive scan inside the wave
+    // the thread's weight in tile j (the SAMPLE_THREADS consecutive tokens from j * SAMPLE_THREADS on), 0 if dropped
+    auto weight = [&](int j, bool& kept) -> float {
+        const float z = raw(j) * inv_t;
+        kept = j * SAMPLE_THREADS + (int)threadIdx.x < vocab && order_key(z) >= thr;
+        return kept ? expf(z - zmax) : 0.f;
+    };
+    auto wave_scan = [&](float v) -> float {  // inclusive, in lane order
 #pragma unroll
         for (int o = 1; o < LLMS_WAVE; o <<= 1) {
-            const float t = __shfl_up(scan, o, LLMS_WAVE);
-            if (lane >= o) scan += t;
+            const float t = __shfl_up(v, o, LLMS_WAVE);
+            if (lane >= o) v += t;
+        }
+        return v;
+    };
+    if (VPT > 0) {
+        // every wave's sum of every tile at once, then each thread walks the tiles' sums to the tile where the
+        // running sum passes the target, and only that tile is scanned: 3 barriers instead of 3 per tile
+        __shared__ float wave_total[VPT > 0 ? VPT : 1][NWAVES];
+#pragma unroll
+        for (int j = 0; j < nj; ++j) {
+            bool kept;
+            const float s = wave_scan(weight(j, kept));
+            if (kept) last_kept = j * SAMPLE_THREADS + threadIdx.x;
+            if (lane == LLMS_WAVE - 1) wave_total[j][wave] = s;
         }
         __syncthreads();
-        if (lane == LLMS_WAVE - 1) fl[wave] = scan;
-        __syncthreads();
-        float before = running;
-        for (int w = 0; w < wave; ++w) before += fl[w];
-        float tile_total = 0.f;
-        for (int w = 0; w < SAMPLE_THREADS / LLMS_WAVE; ++w) tile_total += fl[w];
-        if (kept) {
-            last_kept = i;
-            if (before + scan > target) atomicMin(&found, i);
+        float running = 0.f;
+#pragma unroll
+        for (int j = 0; j < nj; ++j) {
+            float before = running, end = running;  // sums up to this wave, up to the tile's end: the same additions
+            for (int w = 0; w < NWAVES; ++w) {
+                if (w == wave) before = end;
+                end += wave_total[j][w];
+            }
+            if (end > target) {  // (the same for every thread)
+                bool kept;
+                const float s = wave_scan(weight(j, kept));
+                if (kept && before + s > target) atomicMin(&found, j * SAMPLE_THREADS + (int)threadIdx.x);
+                break;
+            }
+            running = end;
         }
-        running += tile_total;
         __syncthreads();
-        if (found != 0x7fffffff) break;
+    } else {
+        float running = 0.f;
+        for (int j = 0; j < nj; ++j) {
+            bool kept;
+            const float scan = wave_scan(weight(j, kept));
+            __syncthreads();
+            if (lane == LLMS_WAVE - 1) fl[wave] = scan;
+            __syncthreads();
+            float before = running;
+            for (int w = 0; w < wave; ++w) before += fl[w];
+            float tile_total = 0.f;
+            for (int w = 0; w < NWAVES; ++w) tile_total += fl[w];
+            if (kept) {
+                last_kept = j * SAMPLE_THREADS + threadIdx.x;
+                if (before + scan > target) atomicMin(&found, j * SAMPLE_THREADS + (int)threadIdx.x);
+            }
+            running += tile_total;
+            __syncthreads();
+            if (found != 0x7fffffff) break;
+        }
     }
     if (found == 0x7fffffff) {
         // rounding left the running sum at or below the target: take the last surviving index
@@ -204,8 +254,10 @@ int llms_sample_rows(int* out, const float* logits, int ld, int n_rows, int voca
                      const int* top_k, const float* top_p, const float* uniform, hipStream_t stream) {
     LLMS_REQUIRE(n_rows > 0 && vocab > 0 && ld >= vocab, "sample_rows: bad sizes");
     LLMS_REQUIRE(temperature == nullptr || uniform != nullptr, "sample_rows: temperature needs uniform numbers");
-    sample_rows_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(out, logits, ld, vocab, temperature, top_k, top_p,
-                                                              uniform);
+    if (vocab <= 32 * SAMPLE_THREADS)  // (64 logits per thread would not fit the registers of 1,024 threads)
+        sample_rows_kernel<32><<<n_rows, SAMPLE_THREADS, 0, stream>>>(out, logits, ld, vocab, temperature, top_k, top_p, uniform);
+    else
+        sample_rows_kernel<0><<<n_rows, SAMPLE_THREADS, 0, stream>>>(out, logits, ld, vocab, temperature, top_k, top_p, uniform);
     LLMS_LAUNCH_CHECK();
 }
 

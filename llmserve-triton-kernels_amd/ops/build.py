@@ -34,7 +34,7 @@ HIPCC_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",
-    "-Wno-unused-result", "-Wno-unknown-warning-option",
+    "-Wno-unused-result", "-Wno-unknown-warning-option", "-Wno-pass-failed",
 ]
 
 # Which libraries the step function of a model of a given dtype needs (the sampler's library is
