@@ -72,6 +72,25 @@ def test_bfloat16_generation_follows_plain_logits(model_dirs):
         assert row.max() - row[tok] <= 2 * max_tol, f"token {i} = {tok} is not near the top of the plain logits"
 
 
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_bfloat16_generation_of_many_requests_at_once(model_dirs, name):
+    """48 requests decoding in one step: from 17 and from 33 rows on the products of a step take other kernels
+    (a slice of all rows in LDS, partial sums added up by the norm and by the rotation), replayed from a graph."""
+    from llmserve import SamplingParams
+
+    vocab = TINY[name][0]["vocab_size"]
+    prompts = [traces.random_ids(vocab, 3 + (5 * i) % 18, 500 + i) for i in range(48)]
+    llm = _llm(model_dirs[name], name, "bfloat16", num_blocks=48 * 8, max_num_seqs=48, max_num_batched_tokens=256)
+    results = llm.generate(prompts, SamplingParams(max_new_tokens=10))
+    assert llm.engine.stats.preemptions == 0
+    for prompt, result in zip(prompts, results):
+        ref = traces.plain_logits(model_dirs[name], prompt + result.tokens, torch.bfloat16)
+        max_tol, _ = traces.tolerance(torch.bfloat16, ref)
+        for i, tok in enumerate(result.tokens):
+            row = ref[len(prompt) - 1 + i]
+            assert row.max() - row[tok] <= 2 * max_tol, f"token {i} = {tok} is not near the top of the plain logits"
+
+
 def test_temperature_sampling_is_seeded_and_matches_plain_sampler(model_dirs):
     from llmserve import SamplingParams
     from llmserve.sampling import uniform
