@@ -663,7 +663,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                                                                           token_begin, n_heads, head_dim, num_splits);
         }
     } else {
-        const bool paired = window == 0 && head_dim <= 192;  // early and late blocks of tokens in one workgroup
+        bool paired = window == 0 && head_dim <= 192;  // early and late blocks of tokens in one workgroup
         // (8 waves of wider heads would not fit the registers)
         auto grid_for = [&](int cg) {
             const int per_block = PROMPT_WB * cg;  // column groups of a block of tokens
@@ -671,9 +671,14 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
             if (paired) grid.x = (grid.x + 1) / 2;
             return grid;
         };
+        auto workgroups = [](dim3 g) { return (long long)g.x * g.y * g.z; };
         int cg = PROMPT_CG_MAX(head_dim / 16);
         dim3 grid = grid_for(cg);
-        if (cg == 2 && (long long)grid.x * grid.y * grid.z < PROMPT_FULL_CHIP) grid = grid_for(cg = 1);
+        if (cg == 2 && workgroups(grid) < PROMPT_FULL_CHIP) grid = grid_for(cg = 1);
+        if (paired && workgroups(grid) < PROMPT_FULL_CHIP) {  // a short portion: workgroups for more CUs matter more
+            paired = false;                                    // than equal work for each
+            grid = grid_for(cg);
+        }
         if (int e = launch_prompt(head_dim / 16, cg, grid, paired, a, stream)) return e;
     }
     LLMS_LAUNCH_CHECK();

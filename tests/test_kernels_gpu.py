@@ -595,26 +595,27 @@ def test_attention_mfma(case, arrangement):
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
 
 
-# The prompt kernel gives a wave two column groups (32 columns) up to head_dim 128 once the launch has a workgroup
-# for each of the 256 CUs; the cases above are too small for that.
+# The prompt kernel gives a wave two column groups (32 columns) up to head_dim 128, and pairs early with late blocks of
+# tokens, once the launch has a workgroup for each of the 256 CUs; the cases above are too small for that.
 WIDE_LAUNCH_CASES = [  # nh, nkv, d, bs, lens, new, window
     (16, 16, 32, 8, [260, 200, 131, 97, 260, 33, 1, 17], [260, 200, 131, 97, 260, 33, 1, 17], 0),  # a second group without tokens
     (16, 4, 64, 16, [520, 300, 77, 515, 512, 511, 2, 64], [520, 300, 77, 100, 512, 31, 2, 64], 0),  # portions beside whole prompts
     (16, 16, 32, 8, [300, 290, 280, 31, 300, 47], [300, 290, 280, 31, 300, 16], 50),               # a window: no pairing
     (16, 16, 128, 16, [300, 129, 128, 127, 33, 290, 150, 257], [300, 129, 128, 127, 33, 290, 7, 257], 0),
     (24, 8, 80, 8, [330, 190, 1, 64, 200, 326, 65, 200], [330, 190, 1, 64, 200, 3, 65, 200], 0),
+    (16, 16, 160, 8, [300, 150, 17, 290, 300, 64, 300, 1], [300, 150, 17, 290, 300, 64, 300, 1], 0),  # one group, paired
 ]
 
 
 @pytest.mark.parametrize("case", WIDE_LAUNCH_CASES)
-def test_attention_mfma_two_column_groups_per_wave(case):
+def test_attention_mfma_launches_that_fill_the_chip(case):
     nh, nkv, d, bs, lens, new, window = case
     g = nh // nkv
     hg = min(g, 16)
     groups = -(-max(new) // (16 // hg))
-    blocks = -(-groups // 8)
+    blocks = -(-groups // (8 if d <= 128 else 4))
     workgroups = (blocks if window else -(-blocks // 2)) * nkv * -(-g // hg) * len(lens)
-    assert workgroups >= 256, "this case would run with one column group per wave"
+    assert workgroups >= 256, "this case would run with one column group per wave and without pairing"
     got, ref = run_attention_mfma(nh, nkv, d, bs, lens, new, window, seed=55)
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
 
