@@ -345,7 +345,8 @@ __global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const A
 // instead of 16: with head_dim 128 the LDS reads were what the loop waited for (twice the matrix instructions'
 // time), with head_dim 64 it was instruction issue, of which the reads and the loop's own work are a third.
 //
-// PAIRED (no window): the causal triangle gives the last tokens of a prompt the most keys, and a workgroup with
+// PAIRED (no window, and enough tokens that the paired launch still has a workgroup for every CU): the causal
+// triangle gives the last tokens of a prompt the most keys, and a workgroup with
 // few keys leaves its CU idle while others still run.  A workgroup then has 2 WB waves and takes two blocks of
 // tokens, number x from the front and number x from the back: the first WB waves the late block, the others the early
 // block, which sees a prefix of the same keys, stops multiplying when it has passed its own position, and
