@@ -226,21 +226,7 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const float* __restrict__
 // depends on the token and on i only; computed per element they cost more than the kernel's memory traffic); a
 // thread takes 8 consecutive pairs (i .. i+7 and their partners at + head_dim/2) of one head with 16-byte loads and
 // stores; values leave in 16-byte reads and single stores (transposed in the page).
-// PARTS: the projection arrives as n_parts arrays of 32-bit partial sums [tokens, row_width] (ops.gemm_slices); they
-// are added up in order, the bias (nullable) last, and rounded to bfloat16 as the projection's result is, and the
-// rotated queries go to q_out [tokens, q_stride] instead of back in place.
-struct RopeParts {
-    const float* parts;
-    int n_parts;
-    size_t part_stride;
-    const bf16* bias;
-    bf16* q_out;
-    int q_stride;
-};
-
-template <bool PARTS>
-__global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restrict__ qkv, const RopeParts src,
-                                                                  const float* __restrict__ inv_freq,
+__global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restrict__ qkv, const float* __restrict__ inv_freq,
                                                                   const int* __restrict__ positions,
                                                                   const int* __restrict__ slots, bf16* __restrict__ k_pool,
                                                                   bf16* __restrict__ v_pool, int n_tokens, int n_heads,
@@ -252,18 +238,7 @@ __global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restri
     if (n >= n_tokens) return;
     const int half = head_dim / 2, chunks = half / 8;
     const int row_width = (n_heads + 2 * n_kv_heads) * head_dim;
-    bf16* row = PARTS ? nullptr : qkv + (size_t)n * row_width;
-    // 8 consecutive elements of the token's projection, from column `col` on
-    auto load8 = [&](int col) -> uint4 {
-        if (!PARTS) return *reinterpret_cast<const uint4*>(row + col);
-        float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        sum_parts8(f, src.parts + (size_t)n * row_width + col, src.n_parts, src.part_stride);
-        if (src.bias) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) f[e] += bf16_bits_to_f32(src.bias[col + e].bits);
-        }
-        return make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7]));
-    };
+    bf16* row = qkv + (size_t)n * row_width;
     const int slot = slots ? slots[n] : -1;
     const int page = slot >= 0 ? slot / block_size : 0;
     const int off = slot >= 0 ? slot % block_size : 0;
@@ -287,9 +262,9 @@ __global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restri
         const int rot_heads = n_heads + n_kv_heads;
         for (int h = h0; h < rot_heads; h += h_step) {
             const bool is_key = h >= n_heads;
-            if (is_key && (PARTS || k_pool != nullptr) && slot < 0) continue;  // a key with nowhere to go
-            const int col = h * head_dim + 8 * c;
-            const uint4 av = load8(col), bv = load8(col + half);
+            if (is_key && k_pool != nullptr && slot < 0) continue;  // a key with nowhere to go
+            bf16* x = row + (size_t)h * head_dim + 8 * c;
+            const uint4 av = *reinterpret_cast<const uint4*>(x), bv = *reinterpret_cast<const uint4*>(x + half);
             const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
             uint32_t ra[4] = {aw[0], aw[1], aw[2], aw[3]}, rb[4] = {bw[0], bw[1], bw[2], bw[3]};
             if (inv_freq) {
@@ -307,19 +282,17 @@ __global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restri
                     rb[j] = pack_bf16x2(lo_b[0], lo_b[1]);
                 }
             }
-            bf16* dst;
-            if (is_key && (PARTS || k_pool != nullptr))
+            bf16* dst = x;
+            if (is_key && k_pool != nullptr)
                 dst = k_pool + (((size_t)page * n_kv_heads + (h - n_heads)) * block_size + off) * head_dim + 8 * c;
-            else
-                dst = PARTS ? src.q_out + (size_t)n * src.q_stride + col : row + col;
             *reinterpret_cast<uint4*>(dst) = make_uint4(ra[0], ra[1], ra[2], ra[3]);
             *reinterpret_cast<uint4*>(dst + half) = make_uint4(rb[0], rb[1], rb[2], rb[3]);
         }
     }
     if (slot >= 0) {
-        const int v_col = (n_heads + n_kv_heads) * head_dim;
+        const bf16* v = row + (size_t)(n_heads + n_kv_heads) * head_dim;
         for (int t = threadIdx.x; t < n_kv_heads * head_dim / 8; t += blockDim.x) {
-            const uint4 vv = load8(v_col + 8 * t);
+            const uint4 vv = *reinterpret_cast<const uint4*>(v + 8 * t);
             const uint32_t vw[4] = {vv.x, vv.y, vv.z, vv.w};
             const int kvh = (8 * t) / head_dim, d = (8 * t) % head_dim;
             bf16* dst = v_pool + (((size_t)page * n_kv_heads + kvh) * head_dim + d) * block_size + off;
@@ -439,37 +412,14 @@ int llms_rope_store(int dtype, void* qkv, const float* inv_freq, const int* posi
     if (dtype == 1 && head_dim % 16 == 0 && head_dim <= 4096 && ((uintptr_t)qkv % 16) == 0 &&
         (k_pool == nullptr || ((uintptr_t)k_pool % 16) == 0)) {
         const unsigned grid = (unsigned)((n_tokens + 127) / 128 * 128);
-        rope_store_bf16_vec_kernel<false><<<grid, 256, head_dim * sizeof(float), stream>>>(
-            (bf16*)qkv, RopeParts{}, inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool, n_tokens, n_heads,
-            n_kv_heads, head_dim, block_size);
+        rope_store_bf16_vec_kernel<<<grid, 256, head_dim * sizeof(float), stream>>>(
+            (bf16*)qkv, inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool, n_tokens, n_heads, n_kv_heads, head_dim,
+            block_size);
         LLMS_LAUNCH_CHECK();
     }
     DISPATCH_DTYPE(dtype, rope_store_kernel<T><<<n_tokens, 256, 0, stream>>>(
                               (T*)qkv, inv_freq, positions, slots, (T*)k_pool, (T*)v_pool, n_heads,
                               n_kv_heads, head_dim, block_size);)
-    LLMS_LAUNCH_CHECK();
-}
-
-// The same for a projection that arrives as `n_parts` arrays of 32-bit partial sums [n_tokens, (n_heads + 2 n_kv_heads)
-// * head_dim], part_stride elements apart (bfloat16 engine only): their sum (+ bias, nullable) is rounded to bfloat16,
-// rotated, the queries written to q_out [n_tokens, q_stride], keys and values stored at `slots` (nullable: dropped).
-int llms_rope_store_parts(void* q_out, int q_stride, const float* parts, int n_parts, size_t part_stride, const void* bias,
-                          const float* inv_freq, const int* positions, const int* slots, void* k_pool, void* v_pool,
-                          int n_tokens, int n_heads, int n_kv_heads, int head_dim, int block_size, hipStream_t stream) {
-    LLMS_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0, "rope_store_parts: sizes must be positive");
-    LLMS_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 4096, "rope_store_parts: head_dim must be a multiple of 16");
-    LLMS_REQUIRE(block_size > 0, "rope_store_parts: block_size must be positive");
-    LLMS_REQUIRE(parts && n_parts > 0 && q_out, "rope_store_parts: needs partial sums and an output");
-    LLMS_REQUIRE(part_stride % 4 == 0 && ((uintptr_t)parts % 16) == 0 && ((uintptr_t)q_out % 16) == 0 && q_stride % 8 == 0 &&
-                     q_stride >= n_heads * head_dim, "rope_store_parts: operands must keep 16-byte alignment");
-    LLMS_REQUIRE(slots == nullptr || (k_pool && v_pool && ((uintptr_t)k_pool % 16) == 0),
-                 "rope_store_parts: slots given without (aligned) pools");
-    LLMS_REQUIRE(positions != nullptr || inv_freq == nullptr, "rope_store_parts: rotation needs positions");
-    const RopeParts src = {parts, n_parts, part_stride, (const bf16*)bias, (bf16*)q_out, q_stride};
-    const unsigned grid = (unsigned)((n_tokens + 127) / 128 * 128);
-    rope_store_bf16_vec_kernel<true><<<grid, 256, head_dim * sizeof(float), stream>>>(
-        nullptr, src, inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool, n_tokens, n_heads, n_kv_heads, head_dim,
-        block_size);
     LLMS_LAUNCH_CHECK();
 }
 

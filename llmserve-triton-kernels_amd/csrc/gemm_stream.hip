@@ -1,15 +1,18 @@
 // bfloat16 matrix product for few rows (decoding):  C[M,N] = X[M,K] * W[N,K]^T, 32-bit sums on the gfx950
 // matrix cores, built around reading the weight once at memory speed.
 //
-// A workgroup owns 16 weight rows and 16 rows of X; its 4 waves take the K chunks (512 wide) in turn.
+// A workgroup owns 16 weight rows and 16 rows of X; its 4 waves take the K chunks (ST_KC = 128 wide) in turn.
 // (More than 16 rows of X, up to 64: one workgroup per block of 16 rows; the workgroups that share weight
 // rows get consecutive places on the same XCD, so the weights cross HBM once and come from that XCD's L2
-// for the others.)  One load instruction
-// of a wave covers 1 KB of one weight row (fully coalesced, non-temporal), 16 such loads are in flight per
-// wave before anything waits, and the next chunk's loads are issued before the arithmetic of this one.
-// The 16 KB go through a wave-private, XOR-swizzled LDS tile to reach the layout of
-// v_mfma_f32_16x16x32_bf16 (lane l: A[i = l%16][k = 8*(l/16) .. +7], here i = weight row; B likewise
+// for the others.)  One load instruction of a wave covers whole 256-byte pieces of 4 weight rows (coalesced,
+// non-temporal); the 4 loads of a chunk are in flight before anything waits, and the next chunk's loads are
+// issued before the arithmetic of this one.  The 4 KB go through a wave-private, XOR-swizzled LDS tile to reach
+// the layout of v_mfma_f32_16x16x32_bf16 (lane l: A[i = l%16][k = 8*(l/16) .. +7], here i = weight row; B likewise
 // with j = row m of X; D[i = 4*(l/16) + r][j = l%16]).  The waves' partial sums meet in LDS in a fixed order.
+// The chunk was 512 wide at first (1 KB per row and load, 64 KB of LDS, two workgroups per CU): a CU takes only
+// so many bytes a microsecond however much a wave has in flight, so what counts is that every CU has work at
+// every moment; with 16 KB of LDS eight workgroups fit, a launch of 704 or 2,000 tiles no longer runs in rounds,
+// and a step of the 7B shape at batch 8 went from 3.98 to 3.73 ms.
 //
 // Because a launch costs more than most of these products take, what surrounds the product is fused in:
 //   NORM      prologue: x = bf16(residual + delta) (written to resid_out by workgroup 0), then
@@ -46,7 +49,7 @@ __device__ __forceinline__ void store_out<float>(float* p, float v) { *p = v; }
 template <>
 __device__ __forceinline__ void store_out<bf16>(bf16* p, float v) { p->bits = f32_to_bf16_bits(v); }
 
-#define ST_KC 512
+#define ST_KC 128
 #define ST_WAVES 4
 #define EPI_PLAIN 0
 #define EPI_SWIGLU 1
@@ -97,7 +100,7 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
 
 template <typename TOut, int EPI, bool NORM>
 __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const StreamArgs a) {
-    __shared__ uint4 lds[ST_WAVES * 16 * (ST_KC / 8)];  // 64 KB: per wave 16 rows x 64 chunks of 16 bytes
+    __shared__ uint4 lds[ST_WAVES * 16 * (ST_KC / 8)];  // per wave 16 rows x ST_KC / 8 pieces of 16 bytes
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
     const int r16 = lane % 16, g = lane / 16;
     // Workgroups go round the 8 XCDs; tile t lives on XCD t % 8, its blocks of 16 rows of X next to each other
@@ -135,15 +138,20 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     uint4* tile = lds + wave * 16 * (ST_KC / 8);
     // this workgroup's chunks of K: all of them, or its share when K is split over workgroups
     const int all_chunks = (K + ST_KC - 1) / ST_KC;
-    const int per_split = (all_chunks + a.k_splits - 1) / a.k_splits;
+    const int shares = (K + 511) / 512;  // K is shared out in pieces of 512, whatever the chunk
+    const int per_split = (shares + a.k_splits - 1) / a.k_splits * (512 / ST_KC);
     const int split = blockIdx.y, c_begin = split * per_split;
     const int chunks = min(all_chunks, c_begin + per_split);
-    uint4 wreg[16];
+    constexpr int LPR = ST_KC / 8;        // lanes that cover a row's piece of a chunk (16 bytes each)
+    constexpr int RPL = LLMS_WAVE / LPR;  // rows per load instruction
+    constexpr int NLOAD = 16 / RPL;       // load instructions per chunk
+    constexpr int KSTEPS = ST_KC / 32;    // matrix instructions per chunk
+    uint4 wreg[NLOAD];
     auto load_weights = [&](int c) {
-        const int kl = c * ST_KC + 8 * lane;
+        const int kl = c * ST_KC + 8 * (lane % LPR);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int n = weight_row(i);
+        for (int i = 0; i < NLOAD; ++i) {
+            const int n = weight_row(i * RPL + lane / LPR);
             wreg[i] = (n >= 0 && kl < K) ? load_streaming(a.W + (size_t)n * K + kl) : zero;
         }
     };
@@ -231,9 +239,9 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
     for (int c = c_begin + wave; c < chunks; c += ST_WAVES) {
         const int k0 = c * ST_KC;
-        uint4 xreg[16];
+        uint4 xreg[KSTEPS];
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
+        for (int s = 0; s < KSTEPS; ++s) {
             const int k = k0 + 32 * s + 8 * g;
             if (m_ok && k < K)
                 xreg[s] = NORM ? h_lds[r16 * hstride + k / 8] : *reinterpret_cast<const uint4*>(xrow + k);
@@ -241,11 +249,14 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
                 xreg[s] = zero;
         }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) tile[i * (ST_KC / 8) + (lane ^ i)] = wreg[i];
+        for (int i = 0; i < NLOAD; ++i) {
+            const int row = i * RPL + lane / LPR;
+            tile[row * LPR + ((lane % LPR) ^ row)] = wreg[i];
+        }
         if (c + ST_WAVES < chunks) load_weights(c + ST_WAVES);  // the registers are free again
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
-            const uint4 av = tile[r16 * (ST_KC / 8) + ((4 * s + g) ^ r16)];
+        for (int s = 0; s < KSTEPS; ++s) {
+            const uint4 av = tile[r16 * LPR + ((4 * s + g) ^ r16)];
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av), as_bf16x8(xreg[s]), acc, 0, 0, 0);
         }
     }

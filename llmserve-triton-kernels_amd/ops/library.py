@@ -213,47 +213,6 @@ def rope_store(qkv: torch.Tensor, inv_freq: torch.Tensor | None, positions: torc
         "rope_store")
 
 
-def rope_store_parts(q_out: torch.Tensor, parts: torch.Tensor, bias: torch.Tensor | None, inv_freq: torch.Tensor | None,
-                     positions: torch.Tensor, slots: torch.Tensor | None, k_pool: torch.Tensor | None,
-                     v_pool: torch.Tensor | None, n_heads: int, n_kv_heads: int, head_dim: int, block_size: int) -> torch.Tensor:
-    """rope_store for a projection that arrives as float32 partial sums [S, N, (n_heads + 2 n_kv_heads) * head_dim]
-    (ops.gemm_slices): their sum in order (+ bias) is rounded to bfloat16, as the projection's result is, then
-    rotated; q_out [N, n_heads * head_dim] (bfloat16) gets the queries, the pools the keys and values at `slots`
-    (without slots they are dropped).  head_dim % 16 == 0."""
-    dev = _dev(q_out, parts, bias, inv_freq, positions, slots, k_pool, v_pool)
-    width = (n_heads + 2 * n_kv_heads) * head_dim
-    if parts.dim() != 3 or parts.dtype != torch.float32 or parts.shape[2] != width or not parts.is_contiguous():
-        raise ValueError(f"parts must be a contiguous float32 [S, N, {width}] tensor")
-    n = parts.shape[1]
-    if head_dim % 16:
-        raise ValueError("rope_store_parts needs head_dim % 16 == 0")
-    _rows(q_out, "q_out", n_heads * head_dim)
-    if q_out.dtype != torch.bfloat16 or q_out.shape[0] != n:
-        raise ValueError("q_out must be bfloat16 [N, n_heads * head_dim]")
-    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != width or not bias.is_contiguous()):
-        raise ValueError(f"bias must be a contiguous bfloat16 vector of {width} elements")
-    _i32(positions, "positions", n)
-    if inv_freq is not None:
-        _f32(inv_freq, "inv_freq", head_dim // 2)
-    if slots is not None:
-        _i32(slots, "slots", n)
-        if k_pool is None or v_pool is None:
-            raise ValueError("slots given without pools")
-        pages = k_pool.shape[0]
-        if (tuple(k_pool.shape) != (pages, n_kv_heads, block_size, head_dim) or not k_pool.is_contiguous()
-                or tuple(v_pool.shape) != (pages, n_kv_heads, head_dim, block_size) or not v_pool.is_contiguous()
-                or k_pool.dtype != torch.bfloat16 or v_pool.dtype != torch.bfloat16):
-            raise ValueError("pools do not have the cache layout [pages, kv, block, D] / [pages, kv, D, block] in bfloat16")
-    if n == 0:
-        return q_out
-    _check(load("elementwise").llms_rope_store_parts(
-        _ptr(q_out), c_int(q_out.stride(0)), _ptr(parts), c_int(parts.shape[0]), ctypes.c_size_t(parts.stride(0)),
-        _ptr(bias), _ptr(inv_freq), _ptr(positions), _ptr(slots), _ptr(k_pool if slots is not None else None),
-        _ptr(v_pool if slots is not None else None), c_int(n), c_int(n_heads), c_int(n_kv_heads), c_int(head_dim),
-        c_int(block_size), _stream(dev)), "rope_store_parts")
-    return q_out
-
-
 def scatter_i32(dst: torch.Tensor, index: torch.Tensor, value: torch.Tensor) -> None:
     """dst.flatten()[index[i]] = value[i] wherever index[i] >= 0.  The caller has checked the indices."""
     dev = _dev(dst, index, value)

@@ -16,7 +16,7 @@ import math
 import torch
 
 from ..ops import library as ops
-from .linear import few_rows, linear, linear_partial_sums, norm_fusable, slices_pay
+from .linear import few_rows, linear, linear_partial_sums, norm_fusable
 from .registry import POSITION_ENCODINGS, DeferredNorm, Mixer, as_tensor, register_mixer
 from .rmsnorm import RMSNorm
 from .spec import PagedCacheSpec, ParamInfo
@@ -90,16 +90,13 @@ class Attention(Mixer):
         return (linear_partial_sums(out, self.o_weight) if to_a_norm else None) or linear(out, self.o_weight)
 
     def _few_rows_unfit(self, rows) -> bool:
-        return (rows.dtype != torch.bfloat16 or self.head_dim % 16 != 0
-                or not (few_rows(rows.shape[0], self.qkv_weight) or slices_pay(rows.shape[0], self.qkv_weight, sum_is_free=False))
+        return (rows.dtype != torch.bfloat16 or not few_rows(rows.shape[0], self.qkv_weight) or self.head_dim % 16 != 0
                 or not ops.gemm_bf16_supported(rows, self.qkv_weight))
 
     def project_few_rows(self, x, batch, cache, slots):
         """With few bfloat16 rows one kernel does the projection, the rotation and the cache store (and,
-        if switched on, the residual sum and the norm before them): ops.gemm_stream.  From 17 rows on, against
-        a weight small enough, the projection is left as partial sums per slice of K (ops.gemm_slices) and a
-        second kernel adds them up, rotates and stores.  Returns the rotated queries, or None when neither
-        applies."""
+        if switched on, the residual sum and the norm before them): ops.gemm_stream.  Returns the rotated
+        queries, or None when that kernel does not apply."""
         deferred = isinstance(x, DeferredNorm)
         rows = x.residual if deferred else x
         m = rows.shape[0]
@@ -110,15 +107,6 @@ class Attention(Mixer):
             return None  # a position encoding this kernel does not know
         if deferred and not (norm_fusable(*rows.shape) and isinstance(x.norm, RMSNorm)):
             x, rows, deferred = None, x.materialize(), False  # the norm by its own kernel, the rest fused
-        if slices_pay(m, self.qkv_weight, sum_is_free=False):  # partial sums per slice of K, then sum + rotation + store
-            rows = x.materialize() if deferred else rows
-            parts = torch.empty((-(-rows.shape[1] // ops.SLICE_K), m, self.qkv_weight.shape[0]), dtype=torch.float32,
-                                device=rows.device)
-            ops.gemm_slices(parts, rows, self.qkv_weight)
-            q = torch.empty((m, self.num_heads * self.head_dim), dtype=rows.dtype, device=rows.device)
-            return ops.rope_store_parts(q, parts, self.qkv_bias, frequencies() if frequencies is not None else None,
-                                        batch.positions, slots, cache.k_pool, cache.v_pool, self.num_heads,
-                                        self.num_kv_heads, self.head_dim, cache.block_size)
         rope = dict(n_heads=self.num_heads, n_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                     inv_freq=frequencies() if frequencies is not None else None, positions=batch.positions,
                     slots=slots, k_pool=cache.k_pool, v_pool=cache.v_pool, block_size=cache.block_size)

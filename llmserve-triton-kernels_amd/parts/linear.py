@@ -60,7 +60,7 @@ def norm_fusable(m: int, k: int) -> bool:
 # several workgroups per tile fills the chip: measured 4.3 -> 3.2 microseconds of reading for 2048 x 2048 and
 # 10.0 -> 6.8 for 2048 x 5632.  The partial sums are added up by the norm kernel that follows.
 SPLIT_K = os.environ.get("LLMSERVE_SPLIT_K", "1") != "0"
-SPLIT_K_WORKGROUPS = 512  # aim for about this many workgroups
+SPLIT_K_WORKGROUPS = 1024  # aim for about this many workgroups (a CU holds eight of them)
 SPLIT_K_MAX = 4
 
 
@@ -78,16 +78,10 @@ def k_splits_for(m: int, weight: torch.Tensor) -> int:
 SLICES_MAX_WEIGHT_BYTES = 24e6
 
 
-# Where the sums need a kernel of their own (the projection to q, k, v: sum, rotation, store), from this many rows on;
-# below, the streaming kernel with its epilogue is faster (32 rows: 8.6 against 5.0 + 5 microseconds).
-SLICES_MIN_ROWS_OWN_SUM = 33
-
-
-def slices_pay(m: int, weight: torch.Tensor, sum_is_free: bool = True) -> bool:
-    """Whether `m` bfloat16 rows against `weight` are best left as partial sums per slice of K (ops.gemm_slices).
-    `sum_is_free`: a kernel that runs anyway (the norm) adds them up."""
-    least = STREAM_ROWS + 1 if sum_is_free else SLICES_MIN_ROWS_OWN_SUM
-    return SPLIT_K and least <= m <= STREAM_MAX_ROWS and weight.numel() * 2 <= SLICES_MAX_WEIGHT_BYTES
+def slices_pay(m: int, weight: torch.Tensor) -> bool:
+    """Whether `m` bfloat16 rows against `weight` are best left as partial sums per slice of K (ops.gemm_slices),
+    for a norm to add up."""
+    return SPLIT_K and STREAM_ROWS < m <= STREAM_MAX_ROWS and weight.numel() * 2 <= SLICES_MAX_WEIGHT_BYTES
 
 
 def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor):

@@ -148,47 +148,6 @@ def test_rope_store(dtype, nh, nkv, d, bs, theta):
     assert torch.equal(k_pool.cpu()[page, :, off], k.transpose(0, 1)[0])
 
 
-@pytest.mark.parametrize("nh,nkv,d,bs,theta,parts,n,bias", [(4, 2, 16, 16, 1e4, 1, 7, False), (3, 1, 32, 8, 5e5, 4, 40, True),
-                                                            (32, 4, 64, 16, 1e4, 4, 64, False), (5, 5, 48, 8, 1e6, 3, 17, True),
-                                                            (16, 2, 128, 32, 1e4, 11, 33, False)])
-def test_rope_store_from_partial_sums(nh, nkv, d, bs, theta, parts, n, bias):
-    """The projection as 32-bit partial sums: the same bits, in the queries and in the pools, as rounding their sum
-    (+ bias) to bfloat16 and handing it to rope_store; tokens without a slot store nothing."""
-    width = (nh + 2 * nkv) * d
-    p = torch.stack([rnd(n, width, seed=40 + i) for i in range(parts)]).to(DEV)
-    b = rnd(width, seed=39).bfloat16().to(DEV) if bias else None
-    total = p[0].clone()
-    for i in range(1, parts):
-        total += p[i]
-    if bias:
-        total += b.float()
-    qkv = total.bfloat16()
-    positions = torch.randint(0, 4000, (n,), generator=torch.Generator().manual_seed(n), dtype=torch.int32).to(DEV)
-    pages = -(-n // bs) + 2
-    slots = torch.randperm(pages * bs, generator=torch.Generator().manual_seed(d))[:n].to(torch.int32)
-    slots[n // 2] = -1
-    slots = slots.to(DEV)
-    inv_freq = (1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
-    pools = [(torch.full((pages, nkv, bs, d), 7.0, dtype=torch.bfloat16, device=DEV),
-              torch.full((pages, nkv, d, bs), 7.0, dtype=torch.bfloat16, device=DEV)) for _ in range(2)]
-    ops().rope_store(qkv, inv_freq, positions, slots, *pools[0], nh, nkv, d, bs)
-    q = ops().rope_store_parts(torch.empty(n, nh * d, dtype=torch.bfloat16, device=DEV), p, b, inv_freq, positions, slots,
-                               *pools[1], nh, nkv, d, bs)
-    assert torch.equal(q, qkv[:, : nh * d])
-    assert torch.equal(pools[0][0], pools[1][0]) and torch.equal(pools[0][1], pools[1][1])
-    # no slots: queries only
-    q2 = ops().rope_store_parts(torch.empty(n, nh * d, dtype=torch.bfloat16, device=DEV), p, b, inv_freq, positions, None,
-                                None, None, nh, nkv, d, bs)
-    assert torch.equal(q2, q)
-    # no frequencies: nothing is rotated
-    q3 = ops().rope_store_parts(torch.empty(n, nh * d, dtype=torch.bfloat16, device=DEV), p, b, None, positions, None,
-                                None, None, nh, nkv, d, bs)
-    assert torch.equal(q3, total.bfloat16()[:, : nh * d])
-    with pytest.raises(ValueError, match="head_dim"):
-        ops().rope_store_parts(torch.empty(n, nh * 24, dtype=torch.bfloat16, device=DEV),
-                               torch.zeros(1, n, (nh + 2 * nkv) * 24, device=DEV), None, None, positions, None, None, None,
-                               nh, nkv, 24, bs)
-
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("inter", [176, 5632, 33])
