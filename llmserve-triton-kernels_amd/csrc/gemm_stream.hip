@@ -1,18 +1,18 @@
 // bfloat16 matrix product for few rows (decoding):  C[M,N] = X[M,K] * W[N,K]^T, 32-bit sums on the gfx950
 // matrix cores, built around reading the weight once at memory speed.
 //
-// A workgroup owns 16 weight rows and 16 rows of X; its 4 waves take the K chunks (ST_KC = 128 wide) in turn.
+// A workgroup owns 16 weight rows and 16 rows of X; its 4 waves take the K chunks (ST_KC = 128 or 512 wide) in turn.
 // (More than 16 rows of X, up to 64: one workgroup per block of 16 rows; the workgroups that share weight
 // rows get consecutive places on the same XCD, so the weights cross HBM once and come from that XCD's L2
 // for the others.)  One load instruction of a wave covers whole 256-byte pieces of 4 weight rows (coalesced,
-// non-temporal); the 4 loads of a chunk are in flight before anything waits, and the next chunk's loads are
-// issued before the arithmetic of this one.  The 4 KB go through a wave-private, XOR-swizzled LDS tile to reach
+// non-temporal; with chunks of 512 it is 1 KB of one row); the loads of a chunk are in flight before anything waits,
+// and the next chunk's loads are issued before the arithmetic of this one.  The chunk goes through a wave-private, XOR-swizzled LDS tile to reach
 // the layout of v_mfma_f32_16x16x32_bf16 (lane l: A[i = l%16][k = 8*(l/16) .. +7], here i = weight row; B likewise
 // with j = row m of X; D[i = 4*(l/16) + r][j = l%16]).  The waves' partial sums meet in LDS in a fixed order.
-// The chunk was 512 wide at first (1 KB per row and load, 64 KB of LDS, two workgroups per CU): a CU takes only
-// so many bytes a microsecond however much a wave has in flight, so what counts is that every CU has work at
-// every moment; with 16 KB of LDS eight workgroups fit, a launch of 704 or 2,000 tiles no longer runs in rounds,
-// and a step of the 7B shape at batch 8 went from 3.98 to 3.73 ms.
+// With chunks of 512 (64 KB of LDS) two workgroups fit a CU; a CU takes only so many bytes a microsecond however
+// much a wave has in flight, so what counts is that every CU has work at every moment: with chunks of 128 (16 KB)
+// eight workgroups fit, a launch of 704 or 2,000 tiles no longer runs in rounds, and a step of the 7B shape at
+// batch 8 went from 3.98 to 3.73 ms.  A launch of at most a workgroup per CU keeps the chunks of 512.
 //
 // Because a launch costs more than most of these products take, what surrounds the product is fused in:
 //   NORM      prologue: x = bf16(residual + delta) (written to resid_out by workgroup 0), then
@@ -49,7 +49,6 @@ __device__ __forceinline__ void store_out<float>(float* p, float v) { *p = v; }
 template <>
 __device__ __forceinline__ void store_out<bf16>(bf16* p, float v) { p->bits = f32_to_bf16_bits(v); }
 
-#define ST_KC 128
 #define ST_WAVES 4
 #define EPI_PLAIN 0
 #define EPI_SWIGLU 1
@@ -98,7 +97,7 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-template <typename TOut, int EPI, bool NORM>
+template <typename TOut, int EPI, bool NORM, int ST_KC>  // ST_KC: width of a chunk of K, 128 or 512
 __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const StreamArgs a) {
     __shared__ uint4 lds[ST_WAVES * 16 * (ST_KC / 8)];  // per wave 16 rows x ST_KC / 8 pieces of 16 bytes
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
@@ -410,22 +409,32 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_slices_kernel(const 
 
 #define ST_NORM_LDS_MAX (96 * 1024)  // beside the 64 KB of weight tiles, of the 160 KB a workgroup may hold
 
-template <typename TOut, int EPI>
-static int launch_stream(bool norm, unsigned tiles, const StreamArgs& a, hipStream_t stream) {
-    const dim3 grid(tiles, a.k_splits);
+// A launch with a workgroup or less per CU gets chunks of 512 (16 KB in flight per wave: all a lone workgroup can
+// do for its CU), a larger one chunks of 128 (eight workgroups per CU, no rounds).
+#define ST_FEW_WORKGROUPS 256
+
+template <typename TOut, int EPI, int KC>
+static int launch_stream_kc(bool norm, dim3 grid, const StreamArgs& a, hipStream_t stream) {
     if (norm) {
         static bool raised = false;  // (per instantiation) allow more dynamic LDS than the default limit
         if (!raised) {
-            LLMS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<TOut, EPI, true>),
+            LLMS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<TOut, EPI, true, KC>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, ST_NORM_LDS_MAX));
             raised = true;
         }
         const size_t h_bytes = (size_t)a.M * (a.K / 8 + 1) * 16;
-        gemm_stream_kernel<TOut, EPI, true><<<grid, ST_WAVES * LLMS_WAVE, h_bytes, stream>>>(a);
+        gemm_stream_kernel<TOut, EPI, true, KC><<<grid, ST_WAVES * LLMS_WAVE, h_bytes, stream>>>(a);
     } else {
-        gemm_stream_kernel<TOut, EPI, false><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(a);
+        gemm_stream_kernel<TOut, EPI, false, KC><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(a);
     }
     return LLMS_OK;
+}
+
+template <typename TOut, int EPI>
+static int launch_stream(bool norm, unsigned tiles, const StreamArgs& a, hipStream_t stream) {
+    const dim3 grid(tiles, a.k_splits);
+    if ((long long)tiles * a.k_splits <= ST_FEW_WORKGROUPS) return launch_stream_kc<TOut, EPI, 512>(norm, grid, a, stream);
+    return launch_stream_kc<TOut, EPI, 128>(norm, grid, a, stream);
 }
 
 extern "C" {
