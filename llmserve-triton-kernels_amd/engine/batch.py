@@ -284,10 +284,6 @@ class StaticStepBatch:
         for j, g in enumerate(self.group_ids):
             ops.scatter_i32(self.storage.tables[g], self._view(8 + 3 * j), self._view(9 + 3 * j))
 
-    def fits(self, n_decode: int, n_prefill: int, n_prefill_tokens: int, n_logits: int) -> bool:
-        return (n_decode <= self.decode and n_prefill <= self.prefill and n_prefill_tokens <= self.tokens
-                and n_logits <= self.logits)
-
     def fill(self, layout: StepLayout, tokens: list[list[int]], logit_rows: list[int]) -> None:
         """Write a step into the buffers: `layout` lists the requests that bring one token first."""
         import numpy as np

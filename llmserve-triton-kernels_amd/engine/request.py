@@ -32,10 +32,6 @@ class Request:
     num_preemptions: int = 0
 
     @property
-    def all_ids(self) -> list[int]:
-        return self.prompt_ids + self.generated
-
-    @property
     def num_tokens(self) -> int:
         return len(self.prompt_ids) + len(self.generated)
 
