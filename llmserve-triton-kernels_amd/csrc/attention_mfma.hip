@@ -18,7 +18,8 @@
 //     and optionally to `num_splits` workgroups whose partial results a second kernel merges.
 //   attn_prompt_kernel (prompts): consecutive column groups of one request want the same keys and share
 //     each tile through LDS, one or two groups per wave; without a window, a block of late tokens and a block of
-//     early ones are paired.
+//     early ones are paired, or (a short portion behind a long prefix) the keys of a block are shared out to
+//     `num_splits` workgroups.
 // All merges run in a fixed order, so a token's result does not depend on the batch around it.
 //
 // Needs block_size % 8 == 0, head_dim % 16 == 0 and <= 256, 16-byte aligned rows.
@@ -384,9 +385,12 @@ __global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt
         my_first = (wave < WB ? late : early) * BLK;
         wave_on = wave < WB || early != late;  // (the middle block of an odd number is its own partner)
     } else {
-        wg_first = my_first = blockIdx.x * BLK;
+        wg_first = my_first = ((int)blockIdx.x / a.num_splits) * BLK;
         if (wg_first >= n_new || ctx <= 0) return;
     }
+    // Without pairing the keys of a block may be shared out to num_splits workgroups (blockIdx.x % num_splits), whose
+    // partial results attn_merge adds up: a short portion with a long prefix has few blocks and many keys.
+    const int n_splits = PAIRED ? 1 : a.num_splits, split = PAIRED ? 0 : (int)blockIdx.x % a.num_splits;
     // The tiles are brought in by the waves that have time for it: those of the early block, which stop
     // multiplying half way on average (without pairing, by everyone).
     const bool loader = !PAIRED || tid >= LT;
@@ -496,15 +500,17 @@ __global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt
         }
     };
 
-    if (loader) {
-        load_pages(block_of(j_begin));
-        load_tile(j_begin);
-        store_tile(0, j_begin);
-        if (n_tiles > 1) load_tile(j_begin + 32);
+    const int per_split = (n_tiles + n_splits - 1) / n_splits;
+    const int t_lo = split * per_split, t_hi = min(n_tiles, t_lo + per_split);  // this workgroup's tiles (maybe none)
+    if (loader && t_lo < t_hi) {
+        load_pages(block_of(j_begin + 32 * t_lo));
+        load_tile(j_begin + 32 * t_lo);
+        store_tile(0, j_begin + 32 * t_lo);
+        if (t_lo + 1 < t_hi) load_tile(j_begin + 32 * (t_lo + 1));
     }
     __syncthreads();
-    for (int t = 0; t < n_tiles; ++t) {
-        const int buf = t & 1, j0 = j_begin + 32 * t;
+    for (int t = t_lo; t < t_hi; ++t) {
+        const int buf = (t - t_lo) & 1, j0 = j_begin + 32 * t;
         if (wave_on && j0 <= w_pmax) {  // (a tile beyond the wave's last position adds nothing)
         uint4 kf[2][KS], vf[DB];
 #pragma unroll
@@ -525,15 +531,27 @@ __global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt
                 attend_tile<DB, KS, true>(acc[cg], m_run[cg], l_run[cg], kf, vf, qf[cg], j0 + 8 * g, lo_col[cg], p_col[cg], scale_log2);
         }
         }
-        if (loader && t + 1 < n_tiles) {
+        if (loader && t + 1 < t_hi) {
             store_tile(buf ^ 1, j0 + 32);  // last read two tiles ago, before the previous barrier
-            if (t + 2 < n_tiles) load_tile(j_begin + 32 * (t + 2));
+            if (t + 2 < t_hi) load_tile(j_begin + 32 * (t + 2));
         }
         __syncthreads();
     }
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg) {
         if (!col_ok[cg]) continue;
+        if (n_splits > 1) {  // the share of this workgroup, as the decode kernel leaves its own
+            const size_t item = ((size_t)(tok0 + c_tok[cg]) * a.n_heads + head) * n_splits + split;
+#pragma unroll
+            for (int m = 0; m < DB; ++m)
+                *reinterpret_cast<float4*>(a.ws_o + item * D + 16 * m + 4 * g) =
+                    make_float4(acc[cg][m][0], acc[cg][m][1], acc[cg][m][2], acc[cg][m][3]);
+            if (g == 0) {
+                a.ws_ml[item * 2] = m_run[cg];
+                a.ws_ml[item * 2 + 1] = l_run[cg];
+            }
+            continue;
+        }
         const float inv = 1.f / l_run[cg];
         bf16* orow = a.out + (size_t)(tok0 + c_tok[cg]) * a.out_stride + (size_t)head * D;
 #pragma unroll
@@ -546,27 +564,39 @@ __global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt
     }
 }
 
-// Merge of the splits of one (token, head), split 0 first.
-__global__ void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ ws_o,
-                                  const float* __restrict__ ws_ml, int token_begin, int n_heads, int head_dim,
-                                  int num_splits) {
-    const int token = token_begin + blockIdx.x, head = blockIdx.y;
-    const size_t item0 = ((size_t)token * n_heads + head) * num_splits;
-    float m_tot = -INFINITY;
-    for (int s = 0; s < num_splits; ++s) m_tot = fmaxf(m_tot, ws_ml[(item0 + s) * 2]);
-    float l_tot = 0.f;
-    for (int s = 0; s < num_splits; ++s) {
-        const float m = ws_ml[(item0 + s) * 2];
-        if (m != -INFINITY) l_tot += ws_ml[(item0 + s) * 2 + 1] * exp2_fast(m - m_tot);
-    }
-    const float inv = 1.f / l_tot;
-    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-        float o = 0.f;
+// Merge of the splits of every (token, head), split 0 first: a workgroup per token, a thread per head and 4 dimensions.
+__global__ __launch_bounds__(256) void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ ws_o,
+                                                         const float* __restrict__ ws_ml, int token_begin, int n_heads,
+                                                         int head_dim, int num_splits) {
+    const int token = token_begin + blockIdx.x;
+    const int q4 = head_dim / 4;
+    for (int idx = threadIdx.x; idx < n_heads * q4; idx += blockDim.x) {
+        const int head = idx / q4, d = 4 * (idx % q4);
+        const size_t item0 = ((size_t)token * n_heads + head) * num_splits;
+        const float2* ml = reinterpret_cast<const float2*>(ws_ml) + item0;  // (maximum, sum) of each split
+        float m_tot = -INFINITY;
+#pragma unroll 4
+        for (int s = 0; s < num_splits; ++s) m_tot = fmaxf(m_tot, ml[s].x);
+        float l_tot = 0.f;
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
         for (int s = 0; s < num_splits; ++s) {
-            const float m = ws_ml[(item0 + s) * 2];
-            if (m != -INFINITY) o += ws_o[(item0 + s) * head_dim + d] * exp2_fast(m - m_tot);
+            const float2 v = ml[s];
+            const float4 p = *reinterpret_cast<const float4*>(ws_o + (item0 + s) * head_dim + d);
+            if (v.x != -INFINITY) {  // (a split that saw no key of this column)
+                const float w = exp2_fast(v.x - m_tot);
+                l_tot += v.y * w;
+                o.x += p.x * w;
+                o.y += p.y * w;
+                o.z += p.z * w;
+                o.w += p.w * w;
+            }
         }
-        out[(size_t)token * out_stride + (size_t)head * head_dim + d].bits = f32_to_bf16_bits(o * inv);
+        const float inv = 1.f / l_tot;
+        uint2 pk;
+        pk.x = pack_bf16(o.x * inv, o.y * inv);
+        pk.y = pack_bf16(o.z * inv, o.w * inv);
+        *reinterpret_cast<uint2*>(out + (size_t)token * out_stride + (size_t)head * head_dim + d) = pk;
     }
 }
 
@@ -619,7 +649,8 @@ extern "C" {
 // Attention for the requests [seq_begin, seq_begin + n_seqs) of a step.  max_new: most new tokens any of
 // them brings.  split_waves = 0: prompt portions (attn_prompt_kernel);
 // split_waves = 1 deals the keys of each column group to `waves` (4 or 8) waves and
-// `num_splits` workgroups (decoding); with num_splits > 1 the caller provides ws_o [tokens * heads * splits * D] and
+// `num_splits` workgroups (decoding); split_waves = 0 with num_splits > 1 shares the keys of each block of prompt
+// tokens out to that many workgroups (no window then); with num_splits > 1 the caller provides ws_o [tokens * heads * splits * D] and
 // ws_ml [tokens * heads * splits * 2] floats, indexed by absolute token row.
 int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
                         const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
@@ -642,8 +673,9 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     LLMS_REQUIRE(split_waves == 0 || split_waves == 1, "attention_mfma: split_waves is 0 or 1");
     LLMS_REQUIRE(waves == 4 || (split_waves > 0 && waves == 8), "attention_mfma: 4 waves, or 8 when the waves share the keys");
     LLMS_REQUIRE(waves == 4 || head_dim <= 160, "attention_mfma: 8 waves take head_dim up to 160");
-    LLMS_REQUIRE(split_waves > 0 || num_splits == 1, "attention_mfma: splits need split_waves");
-    LLMS_REQUIRE(num_splits == 1 || (ws_o && ws_ml), "attention_mfma: splits need a workspace");
+    LLMS_REQUIRE(split_waves > 0 || num_splits == 1 || window == 0, "attention_mfma: portions with a window are not split");
+    LLMS_REQUIRE(num_splits == 1 || (ws_o && ws_ml && ((uintptr_t)ws_o % 16) == 0 && ((uintptr_t)ws_ml % 8) == 0),
+                 "attention_mfma: splits need a (16-byte aligned) workspace");
     LLMS_REQUIRE(n_seqs <= 65535, "attention_mfma: too many requests for one launch");
     const int G = n_heads / n_kv_heads, HG = G < 16 ? G : 16, TPG = 16 / HG, HB = (G + HG - 1) / HG;
     const int groups = (max_new + TPG - 1) / TPG;
@@ -660,15 +692,15 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                 fprintf(stderr, "llmserve kernel launch failed: %s\n", hipGetErrorString(e1));
                 return LLMS_ERR_LAUNCH;
             }
-            attn_merge_kernel<<<dim3(n_tokens, n_heads), 64, 0, stream>>>((bf16*)out, out_stride, ws_o, ws_ml,
-                                                                          token_begin, n_heads, head_dim, num_splits);
+            attn_merge_kernel<<<n_tokens, 256, 0, stream>>>((bf16*)out, out_stride, ws_o, ws_ml, token_begin, n_heads,
+                                                            head_dim, num_splits);
         }
     } else {
-        bool paired = window == 0 && head_dim <= 192;  // early and late blocks of tokens in one workgroup
+        bool paired = window == 0 && head_dim <= 192 && num_splits == 1;  // early and late blocks of tokens in one workgroup
         // (8 waves of wider heads would not fit the registers)
         auto grid_for = [&](int cg) {
             const int per_block = PROMPT_WB * cg;  // column groups of a block of tokens
-            dim3 grid((groups + per_block - 1) / per_block, n_kv_heads * HB, n_seqs);
+            dim3 grid((groups + per_block - 1) / per_block * num_splits, n_kv_heads * HB, n_seqs);
             if (paired) grid.x = (grid.x + 1) / 2;
             return grid;
         };
@@ -681,6 +713,15 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
             grid = grid_for(cg);
         }
         if (int e = launch_prompt(head_dim / 16, cg, grid, paired, a, stream)) return e;
+        if (num_splits > 1) {
+            hipError_t e1 = hipGetLastError();
+            if (e1 != hipSuccess) {
+                fprintf(stderr, "llmserve kernel launch failed: %s\n", hipGetErrorString(e1));
+                return LLMS_ERR_LAUNCH;
+            }
+            attn_merge_kernel<<<n_tokens, 256, 0, stream>>>((bf16*)out, out_stride, ws_o, ws_ml, token_begin, n_heads,
+                                                            head_dim, num_splits);
+        }
     }
     LLMS_LAUNCH_CHECK();
 }

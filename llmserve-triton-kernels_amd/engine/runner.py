@@ -228,7 +228,7 @@ class ModelRunner:
             return p
         step = 64 if n_prefill_tokens <= 512 else 256
         return (pow2(n_decode) if n_decode else 0, pow2(n_prefill), -(-n_prefill_tokens // step) * step,
-                pow2(max(n_logits, 1)), pow2(context, 256) if n_decode else 256)  # (the reach matters to decoding only)
+                pow2(max(n_logits, 1)), pow2(context, 256))  # (the reach sets how attention spreads its work)
 
     def _shape_of(self, layout, n_logits: int) -> tuple:
         n_dec = 0

@@ -500,7 +500,8 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
     step, whose new tokens are rows [token_begin, token_begin + n_tokens) of q and out and bring at most
     `max_new` tokens each.  `split_waves` (with `waves` = 4 or 8 and `num_splits`) spreads each request's keys
     over the waves of a workgroup and over workgroups: the arrangement for single decoded tokens.  Without
-    it the 4 waves of a workgroup take neighbouring tokens and share each tile of keys through LDS."""
+    it the 4 waves of a workgroup take neighbouring tokens and share each tile of keys through LDS; `num_splits`
+    then shares the keys of such a block of tokens out to several workgroups (short portions, long prefixes)."""
     dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, table_rows)
     _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
     if not attention_mfma_supported(q.dtype, head_dim, block_size):
@@ -519,8 +520,8 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
         raise ValueError("token range is outside the batch")
     if q.stride(0) % 8 or q.data_ptr() % 16 or out.data_ptr() % 16:
         raise ValueError("q rows must be 16-byte aligned")
-    if num_splits > 1 and not split_waves:
-        raise ValueError("num_splits > 1 needs split_waves")
+    if num_splits > 1 and not split_waves and window:
+        raise ValueError("portions of prompts with a window are not split over workgroups")
     if waves != 4 and not (split_waves and waves == 8):
         raise ValueError("4 waves, or 8 when the waves share the keys")
     if waves == 8 and head_dim > 160:

@@ -135,9 +135,24 @@ class Attention(Mixer):
             ops.attention_mfma(*common, 0, n_dec, 1, 0, n_dec, nh, nkv, d, bs, window, self.scale,
                                split_waves=True, num_splits=splits, waves=waves, table_rows=batch.state_slots)
         if n_dec < batch.num_seqs:  # portions of prompts: one wave per group of tokens and heads
+            splits = self.prompt_splits(batch.num_seqs - n_dec, batch.max_count, batch.max_context)
             ops.attention_mfma(*common, n_dec, batch.num_seqs - n_dec, batch.max_count, n_dec,
-                               batch.num_tokens - n_dec, nh, nkv, d, bs, window, self.scale,
+                               batch.num_tokens - n_dec, nh, nkv, d, bs, window, self.scale, num_splits=splits,
                                table_rows=batch.state_slots)
+
+    def prompt_splits(self, n_requests: int, max_new: int, max_context: int) -> int:
+        """Workgroups that share the keys of one block of prompt tokens.  A long prompt has blocks enough to
+        fill the chip by itself; a short portion behind a long prefix has few blocks and many keys, and four
+        waves per CU wait for memory most of the time, so its keys are shared out until every CU has about four
+        workgroups, 8 tiles of keys each at least (a second kernel merges the shares)."""
+        if self.window:
+            return 1
+        g = self.num_heads // self.num_kv_heads
+        hg = min(g, 16)
+        blocks = -(-max_new // (4 * (16 // hg)))  # of 4 waves with one column group each
+        workgroups = blocks * self.num_kv_heads * -(-g // hg) * n_requests
+        tiles = -(-max_context // 32)
+        return max(1, min(1024 // max(workgroups, 1), tiles // 8, 8))
 
     def decode_arrangement(self, n_requests: int, max_context: int) -> tuple[int, int]:
         """(workgroups per request and KV head, waves per workgroup) for decoding.  The waves of a

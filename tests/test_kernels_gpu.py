@@ -538,12 +538,18 @@ MFMA_CASES = [  # nh, nkv, d, bs, lens, new, window
 
 
 # split_waves: False = the prompt kernel (tiles shared through LDS, early and late blocks paired when there is
-# no window), True = the waves (4 or 8) share the keys, optionally split over workgroups
-@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 4), (True, 2, 4), (True, 5, 4), (True, 1, 8), (True, 3, 8)])
+# no window and the launch is large; with splits, the keys of a block shared out to workgroups), True = the waves
+# (4 or 8) share the keys, optionally split over workgroups
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (False, 2, 4), (False, 5, 4), (True, 1, 4), (True, 2, 4), (True, 5, 4),
+                                         (True, 1, 8), (True, 3, 8)])
 @pytest.mark.parametrize("case", MFMA_CASES)
 def test_attention_mfma(case, arrangement):
     nh, nkv, d, bs, lens, new, window = case
     split_waves, num_splits, waves = arrangement
+    if window and not split_waves and num_splits > 1:
+        with pytest.raises(ValueError, match="window"):
+            run_attention_mfma(nh, nkv, d, bs, lens, new, window, seed=50, num_splits=num_splits)
+        return
     if waves == 8 and d > 160:
         with pytest.raises(ValueError, match="8 waves"):
             run_attention_mfma(nh, nkv, d, bs, lens, new, window, seed=50, split_waves=split_waves,
@@ -579,7 +585,7 @@ def test_attention_mfma_launches_that_fill_the_chip(case):
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
 
 
-@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 4), (True, 3, 4), (True, 1, 8)])
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (False, 3, 4), (True, 1, 4), (True, 3, 4), (True, 1, 8)])
 @pytest.mark.parametrize("needle", [0, 15, 16, 31, 32, 299, 300 - 17, 141])
 def test_attention_mfma_finds_one_far_key(needle, arrangement):
     def craft(qs, ks, vs):
@@ -605,7 +611,7 @@ LONG_CASES = [  # nh, nkv, d, bs, lens, new
 ]
 
 
-@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 4), (True, 1, 8), (True, 4, 8), (True, 7, 4)])
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (False, 4, 4), (True, 1, 4), (True, 1, 8), (True, 4, 8), (True, 7, 4)])
 @pytest.mark.parametrize("case", LONG_CASES)
 def test_attention_mfma_long_contexts(case, arrangement):
     nh, nkv, d, bs, lens, new = case
@@ -615,7 +621,7 @@ def test_attention_mfma_long_contexts(case, arrangement):
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
 
 
-@pytest.mark.parametrize("arrangement", [(False, 1, 4), (True, 1, 8), (True, 3, 8)])
+@pytest.mark.parametrize("arrangement", [(False, 1, 4), (False, 3, 4), (True, 1, 8), (True, 3, 8)])
 @pytest.mark.parametrize("needle", [0, 511, 512, 519, 520, 1023, 1024, 1090])
 def test_attention_mfma_finds_one_key_beyond_the_first_pages(needle, arrangement):
     """1,100 keys in pages of 8: the one key that matters lies before, at and after the places where the
