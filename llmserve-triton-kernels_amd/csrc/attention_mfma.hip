@@ -564,13 +564,15 @@ __global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt
     }
 }
 
-// Merge of the splits of every (token, head), split 0 first: a workgroup per token, a thread per head and 4 dimensions.
+// Merge of the splits of every (token, head), split 0 first: a thread per token, head and 4 dimensions (blockIdx.x:
+// token, blockIdx.y: which blockDim.x of the token's heads * head_dim / 4 pieces).
 __global__ __launch_bounds__(256) void attn_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ ws_o,
                                                          const float* __restrict__ ws_ml, int token_begin, int n_heads,
                                                          int head_dim, int num_splits) {
     const int token = token_begin + blockIdx.x;
     const int q4 = head_dim / 4;
-    for (int idx = threadIdx.x; idx < n_heads * q4; idx += blockDim.x) {
+    const int idx = blockIdx.y * blockDim.x + threadIdx.x;
+    if (idx < n_heads * q4) {
         const int head = idx / q4, d = 4 * (idx % q4);
         const size_t item0 = ((size_t)token * n_heads + head) * num_splits;
         const float2* ml = reinterpret_cast<const float2*>(ws_ml) + item0;  // (maximum, sum) of each split
@@ -611,6 +613,14 @@ template <int DB, int CG>
 static void launch_prompt_cg(dim3 grid, bool paired, const AttnArgs& a, hipStream_t stream) {
     if (paired) attn_prompt_kernel<DB, true, CG, PROMPT_WB><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
     else attn_prompt_kernel<DB, false, CG, PROMPT_WB><<<grid, PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
+}
+
+// Few tokens (decoding): small workgroups, so that the merge reaches many CUs; many tokens: 256 threads each.
+static void launch_merge(void* out, int out_stride, const float* ws_o, const float* ws_ml, int token_begin, int n_tokens,
+                         int n_heads, int head_dim, int num_splits, hipStream_t stream) {
+    const int threads = n_tokens <= 64 ? 64 : 256, pieces = n_heads * (head_dim / 4);
+    attn_merge_kernel<<<dim3(n_tokens, (pieces + threads - 1) / threads), threads, 0, stream>>>(
+        (bf16*)out, out_stride, ws_o, ws_ml, token_begin, n_heads, head_dim, num_splits);
 }
 
 static int launch_prompt(int db, int cg, dim3 grid, bool paired, const AttnArgs& a, hipStream_t stream) {
@@ -692,8 +702,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                 fprintf(stderr, "llmserve kernel launch failed: %s\n", hipGetErrorString(e1));
                 return LLMS_ERR_LAUNCH;
             }
-            attn_merge_kernel<<<n_tokens, 256, 0, stream>>>((bf16*)out, out_stride, ws_o, ws_ml, token_begin, n_heads,
-                                                            head_dim, num_splits);
+            launch_merge(out, out_stride, ws_o, ws_ml, token_begin, n_tokens, n_heads, head_dim, num_splits, stream);
         }
     } else {
         bool paired = window == 0 && head_dim <= 192 && num_splits == 1;  // early and late blocks of tokens in one workgroup
@@ -719,8 +728,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                 fprintf(stderr, "llmserve kernel launch failed: %s\n", hipGetErrorString(e1));
                 return LLMS_ERR_LAUNCH;
             }
-            attn_merge_kernel<<<n_tokens, 256, 0, stream>>>((bf16*)out, out_stride, ws_o, ws_ml, token_begin, n_heads,
-                                                            head_dim, num_splits);
+            launch_merge(out, out_stride, ws_o, ws_ml, token_begin, n_tokens, n_heads, head_dim, num_splits, stream);
         }
     }
     LLMS_LAUNCH_CHECK();
