@@ -139,16 +139,24 @@ def wide_model_dir(request, tmp_path_factory):
 
 @pytest.mark.parametrize("mode", list(MODES))
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
-def test_replay_at_full_layer_sizes(wide_model_dir, dtype_name, mode):
+def test_replay_at_full_layer_sizes(wide_model_dir, dtype_name, mode, monkeypatch):
     """The tiny configurations never reach the paths that the sizes of a real model choose: products whose
     K is shared out to several workgroups and summed by the norm, the library's product for many rows, 8 waves
     per decoded token, a vocabulary of 2,000 tiles."""
     model_dir, cfg = wide_model_dir
-    seqs = {f"w{i}": traces.random_ids(cfg["vocab_size"], n, 2000 + i) for i, n in enumerate([40, 150, 300])}
+    # (700 tokens: portions behind a prefix long enough for attention to share a block's keys out to workgroups)
+    seqs = {f"w{i}": traces.random_ids(cfg["vocab_size"], n, 2000 + i) for i, n in enumerate([40, 150, 300, 700])}
     steps = MODES[mode](seqs)
     num_blocks = traces.tokens_needed(steps, round_to=16) // 16
+    from llmserve.ops import library as ops
+    shared_out = []
+    original = ops.attention_mfma
+    monkeypatch.setattr(ops, "attention_mfma", lambda *a, **kw: (shared_out.append((kw.get("split_waves", False),
+                                                                                    kw.get("num_splits", 1))), original(*a, **kw))[1])
     outputs = replay_in_process(model_dir, dtype_name, steps, 16, num_blocks)
     check_against_plain(model_dir, dtype_name, seqs, steps, outputs)
+    if dtype_name == "bfloat16" and mode == "portions":
+        assert any(not waves and splits > 1 for waves, splits in shared_out), "no portion shared its keys out"
 
 
 def test_mixed_trace_reuses_pages(model_dirs):
