@@ -235,10 +235,10 @@ class CacheManager:
             held = [b for t in self.tables[g.group_id].values() for b in t if b >= 0]
             if len(held) != len(set(held)):
                 raise AssertionError(f"group {g.group_id}: a page is held twice")
-            if set(held) != alloc._used:
+            if set(held) != alloc.held_ids():
                 raise AssertionError(f"group {g.group_id}: tables and allocator disagree")
             if alloc.num_free + alloc.num_used != alloc.num_blocks:
                 raise AssertionError(f"group {g.group_id}: pages lost")
         slots = list(self.slot_of.values())
-        if len(slots) != len(set(slots)) or set(slots) != self._slot_alloc._used:
+        if len(slots) != len(set(slots)) or set(slots) != self._slot_alloc.held_ids():
             raise AssertionError("state slots are not unique among live requests")

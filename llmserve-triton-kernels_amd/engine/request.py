@@ -25,11 +25,11 @@ class Request:
     seed: int = 0
     generated: list[int] = field(default_factory=list)
     status: Status = Status.WAITING
-    num_computed_tokens: int = 0  # tokens of prompt + generated already in the cache
-    token_times: list[float] = field(default_factory=list)
+    num_computed_tokens: int = 0  # how much of prompt + generated the cache holds
+    token_times: list[float] = field(default_factory=list)  # host clock at which each generated token was read
     finish_time: float | None = None
-    finish_reason: str | None = None  # "stop" | "length" | "abort"
-    num_preemptions: int = 0
+    finish_reason: str | None = None  # one of "stop" (end-of-sequence id), "length", "abort"
+    num_preemptions: int = 0  # times its pages were taken away and it started over
 
     @property
     def num_tokens(self) -> int:
@@ -70,13 +70,17 @@ class EngineStats:
 @dataclass
 class GenerationResult:
     tokens: list[int]
-    ttft_s: float  # time to first token
-    step_latencies_s: list[float] = field(default_factory=list)  # gaps between later tokens
+    ttft_s: float  # from the call to the first generated token
+    step_latencies_s: list[float] = field(default_factory=list)  # from each token to the next
     total_s: float = 0.0
     peak_memory_bytes: int = 0
     finish_reason: str | None = None
 
     @property
     def decode_tokens_per_s(self) -> float:
-        total = sum(self.step_latencies_s)
-        return len(self.step_latencies_s) / total if total > 0 else 0.0
+        """Tokens after the first, per second of the time between them (0 when there were none)."""
+        gaps = self.step_latencies_s
+        spent = sum(gaps)
+        if not gaps or spent <= 0:
+            return 0.0
+        return len(gaps) / spent

@@ -124,12 +124,12 @@ class ModelRunner:
         self.manager.free_sequence(seq_id)
 
     # ---- the step ---------------------------------------------------------------------------
-    @torch.inference_mode()
     @property
     def takes_device_tokens(self) -> bool:
         """Whether `step(..., device_tokens=...)` is available (decode-only steps are replayed graphs)."""
         return self._use_graphs
 
+    @torch.inference_mode()
     def step(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None) -> torch.Tensor:
         """Run the entries' tokens as one batch; float32 logits [sum(len(want)), vocab] in the
         order of the entries and of their `want`.  Raises `OutOfBlocks` (nothing changed) when

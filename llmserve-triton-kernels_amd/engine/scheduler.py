@@ -1,46 +1,58 @@
 """Continuous batching above the step function.
 
-Public face as the reference's `ContinuousBatchingEngine`
-(src/llmserve/scheduler/engine.py:83-194): `add_request`, `step() -> list[TokenEvent]`,
-`run_until_complete`, `abort`, `reset`, `snapshot`, `validate_request`, `has_unfinished`.
+The class answers to the reference's names (`ContinuousBatchingEngine` with `add_request`,
+`step() -> list[TokenEvent]`, `run_until_complete`, `abort`, `reset`, `snapshot`,
+`validate_request`, `has_unfinished`: src/llmserve/scheduler/engine.py:83-178), so a caller of
+the reference finds what it knows.  What happens inside a step is this engine's own:
 
-One `step()` is one call of the step function with everything that is scheduled:
-  1. aborts asked for since the last step;
-  2. pages: every running request must be able to store the tokens it already has
-     (`prompt + generated`); while the free pages do not cover that, the most recently
-     admitted request is preempted: its pages are freed and it goes to the front of the
-     queue, to be recomputed later (src/llmserve/scheduler/engine.py:255-274);
-  3. one token for every request that is decoding;
-  4. the next portion of every request whose prompt is not yet in the cache, cut to the
-     step's token budget (and to `max_prefill_chunk`);
-  5. new requests, first come first served and never out of order, while there are slots,
-     budget and pages: the whole of `prompt + generated` is reserved at admission and one
-     spare page is kept per live request (src/llmserve/scheduler/engine.py:212-234), so a
-     prompt that was admitted can always finish and only decoding can run out of pages.
-A request samples when its portion reaches the end of `prompt + generated`.  The reference
-prefills a prompt whole and runs two forwards per iteration; portions under a token budget
-and the single mixed batch are this engine's own.
+  one `step()` = one call of the step function, carrying everything that is scheduled:
+    a. requests whose cancellation was asked for leave;
+    b. the pool must hold the tokens every live request already has (`prompt + generated`);
+       while it does not, the request admitted last gives its pages back and returns to the
+       head of the queue, to be computed again from its first token (the reference's rule
+       for a pool that runs dry: src/llmserve/scheduler/engine.py:255-274);
+    c. every request that is decoding brings its one token;
+    d. every request whose prompt is not yet in the cache brings its next portion, cut to what
+       is left of the step's token budget (and to `max_prefill_chunk`);
+    e. queued requests are admitted in arrival order, never one past another, while there is a
+       slot, budget and room: the pages of the whole `prompt + generated` are set aside at
+       admission and one more page per live request stays free
+       (src/llmserve/scheduler/engine.py:212-234), so an admitted prompt can always be
+       finished and only decoding can run short of pages.
+  A request samples when its portion reaches the end of `prompt + generated`.  (The reference
+  runs a whole-prompt forward and a decode forward per iteration; portions under a token budget
+  in one mixed batch replace both here.)
 
-Reading tokens back one step late.  With a sampler that can leave its ids on the device
-(`sample_async`) a step does not wait for them: they are read at the start of the next `step()`.
-And when that next step is a plain continuation (the same requests, all decoding, nothing
-waiting, aborted or about to reach its length, pages at hand) it is started first, on the ids
-still on the device, and the ids of the step before are read while it runs, so the GPU never
-waits for the host's bookkeeping.  A request that turns out to have stopped (its end-of-sequence
-token) has then one more row in the step already started; that row's token is dropped.  Events
-and `token_times` therefore lag a step behind the GPU; which tokens are produced does not change.
+Reading the sampled ids late.  A sampler that offers `sample_async` leaves its ids on the
+device; they are fetched when the next `step()` begins.  If that next step merely continues
+the last one (the same requests, all decoding, nobody queued or cancelled or at its last
+token, pages at hand) and the runner can take its tokens from the device, it is launched
+first and the ids of the step before are fetched while it runs: the GPU never waits for the
+host.  A request that turns out to have produced its end-of-sequence token then already has a
+row in the launched step; that row's result is thrown away.  Events and `token_times` thus
+trail the GPU by one step; the tokens themselves are the same.
 """
 
 from __future__ import annotations
 
 import threading
 from collections import deque
+from dataclasses import dataclass
 from time import perf_counter
 
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import request_seed
 from .request import EngineStats, Request, Status, TokenEvent
 from .runner import StepEntry
+
+
+@dataclass
+class _Share:
+    """One request's part of a planned step."""
+
+    request: Request
+    count: int  # tokens it feeds
+    samples: bool  # whether the last of them ends `prompt + generated`
 
 
 class ContinuousBatchingEngine:
@@ -57,246 +69,265 @@ class ContinuousBatchingEngine:
         self.max_num_batched_tokens = max_num_batched_tokens
         self.max_prefill_chunk = max_prefill_chunk
         self.seed = seed
-        self.waiting: deque[Request] = deque()
-        self.running: list[Request] = []  # in order of admission
+        self.waiting: deque[Request] = deque()  # arrival order; a preempted request re-enters at the left
+        self.running: list[Request] = []  # admission order, oldest first
         self.finished: dict[int, Request] = {}
         self.stats = EngineStats()
-        self._next_id = 0
-        self._aborts: set[int] = set()
-        self._lock = threading.Lock()
-        # the requests (in row order) and the token ids of a step that has been started but not read yet
-        self._pending: tuple[list[Request], object] | None = None
-        self._lagged = hasattr(sampler, "sample_async")
+        self._ids_issued = 0
+        self._cancel: set[int] = set()
+        self._cancel_lock = threading.Lock()
+        # (requests in row order, ids still on the device) of a launched step that has not been fetched
+        self._in_flight: tuple[list[Request], object] | None = None
+        self._reads_late = hasattr(sampler, "sample_async")
 
-    # ------------------------------------------------------------------ public
+    # ================================================================== intake
     def validate_request(self, prompt_len: int, max_new_tokens: int) -> None:
-        """The reference's four checks (src/llmserve/scheduler/engine.py:111-125)."""
-        if prompt_len < 1:
-            raise ValueError("prompt must contain at least one token")
-        if max_new_tokens < 1:
-            raise ValueError("max_new_tokens must be >= 1")
-        total = prompt_len + max_new_tokens
-        limit = self.runner.max_model_len
-        if total > limit:
-            raise ValueError(f"prompt + max_new_tokens = {total} exceeds model limit {limit}")
-        if self.manager.blocks_for(total) > self.manager.num_blocks:
-            raise ValueError(f"request needs {self.manager.blocks_for(total)} KV blocks but the pool has "
-                             f"only {self.manager.num_blocks}")
+        """Refuse, with `ValueError`, a request that could never be served: an empty prompt, nothing
+        to generate, more positions than the model has, more pages than the pool has (the four checks
+        of src/llmserve/scheduler/engine.py:111-125)."""
+        positions = prompt_len + max_new_tokens
+        pages = self.manager.blocks_for(positions)
+        problems = (
+            (prompt_len < 1, "an empty prompt cannot be continued: give at least one token"),
+            (max_new_tokens < 1, f"max_new_tokens is {max_new_tokens}; nothing would be generated"),
+            (positions > self.runner.max_model_len,
+             f"{prompt_len} prompt tokens and {max_new_tokens} new ones need {positions} positions; "
+             f"the model stops at {self.runner.max_model_len}"),
+            (pages > self.manager.num_blocks,
+             f"{positions} tokens fill {pages} cache pages and the whole pool is {self.manager.num_blocks}"),
+        )
+        for failed, message in problems:
+            if failed:
+                raise ValueError(message)
 
     def add_request(self, prompt_ids: list[int], params: SamplingParams, *, req_id: int | None = None,
                     arrival_time: float | None = None) -> int:
+        """Queue a request; returns its id (the caller's, or the next unused number)."""
         self.validate_request(len(prompt_ids), params.max_new_tokens)
         vocab = self.runner.vocab_size
-        bad = [t for t in prompt_ids if not 0 <= t < vocab]
-        if bad:
-            raise ValueError(f"prompt holds token ids outside the vocabulary [0, {vocab}): {bad[:5]}")
-        if req_id is None:
-            req_id = self._next_id
-        self._next_id = max(self._next_id, req_id + 1)
-        self.waiting.append(Request(
-            req_id=req_id, prompt_ids=list(prompt_ids), params=params,
-            arrival_time=perf_counter() if arrival_time is None else arrival_time,
-            seed=request_seed(params, self.seed, req_id)))
-        return req_id
+        strangers = [t for t in prompt_ids if not 0 <= t < vocab]
+        if strangers:
+            raise ValueError(f"token ids {strangers[:5]} of the prompt are not in the vocabulary of {vocab} entries")
+        rid = self._ids_issued if req_id is None else req_id
+        self._ids_issued = max(self._ids_issued, rid + 1)
+        when = perf_counter() if arrival_time is None else arrival_time
+        self.waiting.append(Request(req_id=rid, prompt_ids=list(prompt_ids), params=params, arrival_time=when,
+                                    seed=request_seed(params, self.seed, rid)))
+        return rid
 
     def abort(self, req_id: int) -> None:
-        """Takes effect at the start of the next step.  Thread-safe."""
-        with self._lock:
-            self._aborts.add(req_id)
+        """Ask for a request to be dropped; it leaves when the next step begins.  May be called from
+        another thread."""
+        with self._cancel_lock:
+            self._cancel.add(req_id)
 
     def reset(self) -> None:
-        """Drop every request in flight and give back what they hold."""
-        self._pending = None
-        for r in self.running:
-            self.manager.free_sequence(r.req_id)
-        self.running.clear()
+        """Forget everything in flight: queued requests vanish, live ones give back what they hold,
+        a launched step's ids are never fetched."""
+        self._in_flight = None
+        while self.running:
+            self.manager.free_sequence(self.running.pop().req_id)
         self.waiting.clear()
 
+    # ================================================================== observation
     def has_unfinished(self) -> bool:
-        return bool(self.waiting or self.running)
+        return len(self.waiting) + len(self.running) > 0
 
     def snapshot(self) -> dict:
-        return {
-            "running": len(self.running), "waiting": len(self.waiting),
-            "free_blocks": self.manager.num_free_blocks, "total_blocks": self.manager.num_blocks,
-            "kv_utilization": round(self.manager.utilization(), 4),
-            "internal_fragmentation": round(self.manager.internal_fragmentation(), 4),
-            "preemptions": self.stats.preemptions, "tokens_generated": self.stats.tokens_generated,
-            "steps": self.stats.steps, "prefill_tokens": self.stats.prefill_tokens,
-            "decode_tokens": self.stats.decode_tokens,
-        }
+        """Counters for a dashboard (the keys of src/llmserve/scheduler/engine.py:164-173, and this
+        engine's own beside them)."""
+        m, s = self.manager, self.stats
+        report = dict(running=len(self.running), waiting=len(self.waiting), free_blocks=m.num_free_blocks,
+                      total_blocks=m.num_blocks, kv_utilization=round(m.utilization(), 4),
+                      internal_fragmentation=round(m.internal_fragmentation(), 4))
+        for name in ("preemptions", "tokens_generated", "steps", "prefill_tokens", "decode_tokens"):
+            report[name] = getattr(s, name)
+        return report
 
     def run_until_complete(self) -> dict[int, Request]:
         while self.has_unfinished():
             self.step()
         return self.finished
 
-    # -------------------------------------------------------------------- step
+    # ================================================================== one step
     def step(self) -> list[TokenEvent]:
         events: list[TokenEvent] = []
         self.stats.steps += 1
-        if self._pending is not None:
-            if self._can_continue():
-                self._continue(events)
+        if self._in_flight is not None:
+            if self._is_plain_continuation():
+                self._launch_continuation(events)
                 return events
-            self._read_pending(events)
-        self._process_aborts(events)
-        preempted = self._make_room()
-        plan = self._plan(admit=not preempted)
-        if not plan:
-            return events
-        entries = [StepEntry(r.req_id, r.tokens(r.num_computed_tokens, n),
-                             [n - 1] if samples else []) for r, n, samples in plan]
-        logits = self.runner.step(entries)
-        sampling = [r for r, _, samples in plan if samples]
-        items = [(r.params, r.seed, len(r.generated)) for r in sampling]
-        for r, n, _ in plan:
-            if n == 1 and r.num_computed_tokens > 0 and r.generated:
-                self.stats.decode_tokens += 1
-            else:
-                self.stats.prefill_tokens += n
-            r.num_computed_tokens += n
-        if self._lagged:
-            self._pending = (sampling, self.sampler.sample_async(logits, items))  # read at the next step
-        else:
-            self._append_tokens(sampling, self.sampler.sample(logits, items), events)
+            self._fetch_in_flight(events)
+        self._drop_cancelled(events)
+        evicted = self._evict_until_known_tokens_fit()
+        shares = self._plan(admit=not evicted)
+        if shares:
+            self._launch(shares, events)
         return events
 
-    # ------------------------------------------------- a step whose tokens are read later
-    def _read_pending(self, events: list[TokenEvent]) -> None:
-        reqs, pending = self._pending
-        self._pending = None
-        self._append_tokens(reqs, pending.result(), events)
-
-    def _can_continue(self) -> bool:
-        """Whether the next step is the pending one's requests again, each with the one token
-        that is still on the device."""
-        reqs, pending = self._pending
-        if (self.waiting or self._aborts or not reqs or len(reqs) != len(self.running)
-                or not getattr(self.runner, "takes_device_tokens", False)):
-            return False
-        need = 0
-        for r, q in zip(reqs, self.running):
-            # the same requests in the same order, none stopped meanwhile, none at its last token
-            if r is not q or r.status is not Status.RUNNING or len(r.generated) + 2 > r.params.max_new_tokens:
-                return False
-            if r.num_computed_tokens != r.num_tokens:  # (every token it has is in the cache: it is decoding)
-                return False
-            need += self.manager.extra_blocks_needed(r.req_id, 1)
-        return need <= self.manager.num_free_blocks
-
-    def _continue(self, events: list[TokenEvent]) -> None:
-        reqs, pending = self._pending
-        logits = self.runner.step([StepEntry(r.req_id, [0], [0]) for r in reqs], device_tokens=pending.device)
-        following = self.sampler.sample_async(logits, [(r.params, r.seed, len(r.generated) + 1) for r in reqs])
-        for r in reqs:
-            r.num_computed_tokens += 1
-        self.stats.decode_tokens += len(reqs)
-        self._read_pending(events)  # the step before; a request that stopped there is skipped from now on
-        self._pending = (reqs, following)
-
-    # --------------------------------------------------------------- internals
-    def _process_aborts(self, events: list[TokenEvent]) -> None:
-        with self._lock:
-            aborts, self._aborts = self._aborts, set()
-        for rid in sorted(aborts):
-            req = next((r for r in self.waiting if r.req_id == rid), None)
-            if req is not None:
-                self.waiting.remove(req)
+    def _launch(self, shares: list[_Share], events: list[TokenEvent]) -> None:
+        entries = []
+        for s in shares:
+            r = s.request
+            entries.append(StepEntry(r.req_id, r.tokens(r.num_computed_tokens, s.count),
+                                     [s.count - 1] if s.samples else []))
+        logits = self.runner.step(entries)
+        drawing = [s.request for s in shares if s.samples]
+        draws = [(r.params, r.seed, len(r.generated)) for r in drawing]
+        for s in shares:
+            r = s.request
+            decoding = s.count == 1 and r.generated and r.num_computed_tokens > 0
+            if decoding:
+                self.stats.decode_tokens += 1
             else:
-                req = next((r for r in self.running if r.req_id == rid), None)
-                if req is None:
-                    continue  # already finished
-                self.running.remove(req)
+                self.stats.prefill_tokens += s.count
+            r.num_computed_tokens += s.count
+        if self._reads_late:
+            self._in_flight = (drawing, self.sampler.sample_async(logits, draws))
+        else:
+            self._take_tokens(drawing, self.sampler.sample(logits, draws), events)
+
+    # ------------------------------------------------------------------ ids fetched a step late
+    def _fetch_in_flight(self, events: list[TokenEvent]) -> None:
+        requests, ids = self._in_flight
+        self._in_flight = None
+        self._take_tokens(requests, ids.result(), events)
+
+    def _is_plain_continuation(self) -> bool:
+        """Whether the coming step is exactly the launched one's requests again, each with the one
+        token that still sits on the device, and the runner can read it there."""
+        requests, _ = self._in_flight
+        if not getattr(self.runner, "takes_device_tokens", False):
+            return False
+        if self.waiting or self._cancel or not requests or len(requests) != len(self.running):
+            return False
+        pages = 0
+        for launched, live in zip(requests, self.running):
+            if launched is not live or live.status is not Status.RUNNING:
+                return False  # another set of requests, or one has stopped meanwhile
+            if live.num_computed_tokens != live.num_tokens:
+                return False  # its known tokens are not all in the cache: it is not decoding
+            if len(live.generated) + 2 > live.params.max_new_tokens:
+                return False  # the token on the device is its last: no step follows it
+            pages += self.manager.extra_blocks_needed(live.req_id, 1)
+        return pages <= self.manager.num_free_blocks
+
+    def _launch_continuation(self, events: list[TokenEvent]) -> None:
+        requests, ids = self._in_flight
+        placeholder = [StepEntry(r.req_id, [0], [0]) for r in requests]  # the values come from `ids.device`
+        logits = self.runner.step(placeholder, device_tokens=ids.device)
+        after = self.sampler.sample_async(logits, [(r.params, r.seed, len(r.generated) + 1) for r in requests])
+        for r in requests:
+            r.num_computed_tokens += 1
+        self.stats.decode_tokens += len(requests)
+        self._fetch_in_flight(events)  # the step before this one; who stopped there is skipped from now on
+        self._in_flight = (requests, after)
+
+    # ------------------------------------------------------------------ leaving
+    def _retire(self, request: Request, reason: str, token: int | None, events: list[TokenEvent]) -> None:
+        """Record a request's end (its pages are already back)."""
+        request.status, request.finish_reason, request.finish_time = Status.FINISHED, reason, perf_counter()
+        self.finished[request.req_id] = request
+        events.append(TokenEvent(request.req_id, token, True, reason))
+
+    def _drop_cancelled(self, events: list[TokenEvent]) -> None:
+        with self._cancel_lock:
+            asked, self._cancel = sorted(self._cancel), set()
+        if not asked:
+            return
+        queued = {r.req_id: r for r in self.waiting}
+        live = {r.req_id: r for r in self.running}
+        for rid in asked:
+            if rid in queued:
+                self.waiting.remove(queued[rid])
+                self._retire(queued[rid], "abort", None, events)
+            elif rid in live:
+                self.running.remove(live[rid])
                 self.manager.free_sequence(rid)
-            self._finish(req, "abort", events, emit_token=None)
+                self._retire(live[rid], "abort", None, events)
+            # anything else has ended by itself, or never existed
 
-    def _known_need(self, r: Request) -> int:
-        """Pages `r` still has to take for the tokens it already has."""
-        return self.manager.extra_blocks_needed(r.req_id, r.num_tokens - self.manager.lengths[r.req_id])
+    def _take_tokens(self, requests: list[Request], tokens: list[int], events: list[TokenEvent]) -> None:
+        """Append each sampled id to its request and let those go that are done."""
+        stamp = perf_counter()
+        for request, token in zip(requests, tokens):
+            if request.status is not Status.RUNNING:
+                continue  # stopped one step earlier; this row was computed in vain
+            request.generated.append(token)
+            request.token_times.append(stamp)
+            self.stats.tokens_generated += 1
+            p = request.params
+            if p.eos_token_id is not None and token == p.eos_token_id:
+                verdict = "stop"
+            elif len(request.generated) >= p.max_new_tokens:
+                verdict = "length"
+            else:
+                events.append(TokenEvent(request.req_id, token, False))
+                continue
+            self.running.remove(request)
+            self.manager.free_sequence(request.req_id)
+            self._retire(request, verdict, token, events)
 
-    def _make_room(self) -> bool:
-        """Preempt, newest admission first, until the running requests' known tokens fit."""
-        preempted = False
-        while len(self.running) > 1 and sum(self._known_need(r) for r in self.running) > self.manager.num_free_blocks:
-            self._preempt(self.running[-1])
-            preempted = True
-        return preempted
+    # ------------------------------------------------------------------ pages
+    def _pages_owed(self, request: Request) -> int:
+        """Pages the request has yet to take for tokens it already has."""
+        missing = request.num_tokens - self.manager.lengths[request.req_id]
+        return self.manager.extra_blocks_needed(request.req_id, missing)
 
-    def _preempt(self, req: Request) -> None:
-        self.running.remove(req)
-        self.manager.free_sequence(req.req_id)
-        req.status = Status.WAITING
-        req.num_computed_tokens = 0
-        req.num_preemptions += 1
-        self.stats.preemptions += 1
-        self.waiting.appendleft(req)  # prompt + generated are recomputed when it is admitted again
+    def _evict_until_known_tokens_fit(self) -> bool:
+        """Send the most recent admissions back to the queue until what remains can store its known
+        tokens; the oldest request is never sent back.  True if anyone was."""
+        evicted = False
+        while len(self.running) > 1:
+            owed = sum(self._pages_owed(r) for r in self.running)
+            if owed <= self.manager.num_free_blocks:
+                break
+            victim = self.running.pop()
+            self.manager.free_sequence(victim.req_id)
+            victim.status = Status.WAITING
+            victim.num_computed_tokens = 0  # everything it has, generated tokens too, is computed again
+            victim.num_preemptions += 1
+            self.stats.preemptions += 1
+            self.waiting.appendleft(victim)
+            evicted = True
+        return evicted
 
-    def _portion(self, remaining: int, budget: int) -> int:
-        n = min(remaining, budget)
-        if self.max_prefill_chunk is not None and remaining > 1:
-            n = min(n, self.max_prefill_chunk)
-        return n
+    # ------------------------------------------------------------------ planning
+    def _cut(self, outstanding: int, budget: int) -> int:
+        size = min(outstanding, budget)
+        if outstanding > 1 and self.max_prefill_chunk is not None:
+            size = min(size, self.max_prefill_chunk)
+        return size
 
-    def _plan(self, admit: bool) -> list[tuple[Request, int, bool]]:
-        """(request, tokens it feeds, whether it samples) for this step."""
+    def _plan(self, admit: bool) -> list[_Share]:
         budget = self.max_num_batched_tokens
-        plan: list[tuple[Request, int, bool]] = []
-        decoding = [r for r in self.running if r.num_tokens - r.num_computed_tokens == 1]
-        prefilling = [r for r in self.running if r.num_tokens - r.num_computed_tokens > 1]
-        for r in decoding + prefilling:
+        shares: list[_Share] = []
+
+        def give(request: Request, outstanding: int) -> None:
+            nonlocal budget
+            size = self._cut(outstanding, budget)
+            shares.append(_Share(request, size, size == outstanding))
+            budget -= size
+
+        backlog = {id(r): r.num_tokens - r.num_computed_tokens for r in self.running}
+        # decoding requests first (one token each), then prompts that are under way
+        for r in sorted(self.running, key=lambda r: backlog[id(r)] > 1):  # (stable: admission order within each)
             if budget <= 0:
                 break
-            remaining = r.num_tokens - r.num_computed_tokens
-            n = self._portion(remaining, budget)
-            plan.append((r, n, n == remaining))
-            budget -= n
+            give(r, backlog[id(r)])
         if not admit:
-            return plan
-        reserved = sum(self._known_need(r) for r in self.running)
-        while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
-            req = self.waiting[0]
-            total = req.num_tokens
-            need = self.manager.blocks_for(total)
-            headroom = len(self.running)  # one spare page per request already live
-            if self.manager.num_free_blocks - reserved - need < headroom:
-                break
-            if self.manager.num_free_slots < 1:
-                break
+            return shares
+        set_aside = sum(self._pages_owed(r) for r in self.running)
+        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs:
+            candidate = self.waiting[0]
+            pages = self.manager.blocks_for(candidate.num_tokens)
+            spare = len(self.running)  # one page per request already live stays free
+            if self.manager.num_free_blocks - set_aside - pages < spare or self.manager.num_free_slots < 1:
+                break  # the head of the queue does not fit, and nobody overtakes it
             self.waiting.popleft()
-            self.manager.add_sequence(req.req_id)
-            req.status = Status.RUNNING
-            req.num_computed_tokens = 0
-            self.running.append(req)
-            reserved += need
-            n = self._portion(total, budget)
-            plan.append((req, n, n == total))
-            budget -= n
-        return plan
-
-    def _append_tokens(self, reqs: list[Request], tokens: list[int], events: list[TokenEvent]) -> None:
-        now = perf_counter()
-        for r, tok in zip(reqs, tokens):
-            if r.status is not Status.RUNNING:
-                continue  # it stopped a step earlier; this row was computed for nothing
-            r.generated.append(tok)
-            r.token_times.append(now)
-            self.stats.tokens_generated += 1
-            reason = None
-            if r.params.eos_token_id is not None and tok == r.params.eos_token_id:
-                reason = "stop"
-            elif len(r.generated) >= r.params.max_new_tokens:
-                reason = "length"
-            if reason:
-                self.running.remove(r)
-                self.manager.free_sequence(r.req_id)
-                self._finish(r, reason, events, emit_token=tok)
-            else:
-                events.append(TokenEvent(r.req_id, tok, False))
-
-    def _finish(self, req: Request, reason: str, events: list[TokenEvent], emit_token: int | None) -> None:
-        req.status = Status.FINISHED
-        req.finish_reason = reason
-        req.finish_time = perf_counter()
-        self.finished[req.req_id] = req
-        events.append(TokenEvent(req.req_id, emit_token, True, reason))
+            self.manager.add_sequence(candidate.req_id)
+            candidate.status, candidate.num_computed_tokens = Status.RUNNING, 0
+            self.running.append(candidate)
+            set_aside += pages
+            give(candidate, candidate.num_tokens)
+        return shares
