@@ -39,6 +39,32 @@ def test_greedy_generation_matches_plain(model_dirs, name, lengths, new):
     assert llm.generate_naive(prompts[1], SamplingParams(max_new_tokens=6)).tokens == want[1][:6]
 
 
+@pytest.mark.parametrize("name,lengths,new", [("a", [5, 17, 33], 16), ("b", [1, 7, 40, 64, 100], 24)])
+def test_generation_without_graphs_feeds_the_sampled_ids(model_dirs, name, lengths, new):
+    """With graphs off every decode step is launched kernel by kernel and takes its tokens from the host:
+    the scheduler must then wait for the ids instead of starting the next step on placeholders."""
+    from llmserve import SamplingParams
+
+    vocab = TINY[name][0]["vocab_size"]
+    prompts = [traces.random_ids(vocab, n, 300 + i) for i, n in enumerate(lengths)]
+    cfg, w = plain_llama.read_model_dir(model_dirs[name], torch.float32)
+    want = [plain_llama.generate(cfg, w, p, new, torch.float32) for p in prompts]
+    llm = _llm(model_dirs[name], name, "float32", use_graphs=False)
+    assert llm.runner.takes_device_tokens is False
+    assert [r.tokens for r in llm.generate(prompts, SamplingParams(max_new_tokens=new))] == want
+    from llmserve.engine.runner import StepEntry
+
+    llm.runner.add_sequence("x")
+    with pytest.raises(ValueError, match="from the host only"):
+        llm.runner.step([StepEntry("x", [0], [0])], device_tokens=torch.zeros(1, dtype=torch.int32, device="cuda"))
+    llm.runner.free_sequence("x")
+    # seeded temperature sampling: the same tokens as with graphs, whatever launches the steps
+    params = [SamplingParams(temperature=0.8, seed=40 + i, max_new_tokens=new) for i in range(len(prompts))]
+    eager = [r.tokens for r in llm.generate(prompts, params)]
+    replayed = [r.tokens for r in _llm(model_dirs[name], name, "float32").generate(prompts, params)]
+    assert eager == replayed and len({tuple(t) for t in eager}) == len(prompts)
+
+
 @pytest.mark.parametrize("name", ["a", "b"])
 def test_preemption_by_recompute_keeps_greedy_tokens(model_dirs, name):
     """14 pages of 4 tokens and four requests of 6 + 14 tokens cannot all grow: some are thrown

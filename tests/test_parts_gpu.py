@@ -448,3 +448,27 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype_name):
             traces.assert_close(got[rid], plain_toy_forward(w, ids, dtype), dtype, f"toy {rid} {dtype_name}")
         assert runner.manager.num_free_slots == 3
         assert all(a.num_free == 24 for a in runner.manager.allocators.values())
+
+
+def test_toy_architecture_generates_through_the_scheduler(tmp_path):
+    """The toy mixer reads host fields, so no step of this model is replayed from a graph and the runner takes
+    tokens from the host only: generation through the entry point must still feed every sampled id back."""
+    from safetensors.torch import load_file
+
+    from llmserve import LLM, EngineConfig, SamplingParams
+    from llmserve.weights import write_random_model
+
+    register_toy()
+    write_random_model(tmp_path, TOY, seed=6, std=0.06)
+    w = load_file(str(tmp_path / "model.safetensors"))
+    llm = LLM(tmp_path, dtype="float32", engine=EngineConfig(block_size=8, num_blocks=48, max_num_seqs=3,
+                                                              max_num_batched_tokens=16))
+    assert not llm.runner.takes_device_tokens
+    prompts = [traces.random_ids(97, n, 700 + i) for i, n in enumerate([9, 21, 4])]
+    results = llm.generate(prompts, SamplingParams(max_new_tokens=10))
+    for prompt, result in zip(prompts, results):
+        ids = list(prompt)
+        for _ in range(10):
+            ids.append(int(plain_toy_forward(w, ids, torch.float32)[-1].argmax()))
+        assert result.tokens == ids[len(prompt):]
+    assert llm.runner.manager.num_free_slots == 3
