@@ -24,6 +24,9 @@
 //
 // Needs block_size % 8 == 0, head_dim % 16 == 0 and <= 256, 16-byte aligned rows.
 #include "common.h"
+#include "attention_mfma.h"
+
+#include <mutex>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -732,6 +735,69 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
         }
     }
     LLMS_LAUNCH_CHECK();
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------------------------------
+// Decoding with the keys of a request shared out to several workgroups, without a workspace from the caller:
+// the partial results go through a fixed array in device memory that this library owns.  Every GPU the library
+// runs on holds its own copy of the array (at its own address) until the process ends.
+static __device__ __align__(256) unsigned char scratch[LLMS_ATTN_SCRATCH_BYTES];
+
+#define LLMS_MAX_DEVICES 64
+static void* scratch_ptr[LLMS_MAX_DEVICES];  // device address of `scratch` on each GPU (null: not asked yet)
+static std::mutex scratch_mutex;
+
+// The array's address on the current device.  In host code `scratch` is only a handle for the runtime, never
+// an address a kernel could use: the address comes from hipGetSymbolAddress, once per device.
+static int scratch_of_current_device(unsigned char** out) {
+    int dev = -1;
+    LLMS_HIP_CHECK(hipGetDevice(&dev));
+    LLMS_REQUIRE(dev >= 0 && dev < LLMS_MAX_DEVICES, "attention_decode_noalloc: device index out of range");
+    std::lock_guard<std::mutex> hold(scratch_mutex);
+    if (scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        LLMS_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        LLMS_REQUIRE(p != nullptr && ((uintptr_t)p % 256) == 0, "attention_decode_noalloc: no aligned device address for the scratch array");
+        scratch_ptr[dev] = p;
+    }
+    *out = static_cast<unsigned char*>(scratch_ptr[dev]);
+    return LLMS_OK;
+}
+
+extern "C" {
+
+int llms_attention_decode_noalloc(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
+                                  const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
+                                  const int* cu_seqlens, const int* context_lens, int seq_begin, int n_seqs,
+                                  int token_begin, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                                  int block_size, int window, float scale, int num_splits, int waves,
+                                  hipStream_t stream) {
+    LLMS_REQUIRE(num_splits >= 2, "attention_decode_noalloc: num_splits must be >= 2 (one split needs no scratch: use attention_mfma)");
+    LLMS_REQUIRE(token_begin >= 0 && n_tokens > 0 && n_heads > 0 && head_dim > 0 && head_dim % 16 == 0,
+                 "attention_decode_noalloc: sizes must be positive, head_dim a multiple of 16");
+    // partial results are indexed by absolute token row, as in attention_mfma: [row][head][split][D] sums, then
+    // [row][head][split][2] (maximum, sum of weights)
+    const unsigned long long items = (unsigned long long)(token_begin + n_tokens) * n_heads * num_splits;
+    const unsigned long long o_bytes = items * head_dim * sizeof(float);  // (a multiple of 64)
+    const unsigned long long ml_bytes = items * 2 * sizeof(float);
+    if (o_bytes + ml_bytes > LLMS_ATTN_SCRATCH_BYTES) {
+        fprintf(stderr, "llmserve kernel argument error: attention_decode_noalloc: %llu rows x heads x splits need %llu bytes "
+                        "of scratch, the fixed array has %u\n", items, o_bytes + ml_bytes, (unsigned)LLMS_ATTN_SCRATCH_BYTES);
+        return LLMS_ERR_ARG;
+    }
+    unsigned char* base = nullptr;
+    if (int e = scratch_of_current_device(&base)) return e;
+    float* ws_o = reinterpret_cast<float*>(base);
+    float* ws_ml = reinterpret_cast<float*>(base + o_bytes);
+    // Nothing in the array has to start at zero: the merge reads, for every token row of the launch, exactly the
+    // entries the attention kernel has just written (a request without keys writes nothing and its rows of `out`
+    // are meaningless, as with a caller's workspace).
+    return llms_attention_mfma(out, out_stride, q, q_stride, k_pool, v_pool, block_tables, table_rows, max_blocks,
+                               cu_seqlens, context_lens, seq_begin, n_seqs, /*max_new=*/1, token_begin, n_tokens, n_heads,
+                               n_kv_heads, head_dim, block_size, window, scale, /*split_waves=*/1, num_splits, waves, ws_o,
+                               ws_ml, stream);
 }
 
 }  // extern "C"
