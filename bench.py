@@ -111,6 +111,7 @@ def serve(args) -> int:
         return eng, [eng.finished[i] for i in ids], time.perf_counter() - t0, steps
 
     run(min(4, args.requests), 8)  # warm-up: kernels loaded, graphs of the small batches captured
+    runner.rows_asked = runner.rows_run = 0
     eng, reqs, total_s, steps = run(args.requests, args.new_tokens)
     generated = sum(len(r.generated) for r in reqs)
     ttft = [r.token_times[0] - r.arrival_time for r in reqs]
@@ -130,6 +131,9 @@ def serve(args) -> int:
         "itl_ms": {"p50": round(percentile(itl, 0.5) * 1e3, 3), "p90": round(percentile(itl, 0.9) * 1e3, 3),
                    "p99": round(percentile(itl, 0.99) * 1e3, 3), "max": round(max(itl) * 1e3, 3)},
         "preemptions": eng.stats.preemptions,
+        # rows the steps held, rows that ran with the padding of buckets and graphs, and the padded fraction
+        "rows": {"asked": runner.rows_asked, "run": runner.rows_run,
+                 "padding": round(runner.rows_run / max(runner.rows_asked, 1) - 1, 4)},
     }
     print(json.dumps(line))
     return 0

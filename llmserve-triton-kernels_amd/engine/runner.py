@@ -5,8 +5,8 @@ The reference has no single step function: its scheduler runs one padded forward
 prompts and one for decoding requests (src/llmserve/scheduler/engine.py:186-193,236-246).
 Here one call runs everything a step holds as one flat batch: portions of prompts beside
 single decoded tokens, cut anywhere.  Steps of single tokens are replayed from HIP graphs (one per
-batch size and context range); so are other steps whose shape comes again after a run in which the
-device waited for the host's launches.
+batch size and context range); other steps run at the sizes of a bucket and are replayed from a graph
+from the bucket's second use on.
 """
 
 from __future__ import annotations
@@ -69,12 +69,13 @@ class ModelRunner:
         self._uploader = BatchUploader(device)
         self._graphs: dict[tuple[int, int], "_DecodeGraph"] = {}
         self._use_graphs = engine_config.use_graphs and model.graph_safe()
-        # graphs of steps that bring portions of prompts, by the sizes they were captured for (most
-        # recently used last); a shape is captured when it comes again after a run that the host could
-        # not keep up with (`_step_shapes`: what was measured when the shape ran kernel by kernel)
-        self._step_graphs: dict[tuple, "_StepGraph"] = {}
-        self._step_shapes: dict[tuple, dict] = {}
+        # steps that bring portions of prompts run at the sizes of a bucket: fixed buffers per bucket (most
+        # recently used last), and a graph from the bucket's second use on
+        self._buckets: dict[tuple, "_StepBucket"] = {}
         self._step_graph_pool = None
+        # rows the steps were asked to run, and rows they ran with the padding of buckets and graphs
+        self.rows_asked = 0
+        self.rows_run = 0
 
     # ---- construction ---------------------------------------------------------------------
     @staticmethod
@@ -124,20 +125,27 @@ class ModelRunner:
         self.manager.free_sequence(seq_id)
 
     # ---- the step ---------------------------------------------------------------------------
+    lends_logits = True  # `step(..., borrow=True)` is understood
+
     @property
     def takes_device_tokens(self) -> bool:
         """Whether `step(..., device_tokens=...)` is available (decode-only steps are replayed graphs)."""
         return self._use_graphs
 
     @torch.inference_mode()
-    def step(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None) -> torch.Tensor:
+    def step(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None, *,
+             borrow: bool = False) -> torch.Tensor:
         """Run the entries' tokens as one batch; float32 logits [sum(len(want)), vocab] in the
         order of the entries and of their `want`.  Raises `OutOfBlocks` (nothing changed) when
         the pages do not suffice.
 
         `device_tokens` (int32, one per entry, on the device): every entry brings one token, and
         its value is taken from this tensor instead of the entry (whose token is a placeholder):
-        the ids the sampler chose for the previous step, which the host need not have seen yet."""
+        the ids the sampler chose for the previous step, which the host need not have seen yet.
+
+        The logits belong to the caller.  With `borrow` they may instead be a view of memory that a
+        replayed graph owns: valid until the next call of `step`, which may overwrite them (work
+        queued on the same stream before that call still reads the right values)."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         if device_tokens is not None:
@@ -173,18 +181,17 @@ class ModelRunner:
             row += len(e.tokens)
         logit_rows = [first_row[id(e)] + w for e in entries for w in e.want]
         self.storage.clear_state(layout.fresh_slots)
-        if self._use_graphs and all(len(e.tokens) == 1 for e in ordered):
+        owned = True
+        if not self._use_graphs:  # launched kernel by kernel, on exactly the step's tokens
+            batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
+            logits = self.model.forward(batch, self.storage)
+        elif all(len(e.tokens) == 1 for e in ordered):
             logits = self._replay_decode(layout, [e.tokens[0] for e in ordered], logit_rows, device_tokens)
+            owned = False
         else:
-            logits = self._replay_step(layout, [e.tokens for e in ordered], logit_rows) if self._use_graphs else None
-            if logits is None:
-                watch = self._watch_eager_step(layout, len(logit_rows)) if self._use_graphs else None
-                batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
-                logits = self.model.forward(batch, self.storage)
-                if watch is not None:
-                    watch()
+            logits, owned = self._run_bucketed_step(layout, [e.tokens for e in ordered], logit_rows)
         self.manager.release_passed(layout.seq_ids)
-        return logits
+        return logits if owned or borrow else logits.clone()
 
     # ---- decode-only steps as HIP graphs --------------------------------------------------------
     def _replay_decode(self, layout, tokens: list[int], logit_rows: list[int],
@@ -209,26 +216,37 @@ class ModelRunner:
         if device_tokens is not None:  # (all entries bring one token, so their order is the caller's)
             graph.static.batch.token_ids[:n].copy_(device_tokens)
         graph.graph.replay()
+        self.rows_run += capacity
+        self.rows_asked += n
         if logit_rows == list(range(n)):
             return graph.logits[:n]
         return graph.logits[torch.tensor(logit_rows, dtype=torch.long, device=self.device)]
 
-
-    # ---- steps with portions of prompts as HIP graphs ----------------------------------------------
+    # ---- steps with portions of prompts: padded to a bucket of sizes, replayed from the second time on ------
     MAX_STEP_GRAPHS = 32
+    CAPTURE_AT_USE = 2  # a bucket is captured as a graph when it comes for this many-th time
 
     @staticmethod
-    def _step_shape(n_decode: int, n_prefill: int, n_prefill_tokens: int, n_logits: int, context: int) -> tuple:
+    def _row_bucket(n: int) -> int:
+        """Rows of portions are padded to a multiple of 16, or of an eighth of the power of two below them if
+        that is more: never more than 15 rows or 12.5 % beyond what was asked."""
+        if n <= 0:
+            return 0
+        floor = 1 << (n.bit_length() - 1)
+        unit = max(16, floor // 8)
+        return -(-n // unit) * unit
+
+    @classmethod
+    def _step_shape(cls, n_decode: int, n_prefill: int, n_prefill_tokens: int, n_logits: int, context: int) -> tuple:
         """The sizes a step is padded to: powers of two for the requests, the wanted rows and the reach of
-        the contexts, multiples of 64 (up to 512) or 256 for the rows of the portions."""
+        the contexts (which only sets how attention spreads its work), `_row_bucket` for the rows of the portions."""
         def pow2(x, least=1):
             p = least
             while p < x:
                 p *= 2
             return p
-        step = 64 if n_prefill_tokens <= 512 else 256
-        return (pow2(n_decode) if n_decode else 0, pow2(n_prefill), -(-n_prefill_tokens // step) * step,
-                pow2(max(n_logits, 1)), pow2(context, 256))  # (the reach sets how attention spreads its work)
+        return (pow2(n_decode) if n_decode else 0, pow2(n_prefill), cls._row_bucket(n_prefill_tokens),
+                pow2(max(n_logits, 1)), pow2(context, 256))
 
     def _shape_of(self, layout, n_logits: int) -> tuple:
         n_dec = 0
@@ -237,72 +255,100 @@ class ModelRunner:
         context = max(s + c for s, c in zip(layout.starts, layout.counts))
         return self._step_shape(n_dec, len(layout.counts) - n_dec, sum(layout.counts[n_dec:]), n_logits, context)
 
-    def _watch_eager_step(self, layout, n_logits: int):
-        """Time a step that is launched kernel by kernel, on the host and on the device; returns the
-        function to call when everything has been launched."""
-        from time import perf_counter
-
-        record = self._step_shapes.setdefault(self._shape_of(layout, n_logits), {})
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record(torch.cuda.current_stream(self.device))
-        t0 = perf_counter()
-
-        def done():
-            end.record(torch.cuda.current_stream(self.device))
-            record.update(host_ms=(perf_counter() - t0) * 1e3, start=start, end=end)
-        return done
-
-    def _host_bound(self, record: dict) -> bool:
-        """Whether the last kernel-by-kernel run of this shape kept the device waiting for launches: the
-        device was done about when the host was (a step that keeps the device busy for longer gains nothing
-        from a graph, and capturing one costs two runs)."""
-        end = record.get("end")
-        if end is None or not end.query():
-            return False
-        return record["start"].elapsed_time(end) < 1.5 * record["host_ms"]
-
-    def _replay_step(self, layout, tokens: list[list[int]], logit_rows: list[int]) -> torch.Tensor | None:
-        """A step with portions of prompts, replayed from the graph captured for its padded sizes; None
-        when this shape has no graph (the caller then runs it kernel by kernel).  Launching the ~160
-        kernels of a step one by one costs the host milliseconds; a replay costs microseconds."""
+    def _run_bucketed_step(self, layout, tokens: list[list[int]], logit_rows: list[int]) -> tuple[torch.Tensor, bool]:
+        """A step with portions of prompts.  It always runs at the sizes of its bucket (`_step_shape`), from
+        fixed buffers in which what the step does not use belongs to dummy requests without keys: launched
+        kernel by kernel the first time the bucket comes, captured as a HIP graph the second time and replayed
+        from then on.  Which kernels run, and in which arrangement, is therefore a function of the bucket
+        alone: the first run and every replay give the same bits, and so do two runs of one trace.
+        Returns (logits, whether the caller owns them)."""
         shape = self._shape_of(layout, len(logit_rows))
-        graph = self._step_graphs.pop(shape, None)
-        if graph is None:
-            record = self._step_shapes.get(shape)
-            if record is None or not self._host_bound(record):
-                return None
-            if len(self._step_graphs) >= self.MAX_STEP_GRAPHS:
-                self._step_graphs.pop(next(iter(self._step_graphs)))  # the least recently used
+        bucket = self._buckets.pop(shape, None)
+        if bucket is None:
+            if len(self._buckets) >= self.MAX_STEP_GRAPHS:
+                self._buckets.pop(next(iter(self._buckets)))  # the least recently used
+            bucket = _StepBucket(self, shape)
+        self._buckets[shape] = bucket  # (most recently used last)
+        bucket.static.fill(layout, tokens, logit_rows)
+        bucket.uses += 1
+        self.rows_run += bucket.static.num_rows
+        self.rows_asked += sum(layout.counts)
+        n = len(logit_rows)
+        if bucket.graph is None and bucket.uses >= self.CAPTURE_AT_USE:
             if self._step_graph_pool is None:
                 self._step_graph_pool = torch.cuda.graph_pool_handle()
-            graph = _StepGraph(self, shape, self._step_graph_pool)
-        self._step_graphs[shape] = graph
-        graph.static.fill(layout, tokens, logit_rows)
-        graph.graph.replay()
-        return graph.logits[: len(logit_rows)]
+            bucket.capture(self, self._step_graph_pool)
+        if bucket.graph is not None:
+            bucket.graph.replay()
+            return bucket.logits[:n], False
+        return bucket.run(self)[:n], True
+
+    @property
+    def _step_graphs(self) -> dict:
+        """The buckets that have been captured as graphs."""
+        return {shape: b for shape, b in self._buckets.items() if b.graph is not None}
 
 
-class _StepGraph:
-    """One captured step for up to `decode` single tokens, `prefill` portions of `tokens` rows in all and
-    `logits` wanted rows, contexts up to `reach` (which only sets how decode attention spreads its work).
-    All such graphs share one memory pool: they never run at the same time, and a step's logits are
-    consumed before the next step is replayed."""
+class _capturing:
+    """`with _capturing(graph, pool):` records the launches inside it into `graph`.  Python's cycle collector
+    stays off meanwhile, after one collection up front: an object it finds dead in the middle of a capture may
+    own device memory or another graph, and giving those back is not allowed while a stream is capturing."""
 
-    def __init__(self, runner: "ModelRunner", shape: tuple, pool):
+    def __init__(self, graph: "torch.cuda.CUDAGraph", pool=None):
+        self._context = torch.cuda.graph(graph, pool=pool) if pool is not None else torch.cuda.graph(graph)
+
+    def __enter__(self):
+        import gc
+
+        gc.collect()
+        self._gc_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            return self._context.__enter__()
+        except BaseException:
+            if self._gc_was_on:
+                gc.enable()
+            raise
+
+    def __exit__(self, *exc):
+        import gc
+
+        try:
+            return self._context.__exit__(*exc)
+        finally:
+            if self._gc_was_on:
+                gc.enable()
+
+
+class _StepBucket:
+    """Fixed buffers, and from the second use on a captured graph, for steps of up to `decode` single tokens,
+    `prefill` portions of `tokens` rows in all and `logits` wanted rows, contexts up to `reach`.  All such
+    graphs share one memory pool: they never run at the same time, and a step's logits are consumed (or
+    copied) before the next step is replayed."""
+
+    def __init__(self, runner: "ModelRunner", shape: tuple):
         decode, prefill, tokens, logits, reach = shape
         group_ids = [g.group_id for g in runner.manager.paged_groups]
         self.static = StaticStepBatch(decode, prefill, tokens, logits, runner.storage, group_ids, runner.device)
         batch = self.static.batch
         batch.max_context = batch.max_decode_context = reach
-        # a first run outside the capture: libraries load, memory pools warm up (the buffers describe
-        # dummy requests only, so nothing is stored or attended to)
+        self.uses = 0
+        self.graph = None
+        self.logits = None
+
+    def run(self, runner: "ModelRunner") -> torch.Tensor:
+        """Launch the step that `static.fill` described, kernel by kernel.  (The runner is an argument, not a
+        field: a bucket that pointed back at its runner would keep both alive until the cycle collector runs.)"""
         self.static.apply_table_updates()
-        runner.model.forward(batch, runner.storage)
+        return runner.model.forward(self.static.batch, runner.storage)
+
+    def capture(self, runner: "ModelRunner", pool) -> None:
+        """Record the same launches as a graph (nothing runs; an earlier `run` of this bucket has loaded every
+        library and warmed the memory pools)."""
         torch.cuda.synchronize(runner.device)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph, pool=pool):
-            self.static.apply_table_updates()
-            self.logits = runner.model.forward(batch, runner.storage)
+        with _capturing(self.graph, pool):
+            self.logits = self.run(runner)
 
 
 class _DecodeGraph:
@@ -319,6 +365,6 @@ class _DecodeGraph:
         runner.model.forward(batch, runner.storage)
         torch.cuda.synchronize(runner.device)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        with _capturing(self.graph):
             self.static.apply_table_updates()
             self.logits = runner.model.forward(batch, runner.storage)

@@ -79,6 +79,8 @@ class ContinuousBatchingEngine:
         # (requests in row order, ids still on the device) of a launched step that has not been fetched
         self._in_flight: tuple[list[Request], object] | None = None
         self._reads_late = hasattr(sampler, "sample_async")
+        # a runner whose logits may live in a replayed graph's memory lends them: they are sampled at once
+        self._step_options = {"borrow": True} if getattr(runner, "lends_logits", False) else {}
 
     # ================================================================== intake
     def validate_request(self, prompt_len: int, max_new_tokens: int) -> None:
@@ -171,7 +173,7 @@ class ContinuousBatchingEngine:
             r = s.request
             entries.append(StepEntry(r.req_id, r.tokens(r.num_computed_tokens, s.count),
                                      [s.count - 1] if s.samples else []))
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, **self._step_options)  # (sampled from before the next step)
         drawing = [s.request for s in shares if s.samples]
         draws = [(r.params, r.seed, len(r.generated)) for r in drawing]
         for s in shares:
@@ -215,7 +217,7 @@ class ContinuousBatchingEngine:
     def _launch_continuation(self, events: list[TokenEvent]) -> None:
         requests, ids = self._in_flight
         placeholder = [StepEntry(r.req_id, [0], [0]) for r in requests]  # the values come from `ids.device`
-        logits = self.runner.step(placeholder, device_tokens=ids.device)
+        logits = self.runner.step(placeholder, device_tokens=ids.device, **self._step_options)
         after = self.sampler.sample_async(logits, [(r.params, r.seed, len(r.generated) + 1) for r in requests])
         for r in requests:
             r.num_computed_tokens += 1

@@ -89,10 +89,11 @@ def test_replay_without_graphs(model_dirs, dtype_name, mode):
 
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 def test_steps_with_portions_are_replayed_from_graphs(model_dirs, dtype_name):
-    """A step shape that comes a second time is captured as a graph (padded to its bucket with dummy
-    requests and rows) and replayed from then on: the mixed and the portioned trace, run twice through one
-    runner, must hit such graphs and still agree with the plain implementation, whatever the padding
-    holds (the cache is poisoned) and whichever pages are used again."""
+    """A step with portions always runs at the sizes of its bucket, kernel by kernel the first time the bucket
+    comes and from a captured graph from the second time on.  The mixed and the portioned trace, run twice
+    through one runner, hit such graphs; both passes agree with the plain implementation, whatever the
+    padding holds (the cache is poisoned) and whichever pages are used again, and they agree with each
+    other to the bit: which kernels run is a function of the bucket, not of the way it is launched."""
     from llmserve.config import EngineConfig
     from llmserve.engine.replay import Replayer
     from llmserve.engine.runner import ModelRunner
@@ -106,6 +107,7 @@ def test_steps_with_portions_are_replayed_from_graphs(model_dirs, dtype_name):
         runner = ModelRunner.from_folder(model_dirs[name], EngineConfig(dtype=dtype_name, block_size=block_size,
                                                                         num_blocks=num_blocks, max_num_seqs=4))
         runner.storage.poison()
+        passes = []
         for _ in range(2):
             rep = Replayer(runner)
             outputs = {}
@@ -116,8 +118,60 @@ def test_steps_with_portions_are_replayed_from_graphs(model_dirs, dtype_name):
                     outputs[rec["step"]] = logits.float().cpu()
             check_against_plain(model_dirs[name], dtype_name, seqs, steps, outputs)
             assert runner.manager.num_free_blocks == num_blocks
+            passes.append(outputs)
         assert runner._step_graphs, f"{mode}: no step with portions was replayed from a graph"
-        assert len(runner._step_graphs) <= runner.MAX_STEP_GRAPHS
+        assert len(runner._buckets) <= runner.MAX_STEP_GRAPHS
+        assert all(b.graph is not None for b in runner._buckets.values() if b.uses >= runner.CAPTURE_AT_USE)
+        for step, first in passes[0].items():
+            assert torch.equal(first, passes[1][step]), f"{mode} step {step}: a replay differs from the first run"
+
+
+def test_one_trace_gives_the_same_bits_in_fresh_runners(model_dirs):
+    """The same mixed bfloat16 trace in two fresh runners: equal to the bit (no decision depends on a clock)."""
+    seqs = sequences("b")
+    steps = traces.mixed(seqs, seed=3)
+    bs = TINY["b"][1]
+    num_blocks = traces.tokens_needed(steps, round_to=bs) // bs
+    first = replay_in_process(model_dirs["b"], "bfloat16", steps + steps_renumbered(steps), bs, num_blocks)
+    second = replay_in_process(model_dirs["b"], "bfloat16", steps + steps_renumbered(steps), bs, num_blocks)
+    assert first.keys() == second.keys() and len(first) > len(steps)
+    for step in first:
+        assert torch.equal(first[step], second[step]), f"step {step} differs between two runs"
+
+
+def steps_renumbered(steps):
+    """The same trace once more, as later steps (its requests ended, so their names are free again)."""
+    return [dict(rec, step=rec["step"] + len(steps)) for rec in steps]
+
+
+def test_returned_logits_survive_the_next_step(model_dirs):
+    """Logits that `step` returns belong to the caller: a later step, replayed from the same graph, must not
+    change them (the scheduler, which samples at once, borrows them instead)."""
+    from llmserve.config import EngineConfig
+    from llmserve.engine.runner import ModelRunner, StepEntry
+
+    runner = ModelRunner.from_folder(model_dirs["a"], EngineConfig(dtype="float32", block_size=16, num_blocks=8,
+                                                                   max_num_seqs=2))
+    runner.add_sequence("s")
+    ids = traces.random_ids(256, 12, 3)
+    runner.step([StepEntry("s", ids[:8], [7])])
+    kept, copies = [], []
+    for t in ids[8:]:
+        kept.append(runner.step([StepEntry("s", [t], [0])]))
+        copies.append(kept[-1].cpu().clone())
+    lent = runner.step([StepEntry("s", [ids[0]], [0])], borrow=True)
+    assert all(torch.equal(k.cpu(), c) for k, c in zip(kept, copies))
+    assert len({c.numpy().tobytes() for c in copies}) == len(copies)
+    assert lent.shape == (1, 256)
+    runner.free_sequence("s")
+
+
+def test_padding_of_steps_is_bounded():
+    from llmserve.engine.runner import ModelRunner
+
+    for n in list(range(1, 700)) + [1000, 2047, 2048, 2049, 5000]:
+        padded = ModelRunner._row_bucket(n)
+        assert n <= padded and (padded - n < 16 or padded - n <= n / 8)
 
 
 WIDE = {  # layer sizes of real models, few layers
