@@ -98,19 +98,15 @@ class CacheManager:
         return max(a.num_used for a in self.allocators.values()) / self.num_blocks
 
     def internal_fragmentation(self) -> float:
-        """Fraction of slots in held pages that hold no token (src/llmserve/kvcache/paged.py:149-153);
-        first paged group."""
-        if not self.paged_groups:
-            return 0.0
-        g = self.paged_groups[0]
-        held = self.allocators[g.group_id].num_used * self.block_size
-        if held == 0:
-            return 0.0
-        live = 0
-        for seq, table in self.tables[g.group_id].items():
-            first = next((i for i, b in enumerate(table) if b >= 0), len(table))
-            live += self.lengths[seq] - first * self.block_size
-        return 1.0 - live / held
+        """Fraction of slots in held pages that hold no token (src/llmserve/kvcache/paged.py:149-153), over
+        all paged groups: a windowed group holds fewer pages per request than one that keeps every key."""
+        held = live = 0
+        for g in self.paged_groups:
+            held += self.allocators[g.group_id].num_used * self.block_size
+            for seq, table in self.tables[g.group_id].items():
+                first = next((i for i, b in enumerate(table) if b >= 0), len(table))
+                live += self.lengths[seq] - first * self.block_size
+        return 1.0 - live / held if held else 0.0
 
     # ---- requests -----------------------------------------------------------------------
     def has_sequence(self, seq_id) -> bool:
@@ -144,11 +140,11 @@ class CacheManager:
         del self.lengths[seq_id]
 
     def extra_blocks_needed(self, seq_id, new_tokens: int) -> int:
-        """Pages one group must add for `new_tokens` more tokens (the same for every group)."""
-        if not self.paged_groups:
-            return 0
-        table = self.tables[self.paged_groups[0].group_id][seq_id]
-        return max(0, self.blocks_for(self.lengths[seq_id] + new_tokens) - len(table))
+        """Pages that `new_tokens` more tokens cost in the group where they cost most (`num_free_blocks` is
+        the tightest group's count, so the two compare).  A table keeps its length when a windowed group gives
+        pages back, so today every group answers alike; nothing here relies on that."""
+        want = self.blocks_for(self.lengths[seq_id] + new_tokens)
+        return max((max(0, want - len(self.tables[g.group_id][seq_id])) for g in self.paged_groups), default=0)
 
     def can_append(self, seq_ids, counts) -> bool:
         need = sum(self.extra_blocks_needed(s, n) for s, n in zip(seq_ids, counts))

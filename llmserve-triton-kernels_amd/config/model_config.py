@@ -58,10 +58,14 @@ class LlamaConfig:
         hidden = int(d["hidden_size"])
         if heads <= 0:
             raise ConfigError(f"num_attention_heads={heads} must be positive")
-        head_dim = d.get("head_dim")
-        if head_dim is None:
-            # src/llmserve/config.py:22-24: head_dim = hidden_size // num_heads
-            head_dim = hidden // heads
+        # src/llmserve/config.py:22-24: head_dim = hidden_size // num_heads, always; a config.json that names
+        # another head_dim describes a model the reference cannot hold, and is refused rather than guessed at
+        head_dim = hidden // heads
+        if d.get("head_dim") is not None and int(d["head_dim"]) != head_dim:
+            raise ConfigError(f"head_dim={d['head_dim']} differs from hidden_size // num_attention_heads = {head_dim}; "
+                              "the Llama decoder here takes head_dim from those two")
+        if hidden % heads:
+            raise ConfigError(f"hidden_size={hidden} is not a multiple of num_attention_heads={heads}")
         cfg = cls(
             vocab_size=int(d["vocab_size"]),
             hidden_size=hidden,
@@ -111,10 +115,11 @@ class LlamaConfig:
         return d
 
 
-# Named sizes, as config.json dictionaries.  "tiny" is the reference's own test
+# Named sizes of the Llama architecture, as config.json dictionaries (models/llama.py registers them with the
+# architecture; `config.preset(name)` finds them).  "tiny" is the reference's own test
 # configuration (src/llmserve/config.py:26-37); the others are the shapes this engine
 # is tested and measured on.
-PRESETS: dict[str, dict] = {
+LLAMA_PRESETS: dict[str, dict] = {
     "tiny": dict(vocab_size=256, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
                  num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=512),
     "tiny-a": dict(vocab_size=256, hidden_size=64, intermediate_size=176, num_hidden_layers=2,
@@ -134,13 +139,3 @@ PRESETS: dict[str, dict] = {
                        max_position_embeddings=4096, rope_theta=10000.0, rms_norm_eps=1e-5),
 }
 
-
-def preset(name: str) -> dict:
-    """config.json dictionary of a named size (with the Llama architecture name filled in)."""
-    key = name.lower().replace("_", "-")
-    if key not in PRESETS:
-        raise ConfigError(f"unknown preset {name!r}; known: {sorted(PRESETS)}")
-    d = dict(PRESETS[key])
-    d.setdefault("architectures", ["LlamaForCausalLM"])
-    d.setdefault("model_type", "llama")
-    return d

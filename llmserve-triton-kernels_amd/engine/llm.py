@@ -12,7 +12,7 @@ from time import perf_counter
 import torch
 
 from ..config.engine_config import EngineConfig
-from ..config.model_config import PRESETS, preset
+from ..config.registry import is_preset, preset
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .request import GenerationResult
@@ -24,7 +24,7 @@ class LLM:
     def __init__(self, model: str | Path | dict, *, dtype: str | None = None, random_weights: bool = False,
                  seed: int = 0, engine: EngineConfig | None = None, device=None):
         """`model`: a folder with config.json and safetensors, or, with `random_weights`, the
-        name of a size (`llmserve.config.PRESETS`) or a config.json dictionary."""
+        name of a size (`llmserve.config.preset_names()`: whatever the registered architectures offer) or a config.json dictionary."""
         engine = engine or EngineConfig()
         if dtype is not None:
             engine.dtype = dtype
@@ -34,7 +34,7 @@ class LLM:
             config = model if isinstance(model, dict) else preset(str(model))
             self.runner = ModelRunner.from_random(config, seed, engine, device)
         else:
-            if isinstance(model, str) and not Path(model).exists() and model.lower().replace("_", "-") in PRESETS:
+            if isinstance(model, str) and not Path(model).exists() and is_preset(model):
                 raise FileNotFoundError(f"{model!r} is a size, not a folder; pass random_weights=True to run it "
                                         "with random weights")
             if not Path(model).is_dir():

@@ -6,7 +6,7 @@ model.norm, lm_head."""
 
 from __future__ import annotations
 
-from ..config.model_config import LlamaConfig
+from ..config.model_config import LLAMA_PRESETS, LlamaConfig
 from ..config.registry import register_architecture
 from ..parts.spec import LayerSpec, ModelSpec, PartSpec
 
@@ -35,4 +35,4 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         weights={"embedding": "model.embed_tokens.", "final_norm": "model.norm.", "head": "lm_head."})
 
 
-register_architecture("LlamaForCausalLM", LlamaConfig, llama_spec, model_type="llama")
+register_architecture("LlamaForCausalLM", LlamaConfig, llama_spec, model_type="llama", presets=LLAMA_PRESETS)

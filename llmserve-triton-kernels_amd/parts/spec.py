@@ -102,10 +102,11 @@ class StateCacheSpec:
 
 @dataclass(frozen=True)
 class ParamInfo:
-    """Shape of one tensor of a part, how random weights fill it ("matrix" N(0, std),
-    "norm" 1 + N(0, norm_std), "zeros") and how it is stored ("model": cast to the engine's
-    dtype; "stored": as the file holds it, 32-bit stays 32-bit, integers become int32)."""
+    """Shape of one tensor of a part, how random weights fill it (the name of a registered initializer:
+    "matrix" N(0, std), "norm" 1 + N(0, norm_std), "zeros", or one a part registered with
+    `weights.register_initializer`; or the filling function itself) and how it is stored ("model": cast to
+    the engine's dtype; "stored": as the file holds it, 32-bit stays 32-bit, integers become int32)."""
 
     shape: tuple[int, ...]
-    init: str = "matrix"
+    init: Any = "matrix"
     dtype: str = "model"

@@ -14,10 +14,41 @@ from __future__ import annotations
 import hashlib
 import json
 from pathlib import Path
+from typing import Callable
 
 import torch
 
 from ..parts.spec import ParamInfo
+
+# How a tensor is filled, by the name a part puts into `ParamInfo.init`.  A filler is
+#     fill(shape, generator, device, options) -> float32 tensor
+# with the tensor's own seeded generator and `options` = {"std": ..., "norm_std": ...} (the scales the caller of
+# `random_tensors` chose).  A part with another kind of tensor (a decay in (0, 1), the taps of a convolution)
+# registers a filler of its own, or puts the function itself into `ParamInfo.init`; this file is not edited.
+INITIALIZERS: dict[str, Callable] = {}
+
+
+def register_initializer(name: str, fill: Callable | None = None):
+    def put(fn):
+        INITIALIZERS[name] = fn
+        return fn
+
+    return put if fill is None else put(fill)
+
+
+@register_initializer("matrix")
+def _fill_matrix(shape, generator, device, options):
+    return options["std"] * torch.randn(shape, generator=generator, dtype=torch.float32, device=device)
+
+
+@register_initializer("norm")
+def _fill_norm(shape, generator, device, options):
+    return 1.0 + options["norm_std"] * torch.randn(shape, generator=generator, dtype=torch.float32, device=device)
+
+
+@register_initializer("zeros")
+def _fill_zeros(shape, generator, device, options):
+    return torch.zeros(shape, dtype=torch.float32, device=device)
 
 
 def _generator(seed: int, name: str, device) -> torch.Generator:
@@ -30,16 +61,12 @@ def _generator(seed: int, name: str, device) -> torch.Generator:
 def random_tensor(name: str, info: ParamInfo, seed: int, dtype: torch.dtype, device="cpu",
                   std: float = 0.02, norm_std: float = 0.01) -> torch.Tensor:
     shape = tuple(info.shape)
-    if info.init == "zeros":
-        return torch.zeros(shape, dtype=dtype, device=device)
-    g = _generator(seed, name, device)
-    t = torch.randn(shape, generator=g, dtype=torch.float32, device=device)
-    if info.init == "norm":
-        t = 1.0 + norm_std * t
-    elif info.init == "matrix":
-        t = std * t
-    else:
-        raise ValueError(f"unknown init {info.init!r} for {name}")
+    fill = info.init if callable(info.init) else INITIALIZERS.get(info.init)
+    if fill is None:
+        raise ValueError(f"{name}: no initializer named {info.init!r}; registered: {sorted(INITIALIZERS)}")
+    t = fill(shape, _generator(seed, name, device), device, {"std": std, "norm_std": norm_std})
+    if tuple(t.shape) != shape:
+        raise ValueError(f"{name}: its initializer made shape {tuple(t.shape)}, not {shape}")
     return t.to(dtype)
 
 

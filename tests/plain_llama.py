@@ -1,6 +1,6 @@
 """Plain, slow Llama: whole sequences, no cache, one function for each part.
 
-Written from the formulas of the reference (paths are relative to /root/reference);
+Written from the formulas of the reference (the paths cited are relative to the reference's root);
 it shares no code with the engine: weights come straight from the safetensors file
 as a dict keyed by checkpoint name, the configuration is the raw config.json dict.
 
@@ -118,6 +118,16 @@ def swiglu(x, w, prefix):
     return linear(silu(g) * u, w[prefix + "down_proj.weight"])
 
 
+def decoder_layer(x, w, prefix, n_heads, n_kv_heads, head_dim, theta, eps):
+    """src/llmserve/model/llama.py:131-135: x = x + attn(norm1(x)); x = x + mlp(norm2(x)): both norms sit in front
+    of their branch, and the second branch reads the stream after the first was added."""
+    h = rms_norm(x, w[prefix + "input_layernorm.weight"], eps)
+    x = x + attention_block(x=h, w=w, prefix=prefix + "self_attn.", n_heads=n_heads, n_kv_heads=n_kv_heads,
+                            head_dim=head_dim, theta=theta)
+    h = rms_norm(x, w[prefix + "post_attention_layernorm.weight"], eps)
+    return x + swiglu(h, w, prefix + "mlp.")
+
+
 # --------------------------------------------------------------------------- model
 
 
@@ -146,12 +156,7 @@ def forward(cfg: dict, w: dict[str, torch.Tensor], ids: list[int], dtype: torch.
     eps = cfg.get("rms_norm_eps", 1e-5)
     x = w["model.embed_tokens.weight"][torch.tensor(ids, dtype=torch.long)].to(dtype)
     for i in range(cfg["num_hidden_layers"]):
-        p = f"model.layers.{i}."
-        h = rms_norm(x, w[p + "input_layernorm.weight"], eps)
-        x = x + attention_block(x=h, w=w, prefix=p + "self_attn.", n_heads=n_heads,
-                                n_kv_heads=n_kv, head_dim=head_dim, theta=theta)
-        h = rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
-        x = x + swiglu(h, w, p + "mlp.")
+        x = decoder_layer(x, w, f"model.layers.{i}.", n_heads, n_kv, head_dim, theta, eps)
     x = rms_norm(x, w["model.norm.weight"], eps)
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return x.float() @ head.float().t()  # logits kept in 32-bit

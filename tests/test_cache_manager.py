@@ -167,6 +167,20 @@ def test_random_requests_keep_the_books(ops, window):
     assert all(a.num_free == 24 for a in m.allocators.values()) and m.num_free_slots == 4
 
 
+def test_fragmentation_and_need_count_every_group():
+    """One group keeps every key, one a window of 6: after 22 tokens in pages of 4 the first holds 6 pages
+    (24 slots, 22 used), the second 2 pages after giving 4 back (8 slots, 6 of them live keys 16..21)."""
+    m = CacheManager(group_layers([PagedCacheSpec(1, 16), PagedCacheSpec(1, 16, 6)]), num_blocks=16, block_size=4, max_seqs=2)
+    m.add_sequence("r")
+    m.append(["r"], [22])
+    assert m.release_passed(["r"]) == 4
+    assert [a.num_used for a in m.allocators.values()] == [6, 2]
+    assert abs(m.internal_fragmentation() - (1 - (22 + 6) / (24 + 8))) < 1e-9
+    assert m.extra_blocks_needed("r", 2) == 0 and m.extra_blocks_needed("r", 3) == 1 and m.extra_blocks_needed("r", 11) == 3
+    m.free_sequence("r")
+    assert m.internal_fragmentation() == 0.0
+
+
 def test_sequence_lengths_give_table_lengths():
     # N sequences of 1..30 tokens with pages of 4 (tests/test_paged.py:56-68)
     m = CacheManager(full_groups(), num_blocks=64, block_size=4, max_seqs=8)

@@ -31,7 +31,11 @@ def test_reads_every_key_it_is_given():
 def test_rope_theta_from_rope_parameters_and_head_dim_key():
     base = dict(vocab_size=10, hidden_size=64, intermediate_size=8, num_hidden_layers=1, num_attention_heads=4)
     assert LlamaConfig.from_dict(dict(base, rope_parameters={"rope_theta": 5e5})).rope_theta == 5e5
-    assert LlamaConfig.from_dict(dict(base, head_dim=32)).head_dim == 32
+    assert LlamaConfig.from_dict(dict(base, head_dim=16)).head_dim == 16  # the key may be there if it says the same
+    with pytest.raises(ConfigError, match="head_dim=32 differs"):
+        LlamaConfig.from_dict(dict(base, head_dim=32))  # the reference always derives hidden // heads
+    with pytest.raises(ConfigError, match="not a multiple of num_attention_heads"):
+        LlamaConfig.from_dict(dict(base, hidden_size=66))
 
 
 def test_missing_and_bad_values_are_named():
@@ -64,6 +68,24 @@ def test_presets_have_the_published_sizes():
     assert LlamaConfig.from_dict(preset("llama2-70b")).head_dim == 128
     with pytest.raises(ConfigError, match="unknown preset"):
         preset("nope")
+
+
+def test_presets_belong_to_the_architecture_that_registers_them():
+    """Named sizes come with an architecture's registration; nothing in the framework lists them by hand."""
+    from llmserve.config import is_preset, preset_names, register_architecture
+
+    assert {"tiny", "tinyllama-1.1b", "llama2-7b", "llama2-70b"} <= set(preset_names())
+    assert preset("TinyLlama_1.1B")["architectures"] == ["LlamaForCausalLM"] and preset("tiny")["model_type"] == "llama"
+    register_architecture("PresetProbeForCausalLM", LlamaConfig, lambda cfg: None, model_type="preset_probe",
+                          presets={"probe-small": dict(vocab_size=7, hidden_size=16)})
+    try:
+        assert is_preset("probe_small") and "probe-small" in preset_names()
+        got = preset("probe-small")
+        assert got == dict(vocab_size=7, hidden_size=16, architectures=["PresetProbeForCausalLM"], model_type="preset_probe")
+        assert architecture_of(got).name == "PresetProbeForCausalLM"
+    finally:
+        ARCHITECTURES.pop("PresetProbeForCausalLM")
+    assert not is_preset("probe-small")
 
 
 def test_registry_picks_the_model_by_config(tmp_path):

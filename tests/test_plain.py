@@ -137,6 +137,148 @@ def test_forward_is_causal_and_uses_the_tied_head(cfg):
     assert ("lm_head.weight" in w) == (not cfg["tie_word_embeddings"])
 
 
+# ------------------------------------------------------------------ the whole model, pinned without a second reading
+def library_forward(cfg, w, ids):
+    """The same model put together from the library's own routines only, batched and with complex numbers for
+    the rotation: embedding, rms_norm, linear, scaled_dot_product_attention, silu.  It shares the layer order
+    with the plain implementation (both follow src/llmserve/model/llama.py:131-135,171-185) and nothing else."""
+    nh = cfg["num_attention_heads"]
+    nkv = cfg.get("num_key_value_heads", nh)
+    hidden = cfg["hidden_size"]
+    d = hidden // nh
+    eps, theta = cfg["rms_norm_eps"], cfg["rope_theta"]
+    t = len(ids)
+    x = F.embedding(torch.tensor([ids]), w["model.embed_tokens.weight"])  # [1, T, H]
+    turn = torch.polar(torch.ones(t, d // 2, dtype=torch.float64),
+                       torch.arange(t, dtype=torch.float64)[:, None] * theta ** (-torch.arange(0, d, 2, dtype=torch.float64) / d))
+
+    def rotate(v):  # [1, heads, T, D]; dimension i is the real part, i + D/2 the imaginary part
+        z = torch.complex(v[..., : d // 2].double(), v[..., d // 2:].double()) * turn
+        return torch.cat([z.real, z.imag], dim=-1).float()
+
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        h = F.rms_norm(x, (hidden,), w[p + "input_layernorm.weight"], eps)
+        q = F.linear(h, w[p + "self_attn.q_proj.weight"]).view(1, t, nh, d).transpose(1, 2)
+        k = F.linear(h, w[p + "self_attn.k_proj.weight"]).view(1, t, nkv, d).transpose(1, 2)
+        v = F.linear(h, w[p + "self_attn.v_proj.weight"]).view(1, t, nkv, d).transpose(1, 2)
+        o = F.scaled_dot_product_attention(rotate(q), rotate(k), v, is_causal=True, enable_gqa=True)
+        x = x + F.linear(o.transpose(1, 2).reshape(1, t, hidden), w[p + "self_attn.o_proj.weight"])
+        h = F.rms_norm(x, (hidden,), w[p + "post_attention_layernorm.weight"], eps)
+        x = x + F.linear(F.silu(F.linear(h, w[p + "mlp.gate_proj.weight"])) * F.linear(h, w[p + "mlp.up_proj.weight"]),
+                         w[p + "mlp.down_proj.weight"])
+    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
+    return F.linear(F.rms_norm(x, (hidden,), w["model.norm.weight"], eps), head)[0]
+
+
+def _lively(w, seed=0):
+    """Norm weights well away from 1 and matrices large enough that every branch matters."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, t in w.items():
+        if name.endswith("norm.weight") or "layernorm" in name:
+            out[name] = 1 + 0.5 * torch.randn(t.shape, generator=g)
+        else:
+            out[name] = t * 4
+    return out
+
+
+@pytest.mark.parametrize("cfg", [TINY_A, TINY_B])
+def test_whole_model_from_library_routines(cfg):
+    """atol 1e-4, the bound of the reference's own whole-model test (tests/test_model.py:85-105 there, which
+    compares with an installed model class; no such class is used here)."""
+    w = _lively(_model(cfg, seed=4))
+    ids = torch.randint(0, cfg["vocab_size"], (23,), generator=torch.Generator().manual_seed(10)).tolist()
+    got, want = pl.forward(cfg, w, ids, torch.float32), library_forward(cfg, w, ids)
+    assert float(want.abs().max()) > 0.5
+    assert (got - want).abs().max() <= 1e-4
+
+
+def test_grouped_heads_read_the_kv_head_of_their_group():
+    """A grouped model equals the ungrouped model whose K and V projections repeat each KV head for its group:
+    query head h reads KV head h // group (a map like h % kv_heads fails here)."""
+    cfg = dict(TINY_A, num_hidden_layers=1)
+    w = _lively(_model(cfg, seed=5))
+    nh, nkv, d = 4, 2, 16
+    wide = dict(w)
+    for name in ("k_proj", "v_proj"):
+        key = f"model.layers.0.self_attn.{name}.weight"
+        wide[key] = w[key].view(nkv, d, 64).repeat_interleave(nh // nkv, dim=0).reshape(nh * d, 64)
+    ids = list(range(40, 57))
+    got = pl.forward(cfg, w, ids, torch.float32)
+    assert (got - pl.forward(dict(cfg, num_key_value_heads=nh), wide, ids, torch.float32)).abs().max() <= 1e-5
+    tiled = dict(w)
+    for name in ("k_proj", "v_proj"):
+        key = f"model.layers.0.self_attn.{name}.weight"
+        tiled[key] = w[key].view(nkv, d, 64).repeat(nh // nkv, 1, 1).reshape(nh * d, 64)
+    assert (got - pl.forward(dict(cfg, num_key_value_heads=nh), tiled, ids, torch.float32)).abs().max() > 1e-3
+
+
+def test_a_head_is_a_block_of_consecutive_rows():
+    """Swapping two whole heads (rows h*D..(h+1)*D-1 of q, k, v and the same columns of o_proj) changes nothing;
+    it would if heads were interleaved over the rows."""
+    cfg = dict(TINY_A, num_hidden_layers=1, num_key_value_heads=4)
+    w = _lively(_model(cfg, seed=6))
+    order = torch.cat([torch.arange(32, 48), torch.arange(16, 32), torch.arange(0, 16), torch.arange(48, 64)])
+    swapped = dict(w)
+    for name in ("q_proj", "k_proj", "v_proj"):
+        key = f"model.layers.0.self_attn.{name}.weight"
+        swapped[key] = w[key][order]
+    swapped["model.layers.0.self_attn.o_proj.weight"] = w["model.layers.0.self_attn.o_proj.weight"][:, order]
+    ids = list(range(7, 30))
+    assert (pl.forward(cfg, w, ids, torch.float32) - pl.forward(cfg, swapped, ids, torch.float32)).abs().max() <= 1e-5
+
+
+def test_both_norms_sit_in_front_of_their_branch():
+    """With a tiny eps a normed branch does not feel the scale of its input: layer(c x) - c x = layer(x) - x when
+    the other branch is shut (its output projection zero).  A norm after the branch, or none, fails this."""
+    cfg = TINY_B
+    w = _lively(_model(cfg, seed=7))
+    x = torch.randn(9, 96, generator=torch.Generator().manual_seed(11))
+    args = dict(n_heads=3, n_kv_heads=1, head_dim=32, theta=5e5, eps=1e-12)
+    for shut in ("mlp.down_proj.weight", "self_attn.o_proj.weight"):
+        w1 = dict(w)
+        w1["model.layers.0." + shut] = torch.zeros_like(w["model.layers.0." + shut])
+        branch = pl.decoder_layer(x, w1, "model.layers.0.", **args) - x
+        assert float(branch.abs().max()) > 1e-2
+        assert ((pl.decoder_layer(3 * x, w1, "model.layers.0.", **args) - 3 * x) - branch).abs().max() <= 1e-4
+    both = dict(w)
+    for shut in ("mlp.down_proj.weight", "self_attn.o_proj.weight"):
+        both["model.layers.0." + shut] = torch.zeros_like(w["model.layers.0." + shut])
+    assert torch.equal(pl.decoder_layer(x, both, "model.layers.0.", **args), x)  # the stream itself is never normed
+
+
+def test_the_second_branch_reads_the_stream_after_the_first():
+    cfg = TINY_B
+    w = _lively(_model(cfg, seed=8))
+    x = torch.randn(6, 96, generator=torch.Generator().manual_seed(12))
+    args = dict(n_heads=3, n_kv_heads=1, head_dim=32, theta=5e5, eps=1e-6)
+    p = "model.layers.1."
+    a = pl.attention_block(pl.rms_norm(x, w[p + "input_layernorm.weight"], 1e-6), w, p + "self_attn.", 3, 1, 32, 5e5)
+    mid = x + a
+    want = mid + pl.swiglu(pl.rms_norm(mid, w[p + "post_attention_layernorm.weight"], 1e-6), w, p + "mlp.")
+    assert (pl.decoder_layer(x, w, p, **args) - want).abs().max() <= 1e-6
+    parallel = mid + pl.swiglu(pl.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-6), w, p + "mlp.")
+    assert (want - parallel).abs().max() > 1e-3  # (the test can tell the two arrangements apart)
+
+
+@pytest.mark.parametrize("cfg", [TINY_A, TINY_B])
+def test_final_norm_sits_between_the_last_layer_and_the_head(cfg):
+    w = _lively(_model(cfg, seed=9))
+    ids = list(range(11, 25))
+    base = pl.forward(cfg, w, ids, torch.float32)
+    scaled = dict(w, **{"model.norm.weight": 2.5 * w["model.norm.weight"]})
+    assert (pl.forward(cfg, scaled, ids, torch.float32) - 2.5 * base).abs().max() <= 1e-4 * float(base.abs().max())
+    off = dict(w, **{"model.norm.weight": torch.zeros_like(w["model.norm.weight"])})
+    assert torch.equal(pl.forward(cfg, off, ids, torch.float32), torch.zeros_like(base))
+    # with every branch shut the logits are head(norm(embedding)): no layer norms the stream on its way
+    shut = {k: (torch.zeros_like(v) if k.endswith(("o_proj.weight", "down_proj.weight")) else v) for k, v in w.items()}
+    table = w["model.embed_tokens.weight"]
+    head = table if cfg["tie_word_embeddings"] else w["lm_head.weight"]
+    want = F.linear(F.rms_norm(table[torch.tensor(ids)], (cfg["hidden_size"],), w["model.norm.weight"], cfg["rms_norm_eps"]), head)
+    assert (pl.forward(cfg, shut, ids, torch.float32) - want).abs().max() <= 1e-5
+
+
 def test_forward_bfloat16_stays_near_float32():
     w = _model(TINY_A)
     ids = list(range(3, 40))

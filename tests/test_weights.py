@@ -44,6 +44,32 @@ def test_random_weights_are_seeded_per_tensor(tmp_path):
     assert abs(float(norm.mean()) - 1.0) < 0.01 and float(norm.std()) > 0
 
 
+def test_a_part_brings_its_own_initializer():
+    """A tensor that is neither a matrix nor a norm weight (a decay in (0.9, 1), say) is filled by a function
+    the part registers under a name, or hands over itself: the weights package is not edited."""
+    from llmserve.parts.spec import ParamInfo
+    from llmserve.weights import INITIALIZERS, random_tensors, register_initializer
+
+    @register_initializer("decay_probe")
+    def decay(shape, generator, device, options):
+        return 0.9 + 0.1 * torch.rand(shape, generator=generator, dtype=torch.float32, device=device)
+
+    try:
+        infos = {"a.decay": ParamInfo((5, 3), "decay_probe"),
+                 "a.taps": ParamInfo((4,), lambda shape, g, dev, opt: torch.arange(4.0) * opt["std"]),
+                 "a.proj": ParamInfo((3, 3))}
+        t = random_tensors(infos, 9, torch.float32, std=0.5)
+        assert (t["a.decay"] >= 0.9).all() and (t["a.decay"] < 1.0).all() and t["a.decay"].unique().numel() > 1
+        assert torch.equal(t["a.taps"], torch.tensor([0.0, 0.5, 1.0, 1.5]))
+        assert torch.equal(t["a.decay"], random_tensors(infos, 9, torch.float32)["a.decay"])  # seeded like the rest
+    finally:
+        INITIALIZERS.pop("decay_probe")
+    with pytest.raises(ValueError, match="no initializer named 'decay_probe'"):
+        random_tensors({"a.decay": ParamInfo((5, 3), "decay_probe")}, 9, torch.float32)
+    with pytest.raises(ValueError, match="made shape"):
+        random_tensors({"x": ParamInfo((2, 2), lambda shape, g, dev, opt: torch.zeros(3))}, 1, torch.float32)
+
+
 def test_tied_model_has_no_head_tensor_and_ignores_one(tmp_path):
     write_random_model(tmp_path, TINY_B, seed=1)
     model, infos = _infos(TINY_B)
