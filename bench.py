@@ -139,6 +139,71 @@ def serve(args) -> int:
     return 0
 
 
+def gemv(args) -> int:
+    """The decode step's matrix products one by one, as the step launches them (`ops.gemm_stream` with the
+    epilogue and the split of K the parts choose), at 1, 8 and 64 rows.  Every launch of a chain takes the next
+    of several copies of its weight, a gigabyte in all, so that nothing is left in the 256 MB memory-side cache
+    from the launch before (the convention of the reference's benchmarks/bench_decode_matmul.py:28,78-81); the
+    chain is captured as a graph, so the figure is device time per launch, start and drain included."""
+    import torch
+
+    from llmserve.config import preset
+    from llmserve.ops import library as ops
+    from llmserve.parts import linear as lin
+
+    cfg = preset(args.model)
+    h, inter, vocab = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    nh, nkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    d = h // nh
+    ops.ensure_built("bfloat16")
+    dev = torch.device("cuda:0")
+    shapes = {"qkv": ((nh + 2 * nkv) * d, h), "o_proj": (h, nh * d), "gate_up": (2 * inter, h), "down_proj": (h, inter),
+              "lm_head": (vocab, h)}
+    results = {}
+    for name, (n, k) in shapes.items():
+        copies = max(2, -(-(1 << 30) // (n * k * 2)))
+        weights = [torch.randn(n, k, device=dev, dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+        for m in (1, 8, 64):
+            x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+            if name == "gate_up":
+                out = torch.empty(m, inter, device=dev, dtype=torch.bfloat16)
+                if lin.few_rows(m, weights[0]):
+                    run = lambda w: ops.gemm_stream(out, x, w, swiglu=True)  # noqa: E731
+                else:
+                    wide = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+                    run = lambda w: ops.silu_mul(out, torch.mm(x, w.t(), out=wide))  # noqa: E731
+            elif name in ("o_proj", "down_proj"):
+                run = lambda w: lin.linear_partial_sums(x, w) or lin.linear(x, w)  # noqa: E731
+            else:
+                out_dtype = torch.float32 if name == "lm_head" else torch.bfloat16
+                run = lambda w: lin.linear(x, w, out_dtype=out_dtype)  # noqa: E731
+            for w in weights[:2]:
+                run(w)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for w in weights:
+                    run(w)
+            graph.replay()
+            torch.cuda.synchronize()
+            reps = max(1, 200 // copies)
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                graph.replay()
+            torch.cuda.synchronize()
+            us = (time.perf_counter() - t0) / (reps * copies) * 1e6
+            results[f"{name}_m{m}"] = {"us": round(us, 2), "GBps": round(n * k * 2 / us / 1e3, 1)}
+        del weights
+    line = {"metric": "decode matrix products alone: microseconds per launch, weights streamed from HBM",
+            "value": results["gate_up_m8"]["us"], "unit": "us", "n_gpus": 1, "steps": 0, "warmup": 0, "ms_per_step": 0.0,
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"model": args.model, "hidden": h, "intermediate": inter, "vocab": vocab, "heads": nh,
+                       "kv_heads": nkv, "head_dim": d, "parallelism": "single-gpu"},
+            "gemv": results}
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,8 +216,9 @@ def main() -> int:
     ap.add_argument("--model", default="tinyllama-1.1b")
     ap.add_argument("--no-points", action="store_true", help="skip the further batch sizes")
     ap.add_argument("--points", default="1,64", help="further batch sizes to measure decoding at")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill"], default="all",
-                    help="run one phase only (for profiles; the line then holds zeros for the other)")
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "gemv"], default="all",
+                    help="run one phase only (for profiles; the line then holds zeros for the other); gemv: the "
+                         "decode products alone, each over copies of its weight that do not fit the caches")
     ap.add_argument("--workload", choices=["steps", "serve"], default="steps")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
@@ -166,6 +232,8 @@ def main() -> int:
         return 2
     if args.workload == "serve":
         return serve(args)
+    if args.phase == "gemv":
+        return gemv(args)
 
     import torch
 

@@ -187,7 +187,8 @@ def test_gemm_bf16(kernel, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 16, 64), (3, 333, 96), (16, 2056, 2048), (7, 100, 5632), (9, 48, 176),
-                                   (17, 333, 96), (64, 2056, 2048), (40, 100, 5632), (33, 48, 176)])
+                                   (17, 333, 96), (64, 2056, 2048), (40, 100, 5632), (33, 48, 176),
+                                   (8, 1040, 8192), (3, 64, 28672)])  # (the last two: K of the Llama-2-70B layer)
 def test_gemm_stream_plain(m, n, k):
     x, w, b = rnd(m, k, seed=11).bfloat16(), rnd(n, k, seed=12).bfloat16(), rnd(n, seed=13).bfloat16()
     ref = x.double() @ w.double().t() + b.double()
@@ -196,7 +197,7 @@ def test_gemm_stream_plain(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k,splits", [(1, 16, 64, 2), (8, 2048, 2048, 2), (5, 2048, 5632, 4), (16, 100, 5632 + 96, 3),
-                                          (40, 320, 2048, 2), (3, 48, 1024, 16)])
+                                          (40, 320, 2048, 2), (3, 48, 1024, 16), (8, 512, 28672, 4)])
 def test_gemm_stream_k_split_over_workgroups(m, n, k, splits):
     """K shared out to several workgroups per tile: partial sums whose total is the product (a share may be
     empty when there are fewer chunks of 512 than splits); the bias is in the first."""
@@ -244,7 +245,8 @@ def test_gemm_slices(m, n, k):
         ops().gemm_slices(torch.empty(slices, 65, n, device=DEV), rnd(65, k).bfloat16().to(DEV), w.to(DEV))
 
 
-@pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96), (37, 5632, 2048), (64, 256, 1024)])
+@pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96), (37, 5632, 2048), (64, 256, 1024),
+                                       (8, 1792, 8192)])
 def test_gemm_stream_gated_epilogue(m, inter, k):
     """gate and up of the feed-forward in one product over [gate; up], silu(gate) * up in the epilogue:
     the same bits as the product followed by the activation kernel."""
@@ -528,6 +530,8 @@ MFMA_CASES = [  # nh, nkv, d, bs, lens, new, window
     (4, 4, 128, 32, [257, 31], [1, 31], 0),
     (2, 1, 256, 16, [90], [7], 0),
     (32, 4, 64, 16, [600, 31], [1, 1], 0),
+    (64, 8, 128, 16, [300, 64, 129], [1, 24, 2], 0),  # 8 heads per KV head at head_dim 128: the Llama-2-70B layer
+    (64, 8, 128, 16, [700, 33], [1, 1], 0),
     (32, 1, 32, 8, [45], [3], 0),
     (5, 1, 48, 8, [77], [20], 0),
     (12, 1, 16, 24, [50], [50], 0),

@@ -177,6 +177,7 @@ def test_padding_of_steps_is_bounded():
 WIDE = {  # layer sizes of real models, few layers
     "tinyllama-1.1b": dict(num_hidden_layers=2),               # hidden 2048, 32 heads on 4 KV heads of 64, 5632, 32000
     "llama2-7b": dict(num_hidden_layers=1, vocab_size=4000),   # hidden 4096, 32 heads of 128, 11008 (no multiple of 512)
+    "llama2-70b": dict(num_hidden_layers=1, vocab_size=2000),  # hidden 8192, 64 heads on 8 KV heads of 128, 28672
 }
 
 
