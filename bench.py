@@ -204,6 +204,36 @@ def gemv(args) -> int:
     return 0
 
 
+def sync_costs(args) -> int:
+    """What the two ways of ordering dependent work on the GPU cost (csrc/probe.hip): a kernel boundary in a
+    captured chain of launches, and a barrier over all workgroups inside one kernel, without and with the fences
+    that make stores visible across XCDs.  The decode step is a chain of kernels because of these figures."""
+    import ctypes
+
+    import torch
+
+    from llmserve.ops import library as ops
+
+    lib = ops.load("probe")
+    scratch = torch.zeros(1024 * 256 + 16, dtype=torch.float32, device="cuda:0")
+    results = (ctypes.c_float * 12)()
+    torch.cuda.synchronize()
+    status = lib.llms_probe_sync(results, ctypes.c_void_p(scratch.data_ptr()))
+    if status != 0:
+        print(f"the probe failed with status {status}")
+        return 1
+    r = [round(float(v), 2) for v in results]
+    line = {"metric": "microseconds per kernel boundary in a captured chain of launches", "value": r[1], "unit": "us",
+            "n_gpus": 1, "steps": 0, "warmup": 0, "ms_per_step": 0.0, "higher_is_better": False, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"parallelism": "single-gpu"},
+            "kernel_boundary_us": {"8_workgroups": r[0], "256_workgroups": r[1], "1024_workgroups": r[2]},
+            "grid_barrier_us": {"64": r[3], "256": r[4], "512": r[5], "1024": r[6]},
+            "grid_barrier_with_fences_us": {"64": r[7], "256": r[8], "512": r[9]},
+            "spin_limits_hit": r[10], "stale_reads": r[11]}
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -216,9 +246,10 @@ def main() -> int:
     ap.add_argument("--model", default="tinyllama-1.1b")
     ap.add_argument("--no-points", action="store_true", help="skip the further batch sizes")
     ap.add_argument("--points", default="1,64", help="further batch sizes to measure decoding at")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill", "gemv"], default="all",
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "gemv", "sync"], default="all",
                     help="run one phase only (for profiles; the line then holds zeros for the other); gemv: the "
-                         "decode products alone, each over copies of its weight that do not fit the caches")
+                         "decode products alone, each over copies of its weight that do not fit the caches; sync: what a kernel "
+                         "boundary and a barrier inside a kernel cost")
     ap.add_argument("--workload", choices=["steps", "serve"], default="steps")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
@@ -234,6 +265,8 @@ def main() -> int:
         return serve(args)
     if args.phase == "gemv":
         return gemv(args)
+    if args.phase == "sync":
+        return sync_costs(args)
 
     import torch
 

@@ -15,11 +15,6 @@
 // batch 8 went from 3.98 to 3.73 ms.  A launch of at most a workgroup per CU keeps the chunks of 512.
 //
 // Because a launch costs more than most of these products take, what surrounds the product is fused in:
-//   NORM      prologue: x = bf16(residual + delta) (written to resid_out by workgroup 0), then
-//             h = weight_n * bf16(x * rsqrt(mean(x^2) + eps)): the RMSNorm kernel's rounding points
-//             (src/llmserve/model/llama.py:24-28).  Every workgroup does this for all rows itself, a wave per
-//             pair of rows with coalesced loads, while its first weights are in flight; the normed rows
-//             wait in LDS (dynamic, rows x (K/8 + 1) chunks) for the matrix instructions.
 //   SWIGLU    the 16 rows are 8 gate rows and the 8 up rows of the same features; the epilogue writes
 //             bf16(bf16(silu(bf16(gate))) * bf16(up)) (src/llmserve/model/llama.py:120).
 //   ROPE_QKV  the 16 rows are 8 rows of one head and their 8 rotary partners (i, i + D/2); the epilogue
@@ -64,11 +59,6 @@ struct StreamArgs {
     int M, N, K;
     int num_tiles;  // tiles of 16 weight rows (8 features for the gated and rotary epilogues)
     int k_splits;   // workgroups that share a tile's K (blockIdx.y); each stores its partial sums, 32-bit, in C[split]
-    // NORM
-    const bf16* delta;
-    const bf16* norm_w;
-    float eps;
-    bf16* resid_out;
     // SWIGLU
     int inter;
     // ROPE_QKV
@@ -97,7 +87,7 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-template <typename TOut, int EPI, bool NORM, int ST_KC>  // ST_KC: width of a chunk of K, 128 or 512
+template <typename TOut, int EPI, int ST_KC>  // ST_KC: width of a chunk of K, 128 or 512
 __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const StreamArgs a) {
     __shared__ uint4 lds[ST_WAVES * 16 * (ST_KC / 8)];  // per wave 16 rows x ST_KC / 8 pieces of 16 bytes
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
@@ -154,7 +144,7 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
             wreg[i] = (n >= 0 && kl < K) ? load_streaming(a.W + (size_t)n * K + kl) : zero;
         }
     };
-    if (c_begin + wave < chunks) load_weights(c_begin + wave);  // in flight while the row statistics are computed
+    if (c_begin + wave < chunks) load_weights(c_begin + wave);
 
     const bool m_ok = m0 + r16 < M;
     const bf16* xrow = a.X + (size_t)(m_ok ? m0 + r16 : 0) * a.ldx;
@@ -173,68 +163,6 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
         if (a.slots && m16 < M) epi_slot_v = a.slots[m16];
     }
 
-    // ---- NORM: summed residual, statistics and normed rows, kept in LDS as h[row][K/8 + 1] chunks of 8
-    extern __shared__ uint4 h_lds[];
-    const int hstride = K / 8 + 1;  // (one chunk of padding: the 16 rows of a matrix operand fall into different banks)
-    if (NORM) {
-        // a wave takes the rows wave, wave + 4, ..., two at a time so that their loads are in flight together;
-        // a lane norms the chunks it summed itself, so nothing but the end needs a barrier
-        for (int ma = wave; ma < M; ma += 2 * ST_WAVES) {
-            const int rows[2] = {ma, ma + ST_WAVES};
-            const int nrows = rows[1] < M ? 2 : 1;
-            float ss[2] = {0.f, 0.f};
-#pragma unroll 4
-            for (int c8 = lane; c8 < K / 8; c8 += LLMS_WAVE) {
-                uint4 v[2], d[2];
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    if (j < nrows) {
-                        v[j] = *reinterpret_cast<const uint4*>(a.X + (size_t)rows[j] * a.ldx + 8 * c8);
-                        if (a.delta) d[j] = *reinterpret_cast<const uint4*>(a.delta + (size_t)rows[j] * a.ldx + 8 * c8);
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    if (j < nrows) {
-                        float xf[8];
-                        unpack8(v[j], xf);
-                        if (a.delta) {  // the residual sum in 32-bit, rounded once
-                            float df[8];
-                            unpack8(d[j], df);
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) xf[e] = bfr(xf[e] + df[e]);
-                            v[j] = pack8(xf);
-                            if (a.resid_out && tile_id == 0)
-                                *reinterpret_cast<uint4*>(a.resid_out + (size_t)rows[j] * a.ldx + 8 * c8) = v[j];
-                        }
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) ss[j] += xf[e] * xf[e];
-                        h_lds[rows[j] * hstride + c8] = v[j];
-                    }
-                }
-            }
-            float inv_rms[2];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) inv_rms[j] = rsqrtf(wave_sum(ss[j]) / (float)K + a.eps);
-#pragma unroll 2
-            for (int c8 = lane; c8 < K / 8; c8 += LLMS_WAVE) {
-                float wf[8];
-                unpack8(*reinterpret_cast<const uint4*>(a.norm_w + 8 * c8), wf);
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    if (j < nrows) {
-                        float xf[8];
-                        unpack8(h_lds[rows[j] * hstride + c8], xf);
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) xf[e] = wf[e] * bfr(xf[e] * inv_rms[j]);
-                        h_lds[rows[j] * hstride + c8] = pack8(xf);
-                    }
-                }
-            }
-        }
-        __syncthreads();  // the normed rows are complete
-    }
-
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
     for (int c = c_begin + wave; c < chunks; c += ST_WAVES) {
         const int k0 = c * ST_KC;
@@ -242,8 +170,10 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_stream_kernel(const 
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
             const int k = k0 + 32 * s + 8 * g;
+            // (a branch, not a select: written as `cond ? load : zero` the load is issued for every lane, also for
+            // the rows that do not exist, and the step at batch 8 takes 1.35 instead of 1.05 ms)
             if (m_ok && k < K)
-                xreg[s] = NORM ? h_lds[r16 * hstride + k / 8] : *reinterpret_cast<const uint4*>(xrow + k);
+                xreg[s] = *reinterpret_cast<const uint4*>(xrow + k);
             else
                 xreg[s] = zero;
         }
@@ -407,69 +337,40 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_slices_kernel(const 
     }
 }
 
-#define ST_NORM_LDS_MAX (96 * 1024)  // beside the 64 KB of weight tiles, of the 160 KB a workgroup may hold
-
 // A launch with a workgroup or less per CU gets chunks of 512 (16 KB in flight per wave: all a lone workgroup can
 // do for its CU), a larger one chunks of 128 (eight workgroups per CU, no rounds).
 #define ST_FEW_WORKGROUPS 256
 
-template <typename TOut, int EPI, int KC>
-static int launch_stream_kc(bool norm, dim3 grid, const StreamArgs& a, hipStream_t stream) {
-    if (norm) {
-        static bool raised = false;  // (per instantiation) allow more dynamic LDS than the default limit
-        if (!raised) {
-            LLMS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<TOut, EPI, true, KC>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, ST_NORM_LDS_MAX));
-            raised = true;
-        }
-        const size_t h_bytes = (size_t)a.M * (a.K / 8 + 1) * 16;
-        gemm_stream_kernel<TOut, EPI, true, KC><<<grid, ST_WAVES * LLMS_WAVE, h_bytes, stream>>>(a);
-    } else {
-        gemm_stream_kernel<TOut, EPI, false, KC><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(a);
-    }
-    return LLMS_OK;
-}
-
 template <typename TOut, int EPI>
-static int launch_stream(bool norm, unsigned tiles, const StreamArgs& a, hipStream_t stream) {
+static void launch_stream(unsigned tiles, const StreamArgs& a, hipStream_t stream) {
     const dim3 grid(tiles, a.k_splits);
-    if ((long long)tiles * a.k_splits <= ST_FEW_WORKGROUPS) return launch_stream_kc<TOut, EPI, 512>(norm, grid, a, stream);
-    return launch_stream_kc<TOut, EPI, 128>(norm, grid, a, stream);
+    if ((long long)tiles * a.k_splits <= ST_FEW_WORKGROUPS)
+        gemm_stream_kernel<TOut, EPI, 512><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(a);
+    else
+        gemm_stream_kernel<TOut, EPI, 128><<<grid, ST_WAVES * LLMS_WAVE, 0, stream>>>(a);
 }
 
 extern "C" {
 
 // epilogue: 0 plain (C [M,N] + bias), 1 gated (W = [gate; up] of `inter` rows each, C [M, inter]),
 // 2 rotary q/k/v (W = [q; k; v], C = q [M, n_heads*head_dim], k and v stored at `slots` when given).
-// norm_w != null: X is the residual stream, `delta` (nullable) is added to it, the sum goes to resid_out
-// (nullable) and its RMSNorm with norm_w and eps is what is multiplied.  out_dtype: 0 float32, 1 bfloat16.
+// out_dtype: 0 float32, 1 bfloat16.
 // k_splits > 1 (plain epilogue, float32): K is shared out to k_splits workgroups per tile, a short wide matrix
 // then fills the chip; C is [k_splits][M][ldc], partial sums that the caller adds up (bias in the first).
 int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* X, int ldx, const void* W,
-                     const void* bias, int M, int N, int K, const void* delta, const void* norm_w, float eps,
-                     void* resid_out, int inter, int n_heads, int n_kv_heads, int head_dim, int block_size,
-                     const float* inv_freq, const int* positions, const int* slots, void* k_pool, void* v_pool,
-                     int k_splits, hipStream_t stream) {
+                     const void* bias, int M, int N, int K, int inter, int n_heads, int n_kv_heads, int head_dim,
+                     int block_size, const float* inv_freq, const int* positions, const int* slots, void* k_pool,
+                     void* v_pool, int k_splits, hipStream_t stream) {
     LLMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_stream: needs 1 <= M <= 64 and positive sizes");
-    LLMS_REQUIRE(norm_w == nullptr || (M <= 16 && (size_t)M * (K / 8 + 1) * 16 <= ST_NORM_LDS_MAX),
-                 "gemm_stream: the norm prologue takes at most 16 rows and rows * (K + 8) * 2 bytes up to 96 KB");
     LLMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "gemm_stream: K and the row stride of X must be multiples of 8");
     LLMS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_stream: X and W must be 16-byte aligned");
     LLMS_REQUIRE(C != nullptr && (out_dtype == 0 || out_dtype == 1), "gemm_stream: bad output");
     LLMS_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_stream: epilogue must be 0, 1 or 2");
-    if (norm_w) {
-        LLMS_REQUIRE(((uintptr_t)norm_w % 16) == 0 && (!delta || ((uintptr_t)delta % 16) == 0) &&
-                         (!resid_out || ((uintptr_t)resid_out % 16) == 0), "gemm_stream: norm operands must be 16-byte aligned");
-        LLMS_REQUIRE(resid_out != X, "gemm_stream: the summed residual needs a buffer of its own");
-    } else {
-        LLMS_REQUIRE(!delta && !resid_out, "gemm_stream: delta and resid_out need norm_w");
-    }
     LLMS_REQUIRE(k_splits >= 1 && k_splits <= 16, "gemm_stream: k_splits must be in 1..16");
-    LLMS_REQUIRE(k_splits == 1 || (epilogue == EPI_PLAIN && out_dtype == 0 && norm_w == nullptr),
+    LLMS_REQUIRE(k_splits == 1 || (epilogue == EPI_PLAIN && out_dtype == 0),
                  "gemm_stream: K is split for plain 32-bit partial sums only");
-    StreamArgs a = {C, ldc, (const bf16*)X, ldx, (const bf16*)W, (const bf16*)bias, M, N, K, 0, k_splits, (const bf16*)delta,
-                    (const bf16*)norm_w, eps, (bf16*)resid_out, inter, n_heads, n_kv_heads, head_dim, block_size,
-                    inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool};
+    StreamArgs a = {C, ldc, (const bf16*)X, ldx, (const bf16*)W, (const bf16*)bias, M, N, K, 0, k_splits, inter, n_heads,
+                    n_kv_heads, head_dim, block_size, inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool};
     unsigned grid;
     if (epilogue == EPI_PLAIN) {
         LLMS_REQUIRE(ldc >= N, "gemm_stream: ldc too small");
@@ -488,11 +389,9 @@ int llms_gemm_stream(int out_dtype, int epilogue, void* C, int ldc, const void* 
     }
     a.num_tiles = (int)grid;
     grid = ((grid + 7) / 8) * 8 * ((M + 15) / 16);  // every XCD gets whole tiles with all their row blocks
-    const bool norm = norm_w != nullptr;
-#define ST_EPI(E)                                                                                  \
-    if (int e = out_dtype == 0 ? launch_stream<float, E>(norm, grid, a, stream)                    \
-                               : launch_stream<bf16, E>(norm, grid, a, stream))                    \
-        return e;
+#define ST_EPI(E)                                                   \
+    if (out_dtype == 0) launch_stream<float, E>(grid, a, stream);   \
+    else launch_stream<bf16, E>(grid, a, stream);
     if (epilogue == EPI_PLAIN) { ST_EPI(EPI_PLAIN) }
     else if (epilogue == EPI_SWIGLU) { ST_EPI(EPI_SWIGLU) }
     else { ST_EPI(EPI_ROPE_QKV) }

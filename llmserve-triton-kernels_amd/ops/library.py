@@ -309,19 +309,11 @@ def gemm_bf16(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: torch.T
     return out
 
 
-STREAM_NORM_ROWS = 16  # what gemm_stream's norm prologue takes: rows, and bytes of LDS for them
-STREAM_NORM_LDS_BYTES = 96 * 1024
-
-
 def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, *,
-                norm: tuple | None = None, swiglu: bool = False, rope: dict | None = None,
-                k_splits: int = 1) -> torch.Tensor:
+                swiglu: bool = False, rope: dict | None = None, k_splits: int = 1) -> torch.Tensor:
     """The product for up to 64 bfloat16 rows (built for up to 16), with what surrounds it fused in.
 
     plain:   out[M, N] = x w^T (+ bias).
-    norm = (delta | None, norm_weight, eps, resid_out | None): x is the residual stream; delta is added
-             to it (32-bit sum, rounded once), the sum is written to resid_out, and the product runs on the
-             RMSNorm of the sum.
     swiglu:  w = [gate; up] ([2I, K]); out[M, I] = silu(gate) * up.
     rope = dict(n_heads, n_kv_heads, head_dim, inv_freq | None, positions, slots | None, k_pool, v_pool,
              block_size): w = [q; k; v]; out[M, n_heads * head_dim] = rotated q; rotated k and v are stored at
@@ -330,7 +322,7 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
              matrix then fills the chip); their sum in order is the product, the bias is in the first."""
     dev = _dev(out, x, w, bias)
     if k_splits != 1:
-        if not 1 < k_splits <= 16 or norm is not None or swiglu or rope is not None:
+        if not 1 < k_splits <= 16 or swiglu or rope is not None:
             raise ValueError("k_splits is 1..16 and goes with the plain epilogue only")
         if out.dim() != 3 or out.shape[0] != k_splits or out.dtype != torch.float32 or not out.is_contiguous():
             raise ValueError("with k_splits the output is a contiguous float32 [k_splits, M, N] tensor")
@@ -342,8 +334,6 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
     n = w.shape[0]
     if not 0 < m <= 64:
         raise ValueError("gemm_stream takes 1..64 rows")
-    if norm is not None and (m > STREAM_NORM_ROWS or m * (k // 8 + 1) * 16 > STREAM_NORM_LDS_BYTES):
-        raise ValueError("the norm prologue takes at most 16 rows, and rows * (K + 8) * 2 bytes up to 96 KB")
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or out.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("gemm_stream takes bfloat16 operands and stores bfloat16 or float32")
     if not gemm_bf16_supported(x, w):
@@ -353,18 +343,6 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
         raise ValueError("bias must be a contiguous bfloat16 vector of N elements")
     if swiglu and rope is not None:
         raise ValueError("one epilogue at a time")
-    delta = norm_w = resid_out = None
-    eps = 0.0
-    if norm is not None:
-        delta, norm_w, eps, resid_out = norm
-        for name, t in (("delta", delta), ("resid_out", resid_out)):
-            if t is not None and (t.shape != x.shape or t.dtype != x.dtype or t.stride() != x.stride()):
-                raise ValueError(f"{name} must match x in shape, dtype and strides")
-        if resid_out is not None and resid_out.data_ptr() == x.data_ptr():
-            raise ValueError("the summed residual needs a buffer of its own")
-        if norm_w.dtype != torch.bfloat16 or norm_w.numel() != k or not norm_w.is_contiguous():
-            raise ValueError(f"norm weight must be a contiguous bfloat16 vector of {k} elements")
-        _dev(delta, norm_w, resid_out, x)
     epilogue, inter, cols = 0, 0, n
     r = dict(n_heads=0, n_kv_heads=0, head_dim=0, block_size=0, inv_freq=None, positions=None, slots=None,
              k_pool=None, v_pool=None)
@@ -393,8 +371,7 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
         raise ValueError(f"out shape {tuple(out.shape)} is not {(m, cols)}")
     _check(load("gemm_stream").llms_gemm_stream(
         c_int(_code(out)), c_int(epilogue), _ptr(out), c_int(out.stride(0)), _ptr(x), c_int(x.stride(0)), _ptr(w),
-        _ptr(bias), c_int(m), c_int(n), c_int(k), _ptr(delta), _ptr(norm_w), c_float(eps), _ptr(resid_out),
-        c_int(inter), c_int(r["n_heads"]), c_int(r["n_kv_heads"]), c_int(r["head_dim"]), c_int(r["block_size"]),
+        _ptr(bias), c_int(m), c_int(n), c_int(k), c_int(inter), c_int(r["n_heads"]), c_int(r["n_kv_heads"]), c_int(r["head_dim"]), c_int(r["block_size"]),
         _ptr(r["inv_freq"]), _ptr(r["positions"]), _ptr(r["slots"]), _ptr(r["k_pool"]), _ptr(r["v_pool"]),
         c_int(k_splits), _stream(dev)), "gemm_stream")
     return parts if k_splits != 1 else out

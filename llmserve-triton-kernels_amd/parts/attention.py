@@ -16,9 +16,8 @@ import math
 import torch
 
 from ..ops import library as ops
-from .linear import few_rows, linear, linear_partial_sums, norm_fusable
-from .registry import POSITION_ENCODINGS, DeferredNorm, Mixer, as_tensor, register_mixer
-from .rmsnorm import RMSNorm
+from .linear import few_rows, linear, linear_partial_sums
+from .registry import POSITION_ENCODINGS, DeferredNorm, Mixer, register_mixer
 from .spec import PagedCacheSpec, ParamInfo
 
 
@@ -94,9 +93,8 @@ class Attention(Mixer):
                 or not ops.gemm_bf16_supported(rows, self.qkv_weight))
 
     def project_few_rows(self, x, batch, cache, slots):
-        """With few bfloat16 rows one kernel does the projection, the rotation and the cache store (and,
-        if switched on, the residual sum and the norm before them): ops.gemm_stream.  Returns the rotated
-        queries, or None when that kernel does not apply."""
+        """With few bfloat16 rows one kernel does the projection, the rotation and the cache store:
+        ops.gemm_stream.  Returns the rotated queries, or None when that kernel does not apply."""
         deferred = isinstance(x, DeferredNorm)
         rows = x.residual if deferred else x
         m = rows.shape[0]
@@ -105,19 +103,13 @@ class Attention(Mixer):
         frequencies = getattr(self.position, "rotary_frequencies", None)
         if frequencies is None and not getattr(self.position, "identity", False):
             return None  # a position encoding this kernel does not know
-        if deferred and not (norm_fusable(*rows.shape) and isinstance(x.norm, RMSNorm)):
-            x, rows, deferred = None, x.materialize(), False  # the norm by its own kernel, the rest fused
+        if deferred:
+            rows = x.materialize()  # the residual sum and the norm by the norm's own kernel, the rest fused
         rope = dict(n_heads=self.num_heads, n_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                     inv_freq=frequencies() if frequencies is not None else None, positions=batch.positions,
                     slots=slots, k_pool=cache.k_pool, v_pool=cache.v_pool, block_size=cache.block_size)
         q = torch.empty((m, self.num_heads * self.head_dim), dtype=rows.dtype, device=rows.device)
-        if deferred:
-            new_residual = torch.empty_like(rows) if x.delta is not None else None
-            ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias,
-                            norm=(as_tensor(x.delta), x.norm.weight, x.norm.eps, new_residual), rope=rope)
-            x.resolve(new_residual)
-        else:
-            ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias, rope=rope)
+        ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias, rope=rope)
         return q
 
     def attend(self, out, qkv, cache, view, batch):

@@ -42,19 +42,6 @@ def few_rows(m: int, weight: torch.Tensor) -> bool:
         return m > 0
     return m <= STREAM_MAX_ROWS and -(-m // 16) * weight.numel() * 2 <= STREAM_REREAD_BYTES
 
-# Whether the few-row product also does the residual sum and the norm in front of it
-# (ops.gemm_stream(norm=...)): every workgroup norms the rows itself while its first weights are in
-# flight.  Off by default: it saves the norm kernel, but the rows in LDS leave room for one workgroup
-# per CU instead of two, and the prologue is repeated by hundreds of workgroups.  Measured on the
-# TinyLlama shape: 864 against 898 tokens a second at batch 1, 5,310 against 6,302 at batch 8.
-FUSE_NORM_INTO_PRODUCT = os.environ.get("LLMSERVE_FUSE_NORM", "0") == "1"
-
-
-def norm_fusable(m: int, k: int) -> bool:
-    """Whether ops.gemm_stream's norm prologue takes m rows of k elements (they wait in LDS)."""
-    return FUSE_NORM_INTO_PRODUCT and 0 < m <= ops.STREAM_NORM_ROWS and m * (k // 8 + 1) * 16 <= ops.STREAM_NORM_LDS_BYTES
-
-
 # A short, wide weight gives the streaming kernel fewer tiles than the chip has CUs (TinyLlama's o_proj and
 # down_proj: 128), and long rows make each workgroup wait for several rounds of loads.  Sharing K out to
 # several workgroups per tile fills the chip: measured 4.3 -> 3.2 microseconds of reading for 2048 x 2048 and

@@ -1,18 +1,16 @@
 """Gated feed-forward: down(silu(gate(x)) * up(x)), no biases
 (src/llmserve/model/llama.py:112-120).  Parameters: hidden, intermediate.
 gate_proj and up_proj are stacked into one [2I, H] matrix at load, so one product feeds
-the activation.  With few bfloat16 rows that product also does the residual sum and the
-norm before it and the activation after it (ops.gemm_stream); otherwise the norm, the
-product and the activation are kernels of their own."""
+the activation.  With few bfloat16 rows that product also does the activation after it
+(ops.gemm_stream); otherwise the product and the activation are kernels of their own."""
 
 from __future__ import annotations
 
 import torch
 
 from ..ops import library as ops
-from .linear import few_rows, linear, linear_partial_sums, norm_fusable
-from .registry import DeferredNorm, FeedForward, as_tensor, register_feed_forward
-from .rmsnorm import RMSNorm
+from .linear import few_rows, linear, linear_partial_sums
+from .registry import DeferredNorm, FeedForward, register_feed_forward
 from .spec import ParamInfo
 
 
@@ -44,14 +42,6 @@ class SwiGLU(FeedForward):
         few = dtype == torch.bfloat16 and few_rows(m, self.gate_up) and self.intermediate % 8 == 0
         to_a_norm = isinstance(x, DeferredNorm)  # the caller hands the result to a norm, which takes partial sums
         if isinstance(x, DeferredNorm):
-            norm = x.norm
-            if (few and norm_fusable(m, x.residual.shape[1]) and isinstance(norm, RMSNorm)
-                    and ops.gemm_bf16_supported(x.residual, self.gate_up)):
-                new_residual = torch.empty_like(x.residual) if x.delta is not None else None
-                ops.gemm_stream(act, x.residual, self.gate_up,
-                                norm=(as_tensor(x.delta), norm.weight, norm.eps, new_residual), swiglu=True)
-                x.resolve(new_residual)
-                return self._down(act, to_a_norm)
             x = x.materialize()
         if few and ops.gemm_bf16_supported(x, self.gate_up):
             ops.gemm_stream(act, x, self.gate_up, swiglu=True)  # activation in the product's epilogue

@@ -261,37 +261,6 @@ def test_gemm_stream_gated_epilogue(m, inter, k):
     assert torch.equal(act, out)
 
 
-@pytest.mark.parametrize("m,n,k,eps", [(1, 64, 64, 1e-5), (6, 320, 2048, 1e-6), (16, 100, 2048 + 96, 1e-5),
-                                       (11, 48, 4096 + 96, 1e-5), (3, 40, 8192 + 8, 1e-6)])
-@pytest.mark.parametrize("with_delta", [False, True])
-def test_gemm_stream_norm_prologue(m, n, k, eps, with_delta):
-    """Residual sum and RMSNorm inside the product: the same bits of the summed residual as the norm
-    kernel writes, and a product that agrees with norm kernel + product."""
-    resid, delta = rnd(m, k, seed=19, scale=2.0).bfloat16(), rnd(m, k, seed=20).bfloat16()
-    wn, w = (1 + 0.1 * rnd(k, seed=21)).bfloat16(), rnd(n, k, seed=22).bfloat16()
-    summed = (resid.float() + delta.float()).bfloat16() if with_delta else resid
-    ref = plain_llama.rms_norm(summed, wn, eps).double() @ w.double().t()
-    new_resid = torch.full((m, k), 7.0, dtype=torch.bfloat16, device=DEV) if with_delta else None
-    out = ops().gemm_stream(torch.empty(m, n, device=DEV), resid.to(DEV), w.to(DEV),
-                            norm=(delta.to(DEV) if with_delta else None, wn.to(DEV), eps, new_resid))
-    # the statistics are summed in another order than on the CPU, so a normed element may round the other way
-    assert (out.cpu().double() - ref).abs().max() <= 2.0 ** -8 * float(ref.abs().max())
-    if with_delta:
-        assert torch.equal(new_resid.cpu(), summed)
-    with pytest.raises(ValueError, match="buffer of its own"):
-        r = resid.to(DEV)
-        ops().gemm_stream(torch.empty(m, n, device=DEV), r, w.to(DEV), norm=(delta.to(DEV), wn.to(DEV), eps, r))
-
-
-def test_gemm_stream_norm_prologue_refuses_rows_that_do_not_fit():
-    """The normed rows wait in LDS: 16 rows of 4,192 elements are more than it holds."""
-    x, w, wn = rnd(16, 4192, seed=1).bfloat16().to(DEV), rnd(32, 4192, seed=2).bfloat16().to(DEV), rnd(4192, seed=3).bfloat16().to(DEV)
-    with pytest.raises(ValueError, match="96 KB"):
-        ops().gemm_stream(torch.empty(16, 32, device=DEV), x, w, norm=(None, wn, 1e-5, None))
-    with pytest.raises(ValueError, match="at most 16 rows"):
-        ops().gemm_stream(torch.empty(17, 32, device=DEV), x.new_zeros(17, 64), w[:, :64].contiguous(), norm=(None, wn[:64].contiguous(), 1e-5, None))
-
-
 @pytest.mark.parametrize("nh,nkv,d,bs,theta,bias,m", [(4, 2, 16, 16, 1e4, False, 5), (3, 1, 32, 8, 5e5, True, 5),
                                                       (8, 2, 64, 16, 1e4, False, 64), (2, 2, 48, 8, None, True, 33)])
 def test_gemm_stream_rotary_epilogue(nh, nkv, d, bs, theta, bias, m):
