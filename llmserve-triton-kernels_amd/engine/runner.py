@@ -76,6 +76,11 @@ class ModelRunner:
         # rows the steps were asked to run, and rows they ran with the padding of buckets and graphs
         self.rows_asked = 0
         self.rows_run = 0
+        # matrix elements a token meets on its way through the layers: what a step's device time goes by
+        infos = model.param_infos()
+        outer = tuple(model.spec.weights[role] for role in ("embedding", "head"))
+        self._elements_per_token = sum(info.shape[0] * info.shape[1] for name, info in infos.items()
+                                       if len(info.shape) == 2 and not name.startswith(outer))
 
     # ---- construction ---------------------------------------------------------------------
     @staticmethod
@@ -188,8 +193,13 @@ class ModelRunner:
         elif all(len(e.tokens) == 1 for e in ordered):
             logits = self._replay_decode(layout, [e.tokens[0] for e in ordered], logit_rows, device_tokens)
             owned = False
-        else:
+        elif self._launch_bound(sum(layout.counts)):
             logits, owned = self._run_bucketed_step(layout, [e.tokens for e in ordered], logit_rows)
+        else:  # the device is busy for longer than the host needs to launch the step: nothing to gain from a graph
+            batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
+            logits = self.model.forward(batch, self.storage)
+            self.rows_run += sum(layout.counts)
+            self.rows_asked += sum(layout.counts)
         self.manager.release_passed(layout.seq_ids)
         return logits if owned or borrow else logits.clone()
 
@@ -225,6 +235,15 @@ class ModelRunner:
     # ---- steps with portions of prompts: padded to a bucket of sizes, replayed from the second time on ------
     MAX_STEP_GRAPHS = 32
     CAPTURE_AT_USE = 2  # a bucket is captured as a graph when it comes for this many-th time
+    # A step is worth a graph while launching its kernels one by one (about 20 microseconds each, some two hundred
+    # for a model of 22 layers) takes the host longer than the device needs to run them.  Per layer the host's time
+    # is fixed and the device's goes by rows times matrix elements; up to this product (a step of 1,100 rows of the
+    # 1.1B shape, of 250 rows of the 7B shape) the host is the limit.  A rule by sizes alone: the same step always
+    # takes the same path.
+    LAUNCH_BOUND_WORK_PER_LAYER = 5.0e10
+
+    def _launch_bound(self, rows: int) -> bool:
+        return rows * self._elements_per_token <= self.LAUNCH_BOUND_WORK_PER_LAYER * len(self.model.spec.schedule)
 
     @staticmethod
     def _row_bucket(n: int) -> int:
