@@ -110,7 +110,8 @@ def serve(args) -> int:
         torch.cuda.synchronize()
         return eng, [eng.finished[i] for i in ids], time.perf_counter() - t0, steps
 
-    run(min(4, args.requests), 8)  # warm-up: kernels loaded, graphs of the small batches captured
+    run(min(4, args.requests), 8)  # warm-up: kernels loaded
+    runner.warm_up(args.requests, longest)  # the decode graphs of every batch size, as a server does after loading
     runner.rows_asked = runner.rows_run = 0
     eng, reqs, total_s, steps = run(args.requests, args.new_tokens)
     generated = sum(len(r.generated) for r in reqs)
@@ -289,8 +290,9 @@ def main() -> int:
     point_batches = [int(b) for b in args.points.split(",") if b] if not args.no_points and args.phase == "all" else []
     max_batch = max([args.batch] + point_batches)
     budget = max(PREFILL_TOKENS, max_batch)
-    # requests whose prompt went in first decode while the others' prompts still go in
-    slack = -(-max_batch * args.context // budget) + 2
+    # requests whose prompt went in first decode while the others' prompts still go in (and take a growing share
+    # of every step's budget from them)
+    slack = 2 * -(-max_batch * args.context // budget) + 8
     new_tokens = args.warmup + args.steps + slack
     decode_len = args.context + new_tokens + 1
     cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], PREFILL_TOKENS + 8, decode_len)

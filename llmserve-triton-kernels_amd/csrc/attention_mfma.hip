@@ -169,6 +169,8 @@ __global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const A
     const int b = a.seq_begin + blockIdx.z;
     const int tok0 = a.cu_seqlens[b], n_new = a.cu_seqlens[b + 1] - tok0;
     const int ctx = a.context_lens[b];
+    // (asked for together with the lengths: one trip to memory earlier than where the block table is first needed)
+    const int table_row = a.table_rows ? a.table_rows[b] : b;
 
     const int tile = blockIdx.x / a.num_splits, split = blockIdx.x % a.num_splits;
     const int t_first = tile * TPG;  // first token (within the request's new tokens) of this group
@@ -204,7 +206,7 @@ __global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const A
     for (int m = 0; m < DB; ++m) acc[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    const int* table = a.block_tables + (size_t)(a.table_rows ? a.table_rows[b] : b) * a.max_blocks;
+    const int* table = a.block_tables + (size_t)table_row * a.max_blocks;
     const uint32_t page_stride = (uint32_t)a.n_kv_heads * a.block_size * D;
     const bf16* k_base = a.k_pool + (size_t)kvh * a.block_size * D;
     const bf16* v_base = a.v_pool + (size_t)kvh * a.block_size * D;
@@ -375,6 +377,8 @@ __global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt
     const int b = a.seq_begin + blockIdx.z;
     const int tok0 = a.cu_seqlens[b], n_new = a.cu_seqlens[b + 1] - tok0;
     const int ctx = a.context_lens[b];
+    // (asked for together with the lengths: one trip to memory earlier than where the block table is first needed)
+    const int table_row = a.table_rows ? a.table_rows[b] : b;
     // wg_first: first token (within the request's new tokens) of the block whose keys the workgroup walks;
     // my_first: of the block this wave works for
     int wg_first, my_first;
@@ -438,7 +442,7 @@ __global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt
         l_run[cg] = 0.f;
     }
 
-    const int* table = a.block_tables + (size_t)(a.table_rows ? a.table_rows[b] : b) * a.max_blocks;
+    const int* table = a.block_tables + (size_t)table_row * a.max_blocks;
     const uint32_t page_stride = (uint32_t)a.n_kv_heads * a.block_size * D;
     const bf16* k_base = a.k_pool + (size_t)kvh * a.block_size * D;
     const bf16* v_base = a.v_pool + (size_t)kvh * a.block_size * D;

@@ -60,6 +60,11 @@ class LLM:
             self._tokenizer = AutoTokenizer.from_pretrained(str(self._model_dir))
         return self._tokenizer
 
+    def warm_up(self, max_requests: int | None = None, max_context: int | None = None) -> int:
+        """Capture the decode graphs ahead of time (`ModelRunner.warm_up`): a server calls this once after loading,
+        so that the first request of every batch size does not wait for a capture."""
+        return self.runner.warm_up(max_requests or self.engine.max_num_seqs, max_context)
+
     # ---- generation ------------------------------------------------------------------------------
     def generate(self, prompts, params: SamplingParams | list[SamplingParams] | None = None) -> list[GenerationResult]:
         """Generate for every prompt (lists of token ids, or strings when the folder has a

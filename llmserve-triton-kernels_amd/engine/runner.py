@@ -204,20 +204,46 @@ class ModelRunner:
         return logits if owned or borrow else logits.clone()
 
     # ---- decode-only steps as HIP graphs --------------------------------------------------------
+    @staticmethod
+    def _decode_bucket(n_requests: int, context: int) -> tuple[int, int]:
+        """(capacity, reach) of the graph that a decode step of `n_requests` whose longest context is `context`
+        replays: powers of two, the reach from 256."""
+        capacity = 1
+        while capacity < n_requests:
+            capacity *= 2
+        reach = 256
+        while reach < context:
+            reach *= 2
+        return capacity, reach
+
+    @torch.inference_mode()
+    def warm_up(self, max_requests: int | None = None, max_context: int | None = None) -> int:
+        """Capture, ahead of time, the graphs that decode steps of up to `max_requests` requests with contexts up
+        to `max_context` replay (defaults: all the runner's slots, its longest request), so that no request waits
+        for a capture in the middle of serving.  Returns the number of graphs captured now; 0 for a runner that
+        launches its steps kernel by kernel."""
+        if not self._use_graphs:
+            return 0
+        top_capacity, top_reach = self._decode_bucket(max_requests or self.manager.max_seqs,
+                                                      max_context or self.max_model_len)
+        made, capacity = 0, 1
+        while capacity <= top_capacity:
+            reach = 256
+            while reach <= top_reach:
+                if (capacity, reach) not in self._graphs:
+                    self._graphs[(capacity, reach)] = _DecodeGraph(self, capacity, reach)
+                    made += 1
+                reach *= 2
+            capacity *= 2
+        return made
+
     def _replay_decode(self, layout, tokens: list[int], logit_rows: list[int],
                        device_tokens: torch.Tensor | None = None) -> torch.Tensor:
         """A step of single tokens: replay the graph captured for this batch size and context range
         (capture it at first use).  The logits it returns live in the graph's own memory and are
         overwritten by the next replay of the same graph."""
         n = len(tokens)
-        capacity = 1
-        while capacity < n:
-            capacity *= 2
-        context = max(layout.starts) + 1
-        reach = 256
-        while reach < context:
-            reach *= 2
-        key = (capacity, reach)
+        capacity, reach = key = self._decode_bucket(n, max(layout.starts) + 1)
         graph = self._graphs.get(key)
         if graph is None:
             graph = _DecodeGraph(self, capacity, reach)

@@ -142,6 +142,23 @@ def test_temperature_sampling_is_seeded_and_matches_plain_sampler(model_dirs):
             assert lo - 1e-5 <= u < float(cdf[tok]) + 1e-5, (i, tok, u, lo, float(cdf[tok]))
 
 
+def test_warm_up_captures_the_decode_graphs_ahead(model_dirs):
+    """After `warm_up` no decode step has to capture anything, and the tokens are the same as without it."""
+    from llmserve import SamplingParams
+
+    name = "a"
+    prompts = [traces.random_ids(TINY[name][0]["vocab_size"], n, 300 + i) for i, n in enumerate([5, 17, 33])]
+    cold = _llm(model_dirs[name], name, "bfloat16")
+    want = [r.tokens for r in cold.generate(prompts, SamplingParams(max_new_tokens=12))]
+    warm = _llm(model_dirs[name], name, "bfloat16")
+    made = warm.warm_up()
+    assert made == 3 * 1 and warm.warm_up() == 0  # capacities 1, 2, 4 at the one reach that 128 positions need
+    before = set(warm.runner._graphs)
+    assert [r.tokens for r in warm.generate(prompts, SamplingParams(max_new_tokens=12))] == want
+    assert set(warm.runner._graphs) == before
+    assert _llm(model_dirs[name], name, "float32", use_graphs=False).warm_up() == 0
+
+
 def test_eos_stops_generation(model_dirs):
     from llmserve import SamplingParams
 
