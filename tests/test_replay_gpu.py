@@ -214,6 +214,24 @@ def test_replay_at_full_layer_sizes(wide_model_dir, dtype_name, mode, monkeypatc
         assert any(not waves and splits > 1 for waves, splits in shared_out), "no portion shared its keys out"
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+@pytest.mark.parametrize("name", list(TINY))
+def test_random_mixed_traces(model_dirs, name, seed):
+    """Random numbers of requests of random lengths (up to the model's limit), mixed with random cuts, in a pool
+    of exactly the pages the trace needs: both precisions against the plain implementation."""
+    import random
+
+    cfg, bs = TINY[name]
+    rng = random.Random(1000 * seed + len(name))
+    seqs = {f"r{i}": traces.random_ids(cfg["vocab_size"], rng.randint(1, cfg["max_position_embeddings"] - 2), 100 * seed + i)
+            for i in range(rng.randint(2, 7))}
+    steps = traces.mixed(seqs, seed=seed, live_max=4, tail=rng.randint(1, 8))
+    num_blocks = traces.tokens_needed(steps, round_to=bs) // bs
+    for dtype_name in DTYPES:
+        outputs = replay_in_process(model_dirs[name], dtype_name, steps, bs, num_blocks)
+        check_against_plain(model_dirs[name], dtype_name, seqs, steps, outputs)
+
+
 def test_mixed_trace_reuses_pages(model_dirs):
     """The mixed trace is only a test of reuse if it hands out more pages than the pool has."""
     seqs = sequences("a")
