@@ -235,6 +235,46 @@ def sync_costs(args) -> int:
     return 0
 
 
+def stream_rates(args) -> int:
+    """What memory gives a kernel that only reads (csrc/probe.hip): a gigabyte in one launch, by three ways of
+    sharing the addresses out to a wave's lanes, and pieces as large as the weight matrices of a decode step, each
+    in a launch of its own within a captured chain: the least that a product which must read such a matrix costs."""
+    import ctypes
+
+    import torch
+
+    from llmserve.config import preset
+    from llmserve.ops import library as ops
+
+    cfg = preset(args.model)
+    h, inter, nh, nkv = cfg["hidden_size"], cfg["intermediate_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    d = h // nh
+    pieces = {"qkv": (nh + 2 * nkv) * d * h * 2, "o_proj": h * nh * d * 2, "gate_up": 2 * inter * h * 2, "down_proj": h * inter * 2}
+    lib = ops.load("probe")
+    total = max(1 << 30, 16 * max(pieces.values()))
+    buf = torch.empty(total, dtype=torch.uint8, device="cuda:0")
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda:0")
+    results = (ctypes.c_float * 16)()
+    sizes = (ctypes.c_size_t * len(pieces))(*pieces.values())
+    torch.cuda.synchronize()
+    lib.llms_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
+    status = lib.llms_probe_stream(results, ctypes.c_void_p(buf.data_ptr()), total, sizes, len(pieces), ctypes.c_void_p(sink.data_ptr()))
+    if status != 0:
+        print(f"the probe failed with status {status}")
+        return 1
+    r = [float(v) for v in results]
+    per_piece = {name: {"MB": round(nbytes / 1e6, 1), "us": round(r[3 + i], 2), "GBps": round(nbytes / r[3 + i] / 1e3, 1)}
+                 for i, (name, nbytes) in enumerate(pieces.items())}
+    line = {"metric": "GB/s of a kernel that reads 1 GiB once, 1 KB of a row per instruction", "value": round(r[0], 1),
+            "unit": "GB/s", "n_gpus": 1, "steps": 0, "warmup": 0, "ms_per_step": 0.0, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"model": args.model, "parallelism": "single-gpu", "bytes": total},
+            "stream_GBps": {"1KB_of_a_row": round(r[0], 1), "64B_of_16_rows": round(r[1], 1), "256B_of_4_rows": round(r[2], 1)},
+            "one_launch_per_matrix": per_piece}
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -247,10 +287,10 @@ def main() -> int:
     ap.add_argument("--model", default="tinyllama-1.1b")
     ap.add_argument("--no-points", action="store_true", help="skip the further batch sizes")
     ap.add_argument("--points", default="1,64", help="further batch sizes to measure decoding at")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill", "gemv", "sync"], default="all",
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "gemv", "sync", "stream"], default="all",
                     help="run one phase only (for profiles; the line then holds zeros for the other); gemv: the "
                          "decode products alone, each over copies of its weight that do not fit the caches; sync: what a kernel "
-                         "boundary and a barrier inside a kernel cost")
+                         "boundary and a barrier inside a kernel cost; stream: what memory gives a kernel that only reads")
     ap.add_argument("--workload", choices=["steps", "serve"], default="steps")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
@@ -268,6 +308,8 @@ def main() -> int:
         return gemv(args)
     if args.phase == "sync":
         return sync_costs(args)
+    if args.phase == "stream":
+        return stream_rates(args)
 
     import torch
 

@@ -2,7 +2,36 @@
 // captured chain of dependent launches, and what a barrier over the whole grid costs inside one kernel (an atomic
 // counter and a bounded spin), with and without the release/acquire fences that make one workgroup's stores visible
 // to workgroups on other XCDs.  Every spin has a limit, so a mistake gives a count of failures, never a hang.
+// And what memory gives a kernel that only reads: a long stream, and a stream as short as one weight matrix of a
+// decode step, which is the floor for any product that must read that matrix in a launch of its own.
 #include "common.h"
+
+#include <algorithm>
+
+typedef __attribute__((ext_vector_type(4))) unsigned int probe_u32x4;
+
+// Reads a matrix of `rows` rows of 4,096 bytes (a bfloat16 weight with K = 2,048) and keeps nothing.  A wave takes
+// tiles of 16 rows, as the product kernels do.  PATTERN 0: an instruction covers 1 KB of one row; 1: 64 bytes of each
+// of the 16 rows (the matrix instruction's operand layout read straight from memory); 2: 256 bytes of 4 rows.
+template <int PATTERN>
+__global__ __launch_bounds__(256) void probe_read_kernel(const char* __restrict__ buf, int rows, unsigned* sink) {
+    constexpr int ROW = 4096;
+    const int lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
+    probe_u32x4 acc = {0, 0, 0, 0};
+    const int tiles = rows / 16, waves = gridDim.x * 4;
+    for (int t = blockIdx.x * 4 + wave; t < tiles; t += waves) {
+        const char* base = buf + (size_t)t * 16 * ROW;
+#pragma unroll 16
+        for (int i = 0; i < 16 * ROW / 1024; ++i) {
+            size_t off;
+            if (PATTERN == 0) off = (size_t)i * 1024 + lane * 16;
+            else if (PATTERN == 1) off = (size_t)(lane % 16) * ROW + i * 64 + (lane / 16) * 16;
+            else off = (size_t)((i / 16) * 4 + lane / 16) * ROW + (i % 16) * 256 + (lane % 16) * 16;
+            acc ^= __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4*>(base + off));
+        }
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[0] = acc.x;  // (keeps the loads; practically never true)
+}
 
 __global__ void probe_tiny_kernel(float* p, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -40,6 +69,19 @@ __global__ __launch_bounds__(256) void probe_barrier_kernel(unsigned* counter, f
         acc += v;
     }
     if (acc == 12345.678f) sink[0] = acc;
+}
+
+// Reads `bytes` (a multiple of 4 KB) and keeps nothing: a wave takes pieces of 4 KB, four loads in flight.
+__global__ __launch_bounds__(256) void probe_read_flat_kernel(const char* __restrict__ buf, size_t bytes, unsigned* sink) {
+    const int lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
+    probe_u32x4 acc = {0, 0, 0, 0};
+    const size_t pieces = bytes / 4096, waves = (size_t)gridDim.x * 4;
+    for (size_t p = (size_t)blockIdx.x * 4 + wave; p < pieces; p += waves) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            acc ^= __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4*>(buf + p * 4096 + i * 1024 + lane * 16));
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[0] = acc.x;
 }
 
 #define PROBE_CHECK(call)                                                                          \
@@ -124,6 +166,65 @@ int llms_probe_sync(float* results, void* scratch) {
     }
     results[10] = (float)total_fails[0];
     results[11] = (float)total_fails[1];
+    PROBE_CHECK(hipEventDestroy(a));
+    PROBE_CHECK(hipEventDestroy(b));
+    PROBE_CHECK(hipStreamDestroy(stream));
+    return LLMS_OK;
+}
+
+// results[0..2]: GB/s of a kernel that reads all of `buf` once (`bytes` >= 1 GiB, so that nothing comes from the
+// 256 MB memory-side cache), for the three patterns of probe_read_kernel.  results[3 + i]: microseconds per launch in
+// a captured chain of 16 launches that each read the next piece of piece_bytes[i] bytes (probe_read_flat_kernel, a
+// wave for every 4 KB up to 2,048 workgroups), i < n_pieces <= 8: what a kernel that must read that much costs at the
+// least.  `sink`: 4 bytes of
+// device memory.  The caller has synchronized the device; the probe runs on a stream of its own.
+int llms_probe_stream(float* results, const void* buf, size_t bytes, const size_t* piece_bytes, int n_pieces, void* sink) {
+    constexpr size_t TILE = 16 * 4096;
+    LLMS_REQUIRE(buf != nullptr && bytes >= ((size_t)1 << 30) && n_pieces >= 0 && n_pieces <= 8, "probe_stream: bad arguments");
+    for (int i = 0; i < n_pieces; ++i)
+        LLMS_REQUIRE(piece_bytes[i] >= TILE && piece_bytes[i] * 16 <= bytes, "probe_stream: 16 pieces must fit the buffer");
+    hipStream_t stream;
+    PROBE_CHECK(hipStreamCreate(&stream));
+    hipEvent_t a, b;
+    PROBE_CHECK(hipEventCreate(&a));
+    PROBE_CHECK(hipEventCreate(&b));
+    const char* base = static_cast<const char*>(buf);
+    unsigned* out = static_cast<unsigned*>(sink);
+    float ms = 0.f;
+    const int rows = (int)(bytes / TILE) * 16;
+    for (int p = 0; p < 3; ++p) {
+        for (int k = 0; k < 3; ++k) {  // (the last of three is timed)
+            PROBE_CHECK(hipEventRecord(a, stream));
+            if (p == 0) probe_read_kernel<0><<<2048, 256, 0, stream>>>(base, rows, out);
+            else if (p == 1) probe_read_kernel<1><<<2048, 256, 0, stream>>>(base, rows, out);
+            else probe_read_kernel<2><<<2048, 256, 0, stream>>>(base, rows, out);
+            PROBE_CHECK(hipEventRecord(b, stream));
+            PROBE_CHECK(hipStreamSynchronize(stream));
+        }
+        PROBE_CHECK(hipEventElapsedTime(&ms, a, b));
+        results[p] = (float)((double)rows * 4096 / (ms * 1e-3) / 1e9);
+    }
+    for (int i = 0; i < n_pieces; ++i) {
+        const size_t piece = piece_bytes[i] / 4096 * 4096;
+        const int grid = (int)std::min<size_t>(2048, (piece / 4096 + 3) / 4);
+        hipGraph_t graph;
+        hipGraphExec_t exec;
+        PROBE_CHECK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+        for (int k = 0; k < 16; ++k)
+            probe_read_flat_kernel<<<grid, 256, 0, stream>>>(base + (size_t)k * piece, piece, out);
+        PROBE_CHECK(hipStreamEndCapture(stream, &graph));
+        PROBE_CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+        PROBE_CHECK(hipGraphLaunch(exec, stream));
+        PROBE_CHECK(hipStreamSynchronize(stream));
+        PROBE_CHECK(hipEventRecord(a, stream));
+        for (int k = 0; k < 5; ++k) PROBE_CHECK(hipGraphLaunch(exec, stream));
+        PROBE_CHECK(hipEventRecord(b, stream));
+        PROBE_CHECK(hipStreamSynchronize(stream));
+        PROBE_CHECK(hipEventElapsedTime(&ms, a, b));
+        results[3 + i] = ms * 1e3f / 80.f;
+        PROBE_CHECK(hipGraphExecDestroy(exec));
+        PROBE_CHECK(hipGraphDestroy(graph));
+    }
     PROBE_CHECK(hipEventDestroy(a));
     PROBE_CHECK(hipEventDestroy(b));
     PROBE_CHECK(hipStreamDestroy(stream));
