@@ -7,7 +7,7 @@
 //                instruction; a workgroup owns 16 output features and its 8 waves split K; their
 //                partial sums meet in LDS in a fixed order.
 //   gemm_tile    any M: 128x128 tiles through double-buffered LDS, 4 waves of 64x64.
-// (The product for up to 16 rows, with its fused prologue and epilogues, is gemm_stream.hip.)
+// (The product for up to 16 rows, with its fused epilogues, is gemm_stream.hip.)
 //
 // K must be a multiple of 8 and rows 16-byte aligned (the host checks); M, N are arbitrary.
 #include "common.h"

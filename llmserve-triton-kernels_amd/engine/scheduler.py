@@ -260,15 +260,15 @@ class ContinuousBatchingEngine:
             self.stats.tokens_generated += 1
             p = request.params
             if p.eos_token_id is not None and token == p.eos_token_id:
-                verdict = "stop"
+                reason = "stop"
             elif len(request.generated) >= p.max_new_tokens:
-                verdict = "length"
+                reason = "length"
             else:
                 events.append(TokenEvent(request.req_id, token, False))
                 continue
             self.running.remove(request)
             self.manager.free_sequence(request.req_id)
-            self._retire(request, verdict, token, events)
+            self._retire(request, reason, token, events)
 
     # ------------------------------------------------------------------ pages
     def _pages_owed(self, request: Request) -> int:

@@ -81,6 +81,58 @@ def test_preemption_by_recompute_keeps_greedy_tokens(model_dirs, name):
     assert tight.engine.manager.num_free_blocks == 14
 
 
+@pytest.mark.parametrize("name,seed", [("a", 1), ("a", 2), ("b", 3), ("b", 4)])
+def test_random_serving_workloads_keep_greedy_tokens(model_dirs, name, seed):
+    """Requests that arrive while others run, a pool so small that some are thrown out and recomputed, a token
+    budget that cuts prompts anywhere, and requests stopped from outside in the middle: every request that runs to
+    its end has the tokens of the plain implementation, and every page comes back."""
+    import random
+
+    from llmserve import EngineConfig, SamplingParams
+    from llmserve.engine.runner import ModelRunner
+    from llmserve.engine.scheduler import ContinuousBatchingEngine
+    from llmserve.sampling import Sampler
+
+    rng = random.Random(seed)
+    vocab = TINY[name][0]["vocab_size"]
+    cfg, w = plain_llama.read_model_dir(model_dirs[name], torch.float32)
+    block_size = rng.choice([4, 8])
+    jobs = []
+    for i in range(10):
+        prompt = traces.random_ids(vocab, rng.randint(1, 48), 900 + 16 * seed + i)
+        jobs.append(dict(prompt=prompt, new=rng.randint(1, 18), arrive=rng.randint(0, 25), abort_at=None))
+    for job in rng.sample(jobs, 2):
+        job["abort_at"] = job["arrive"] + rng.randint(1, 8)
+    longest = max(len(j["prompt"]) + j["new"] for j in jobs)
+    pages = -(-longest // block_size) + rng.randint(2, 10)  # the longest request fits; several at once do not
+    runner = ModelRunner.from_folder(model_dirs[name], EngineConfig(dtype="float32", block_size=block_size, num_blocks=pages,
+                                                                   max_num_seqs=4, max_num_batched_tokens=rng.choice([8, 24, 64])))
+    engine = ContinuousBatchingEngine(runner, Sampler(runner.device), max_num_seqs=4,
+                                      max_num_batched_tokens=runner.engine_config.max_num_batched_tokens)
+    ids, step = {}, 0
+    while step < 400 and (engine.has_unfinished() or len(ids) < len(jobs)):
+        for i, job in enumerate(jobs):
+            if job["arrive"] == step:
+                ids[i] = engine.add_request(job["prompt"], SamplingParams(max_new_tokens=job["new"]))
+            if job["abort_at"] == step and i in ids:
+                engine.abort(ids[i])
+        engine.step()
+        step += 1
+    assert not engine.has_unfinished() and len(ids) == len(jobs)
+    finished = 0
+    for i, job in enumerate(jobs):
+        request = engine.finished[ids[i]]
+        want = plain_llama.generate(cfg, w, job["prompt"], job["new"], torch.float32)
+        if request.finish_reason == "abort":
+            assert job["abort_at"] is not None and request.generated == want[: len(request.generated)]
+        else:
+            assert request.finish_reason == "length" and request.generated == want, (i, job)
+            finished += 1
+    assert finished >= len(jobs) - 2
+    assert engine.manager.num_free_blocks == pages
+    engine.manager.check_invariants()
+
+
 def test_bfloat16_generation_follows_plain_logits(model_dirs):
     """In bfloat16 greedy ties can fall either way, so the check is on the logits: every token the
     engine picks must be (nearly) the best one under the plain bfloat16 implementation."""
