@@ -147,6 +147,7 @@ class CacheManager:
         return max((max(0, want - len(self.tables[g.group_id][seq_id])) for g in self.paged_groups), default=0)
 
     def can_append(self, seq_ids, counts) -> bool:
+        """Whether `append` with these arguments would find its pages."""
         need = sum(self.extra_blocks_needed(s, n) for s, n in zip(seq_ids, counts))
         return need <= self.num_free_blocks
 

@@ -82,6 +82,7 @@ def test_append_is_atomic():
     m = CacheManager(full_groups(), num_blocks=2, block_size=4, max_seqs=2)
     m.add_sequence(0)
     m.add_sequence(1)
+    assert not m.can_append([0, 1], [4, 8]) and m.can_append([0, 1], [4, 4]) and m.can_append([1], [8])
     with pytest.raises(OutOfBlocks):
         m.append([0, 1], [4, 8])
     assert m.num_free_blocks == 2 and m.lengths == {0: 0, 1: 0}
