@@ -460,6 +460,34 @@ def test_sample_rows_mixed_batch_and_frequencies():
     assert torch.allclose(freq, torch.softmax(logits[0].cpu() / 0.7, -1), atol=0.04)
 
 
+@pytest.mark.parametrize("vocab", [32000, 40000])
+def test_sample_rows_do_not_depend_on_the_batch_or_the_run(vocab):
+    """The thresholds are found with atomic additions to shared histograms: the sums are integers (counts, masses in
+    fixed point), so a row gives the same token wherever it stands in a batch and however often it is asked."""
+    rows = 33
+    logits = rnd(rows, vocab, seed=44, scale=4.0)
+    logits[5, 100:164] = logits[5, 99]  # many keys at one value: ties at a threshold
+    u = torch.rand(rows, generator=torch.Generator().manual_seed(45))
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    temp, k, p = torch.full((rows,), 0.9), torch.full((rows,), 50, dtype=torch.int32), torch.full((rows,), 0.8)
+    k[::3] = 0
+    p[1::3] = 1.0
+    first = ops().sample_rows(torch.empty(rows, dtype=torch.int32, device=DEV), dev(logits), temperature=dev(temp),
+                              top_k=dev(k), top_p=dev(p), uniform=dev(u)).clone()
+    for _ in range(10):
+        again = ops().sample_rows(torch.empty(rows, dtype=torch.int32, device=DEV), dev(logits), temperature=dev(temp),
+                                  top_k=dev(k), top_p=dev(p), uniform=dev(u))
+        assert torch.equal(again, first)
+    order = torch.randperm(rows, generator=torch.Generator().manual_seed(46))
+    moved = ops().sample_rows(torch.empty(rows, dtype=torch.int32, device=DEV), dev(logits[order]), temperature=dev(temp[order]),
+                              top_k=dev(k[order]), top_p=dev(p[order]), uniform=dev(u[order]))
+    assert torch.equal(moved.cpu(), first.cpu()[order])
+    for r in (0, 5, 17):
+        one = ops().sample_rows(torch.empty(1, dtype=torch.int32, device=DEV), dev(logits[r: r + 1]), temperature=dev(temp[r: r + 1]),
+                                top_k=dev(k[r: r + 1]), top_p=dev(p[r: r + 1]), uniform=dev(u[r: r + 1]))
+        assert int(one[0]) == int(first[r])
+
+
 # ------------------------------------------------------------------ attention on the matrix cores
 def run_attention_mfma(nh, nkv, d, bs, lens, new, window=0, seed=0, craft=None, split_waves=False, num_splits=1,
                        waves=4):
