@@ -44,10 +44,6 @@ class Request:
             return self.prompt_ids[start: start + count]
         return self.prompt_ids[start:] + self.generated[: start + count - n]
 
-    @property
-    def first_token_time(self) -> float | None:
-        return self.token_times[0] if self.token_times else None
-
 
 @dataclass
 class TokenEvent:
