@@ -232,6 +232,37 @@ def test_random_mixed_traces(model_dirs, name, seed):
         check_against_plain(model_dirs[name], dtype_name, seqs, steps, outputs)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations(tmp_path, seed):
+    """Configurations drawn at random from what config.json allows (head sizes in steps of 16 up to 256, 1 to 5 KV
+    heads with 1 to 32 query heads each, widths and vocabularies that are no power of two, bias or none, tied or
+    untied head, one to three layers, pages of 4 to 32 tokens): a mixed trace on exactly the pages it needs, in both
+    precisions, with and without graphs, against the plain implementation."""
+    import random
+
+    from llmserve.weights import write_random_model
+
+    rng = random.Random(4000 + seed)
+    head_dim = rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 256])
+    group = rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 24, 32])
+    kv_heads = rng.randint(1, max(1, min(5, 2048 // (head_dim * group))))
+    heads = kv_heads * group
+    cfg = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=rng.choice([97, 256, 333, 1000, 2053, 5003]),
+               hidden_size=heads * head_dim, intermediate_size=8 * rng.randint(3, 60), num_hidden_layers=rng.randint(1, 3),
+               num_attention_heads=heads, num_key_value_heads=kv_heads, max_position_embeddings=rng.choice([96, 160, 300]),
+               rope_theta=rng.choice([1e4, 5e5, 1e6]), rms_norm_eps=rng.choice([1e-5, 1e-6]),
+               tie_word_embeddings=rng.random() < 0.4, attention_bias=rng.random() < 0.3)
+    block_size = rng.choice([4, 8, 16, 32])
+    write_random_model(tmp_path, cfg, seed=seed)
+    longest = cfg["max_position_embeddings"] - 2
+    seqs = {f"s{i}": traces.random_ids(cfg["vocab_size"], rng.randint(1, longest), 100 * seed + i) for i in range(rng.randint(2, 5))}
+    steps = traces.mixed(seqs, seed=seed, live_max=4, tail=rng.randint(1, 6))
+    num_blocks = traces.tokens_needed(steps, round_to=block_size) // block_size
+    for dtype_name in DTYPES:
+        outputs = replay_in_process(tmp_path, dtype_name, steps, block_size, num_blocks, use_graphs=rng.random() < 0.7)
+        check_against_plain(tmp_path, dtype_name, seqs, steps, outputs)
+
+
 def test_mixed_trace_reuses_pages(model_dirs):
     """The mixed trace is only a test of reuse if it hands out more pages than the pool has."""
     seqs = sequences("a")
