@@ -7,13 +7,15 @@ extern "C" {
 
 // bfloat16 causal attention over the paged cache for the requests [seq_begin, seq_begin + n_seqs) of a step
 // (see the comment at its definition).  With num_splits > 1 the caller brings the workspace for the partial
-// results: ws_o [rows * heads * splits * head_dim] and ws_ml [rows * heads * splits * 2] floats.
+// results: ws_o [rows * heads * splits * head_dim] and ws_ml [rows * heads * splits * 2] floats; and, if it wants the
+// shares of a decoding launch added up by the workgroup that finishes last rather than by a second kernel, n_arrive
+// counters that are zero and stay zero (arrive; null: the second kernel).
 int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
                         const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
                         const int* cu_seqlens, const int* context_lens, int seq_begin, int n_seqs, int max_new,
                         int token_begin, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int block_size,
                         int window, float scale, int split_waves, int num_splits, int waves, float* ws_o,
-                        float* ws_ml, hipStream_t stream);
+                        float* ws_ml, unsigned* arrive, int n_arrive, hipStream_t stream);
 
 // The split decode attention (every request brings one token; its keys are dealt to `waves` = 4 or 8 waves and
 // to num_splits >= 2 workgroups, merged in fixed order) for callers that cannot allocate: code under HIP graph

@@ -67,6 +67,10 @@ struct AttnArgs {
     int num_splits;
     float* ws_o;   // [token, head, split, D]
     float* ws_ml;  // [token, head, split, 2]
+    // decoding with num_splits > 1: one counter per column group (request, KV head, block of heads, group of tokens),
+    // zero between launches.  Non-null: the workgroups of a group count themselves here and the last to arrive adds
+    // the shares up (no merge kernel).
+    unsigned* arrive;
 };
 
 // 2^x by the hardware's own instruction.  Scores are kept in units of log2(e) (scale_log2 = scale * log2 e), so
@@ -152,6 +156,69 @@ __device__ __forceinline__ void attend_tile(f32x4 (&acc)[DB], float& m_run, floa
 #pragma unroll
     for (int m = 0; m < DB; ++m)
         acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[m]), as_bf16x8(pf), acc[m], 0, 0, 0);
+}
+
+// 8 bytes to or from memory past the caches that other XCDs do not see (an L2 belongs to one XCD): what one
+// workgroup leaves for another inside a kernel goes this way, with a relaxed atomic access at agent scope, which
+// the compiler turns into a store that is written through and a load that does not hit a stale line.  No fence:
+// a release at agent scope writes a whole L2 back and costs more than the kernel (10 to 130 microseconds a
+// launch where this costs 2 to 4: csrc/probe.hip's companion measurement).
+__device__ __forceinline__ void store_across(float* p, float a, float b) {
+    const unsigned long long v = ((unsigned long long)__float_as_uint(b) << 32) | __float_as_uint(a);
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ float2 load_across(const float* p) {
+    const unsigned long long v =
+        __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return make_float2(__uint_as_float((unsigned)v), __uint_as_float((unsigned)(v >> 32)));
+}
+
+// The last workgroup of a column group adds the shares of all its workgroups up, split 0 first, with the arithmetic
+// of attn_merge_kernel (the same bits).  SMAX >= num_splits: every load of a thread is asked for before the first
+// is used (a split beyond the last is the last once more, with weight 0).
+template <int DB, int SMAX>
+__device__ __forceinline__ void merge_shares(const AttnArgs& a, size_t item0, bool col_ok, int wave, int nw, int g,
+                                             bf16* orow) {
+    constexpr int D = DB * 16;
+    if (!col_ok) return;
+    const int S = a.num_splits;
+    float2 ml[SMAX];
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) ml[s] = load_across(a.ws_ml + 2 * (item0 + min(s, S - 1)));
+    float m_tot = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) m_tot = fmaxf(m_tot, ml[s].x);
+    float w[SMAX], l_tot = 0.f;
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) {
+        w[s] = (s < S && ml[s].x != -INFINITY) ? exp2_fast(ml[s].x - m_tot) : 0.f;
+        if (s < S && ml[s].x != -INFINITY) l_tot += ml[s].y * w[s];
+    }
+    const float inv = 1.f / l_tot;
+    for (int m = wave; m < DB; m += nw) {
+        float2 lo[SMAX], hi[SMAX];
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s) {
+            const float* share = a.ws_o + (item0 + min(s, S - 1)) * D + 16 * m + 4 * g;
+            lo[s] = load_across(share);
+            hi[s] = load_across(share + 2);
+        }
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s) {
+            if (s < S && ml[s].x != -INFINITY) {
+                o.x += lo[s].x * w[s];
+                o.y += lo[s].y * w[s];
+                o.z += hi[s].x * w[s];
+                o.w += hi[s].y * w[s];
+            }
+        }
+        uint2 pk;
+        pk.x = pack_bf16(o.x * inv, o.y * inv);
+        pk.y = pack_bf16(o.z * inv, o.w * inv);
+        *reinterpret_cast<uint2*>(orow + 16 * m + 4 * g) = pk;
+    }
 }
 
 template <int DB>
@@ -332,13 +399,41 @@ __global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const A
             pk.x = pack_bf16(o.x * inv, o.y * inv);
             pk.y = pack_bf16(o.z * inv, o.w * inv);
             *reinterpret_cast<uint2*>(a.out + (size_t)(tok0 + c_tok) * a.out_stride + (size_t)head * D + 16 * m + 4 * g) = pk;
+        } else if (a.arrive) {
+            store_across(a.ws_o + item * D + 16 * m + 4 * g, o.x, o.y);
+            store_across(a.ws_o + item * D + 16 * m + 4 * g + 2, o.z, o.w);
         } else {
             *reinterpret_cast<float4*>(a.ws_o + item * D + 16 * m + 4 * g) = o;
         }
     }
     if (a.num_splits > 1 && wave == 0 && g == 0 && col_ok) {
-        a.ws_ml[item * 2] = m_tot;
-        a.ws_ml[item * 2 + 1] = l_tot;
+        if (a.arrive) {
+            store_across(a.ws_ml + item * 2, m_tot, l_tot);
+        } else {
+            a.ws_ml[item * 2] = m_tot;
+            a.ws_ml[item * 2 + 1] = l_tot;
+        }
+    }
+    if (a.num_splits > 1 && a.arrive) {  // (the same in every thread of the launch)
+        // A thread's stores have been taken by memory before its workgroup is counted; the one that finds all
+        // others counted reads their shares.  Nobody waits for anybody: a workgroup that is not the last leaves.
+        __shared__ unsigned is_last;
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned* counter = a.arrive + ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * (gridDim.x / a.num_splits) + tile;
+            const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = before + 1 == (unsigned)a.num_splits;
+            if (is_last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero again for the next launch
+        }
+        __syncthreads();
+        if (!is_last) return;
+        const size_t item0 = ((size_t)(tok0 + c_tok) * a.n_heads + head) * a.num_splits;
+        bf16* orow = a.out + (size_t)(tok0 + c_tok) * a.out_stride + (size_t)head * D;
+        if (a.num_splits <= 2) merge_shares<DB, 2>(a, item0, col_ok, wave, nw, g, orow);
+        else if (a.num_splits <= 4) merge_shares<DB, 4>(a, item0, col_ok, wave, nw, g, orow);
+        else if (a.num_splits <= 8) merge_shares<DB, 8>(a, item0, col_ok, wave, nw, g, orow);
+        else merge_shares<DB, 16>(a, item0, col_ok, wave, nw, g, orow);
     }
 }
 
@@ -668,14 +763,16 @@ extern "C" {
 // split_waves = 1 deals the keys of each column group to `waves` (4 or 8) waves and
 // `num_splits` workgroups (decoding); split_waves = 0 with num_splits > 1 shares the keys of each block of prompt
 // tokens out to that many workgroups (no window then); with num_splits > 1 the caller provides ws_o [tokens * heads * splits * D] and
-// ws_ml [tokens * heads * splits * 2] floats, indexed by absolute token row.
+// ws_ml [tokens * heads * splits * 2] floats, indexed by absolute token row.  `arrive` (may be null): n_arrive
+// counters in device memory, all zero, which the kernel leaves zero: decoding with 2 to 16 splits then adds the
+// shares up in the workgroup that finishes last instead of in a second kernel.
 int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
                         const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
                         const int* cu_seqlens,
                         const int* context_lens, int seq_begin, int n_seqs, int max_new, int token_begin,
                         int n_tokens, int n_heads, int n_kv_heads, int head_dim, int block_size, int window,
                         float scale, int split_waves, int num_splits, int waves, float* ws_o, float* ws_ml,
-                        hipStream_t stream) {
+                        unsigned* arrive, int n_arrive, hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && n_heads > 0 && n_kv_heads > 0, "attention_mfma: sizes must be positive");
     LLMS_REQUIRE(n_heads % n_kv_heads == 0, "attention_mfma: n_heads must be a multiple of n_kv_heads");
     LLMS_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256, "attention_mfma: head_dim must be a multiple of 16 up to 256");
@@ -698,12 +795,14 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     const int groups = (max_new + TPG - 1) / TPG;
     AttnArgs a = {(bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pool, (const bf16*)v_pool,
                   block_tables, table_rows, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
-                  window, scale, num_splits, ws_o, ws_ml};
+                  window, scale, num_splits, ws_o, ws_ml, nullptr};
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
+    LLMS_REQUIRE(arrive == nullptr || ((uintptr_t)arrive % 4 == 0 && n_arrive > 0), "attention_mfma: bad counters");
     if (split_waves > 0) {
         dim3 grid(groups * num_splits, n_kv_heads * HB, n_seqs);
+        if (arrive && num_splits > 1 && num_splits <= 16 && (long long)groups * grid.y * grid.z <= n_arrive) a.arrive = arrive;
         if (int e = launch_attn(head_dim / 16, grid, waves * LLMS_WAVE, a, stream)) return e;
-        if (num_splits > 1) {
+        if (num_splits > 1 && a.arrive == nullptr) {
             hipError_t e1 = hipGetLastError();
             if (e1 != hipSuccess) {
                 fprintf(stderr, "llmserve kernel launch failed: %s\n", hipGetErrorString(e1));
@@ -801,7 +900,7 @@ int llms_attention_decode_noalloc(void* out, int out_stride, const void* q, int 
     return llms_attention_mfma(out, out_stride, q, q_stride, k_pool, v_pool, block_tables, table_rows, max_blocks,
                                cu_seqlens, context_lens, seq_begin, n_seqs, /*max_new=*/1, token_begin, n_tokens, n_heads,
                                n_kv_heads, head_dim, block_size, window, scale, /*split_waves=*/1, num_splits, waves, ws_o,
-                               ws_ml, stream);
+                               ws_ml, /*arrive=*/nullptr, 0, stream);
 }
 
 }  // extern "C"

@@ -408,6 +408,22 @@ def gemm_slices(parts: torch.Tensor, x: torch.Tensor, w: torch.Tensor) -> torch.
 # ------------------------------------------------------------------------------ attention
 
 
+_ARRIVAL_COUNTERS: dict = {}
+ARRIVAL_COUNTERS = 1 << 16
+
+
+def _arrival_counters(dev) -> torch.Tensor | None:
+    """The device's counters for workgroups that add each other's shares up inside a kernel: all zero, and every
+    kernel that uses them leaves them so.  Made at the first call that is not being captured into a graph (a fill
+    inside a graph would run at every replay); until then there are none and the caller takes its other way."""
+    key = (dev.type, dev.index)
+    if key not in _ARRIVAL_COUNTERS:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        _ARRIVAL_COUNTERS[key] = torch.zeros(ARRIVAL_COUNTERS, dtype=torch.int32, device=dev)
+    return _ARRIVAL_COUNTERS[key]
+
+
 def _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size):
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < n_heads * head_dim:
         raise ValueError("q must be [N, >= n_heads*head_dim] with unit inner stride")
@@ -472,13 +488,16 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
                    seq_begin: int, n_seqs: int, max_new: int, token_begin: int, n_tokens: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, block_size: int, window: int = 0,
                    scale: float | None = None, split_waves: bool = False, num_splits: int = 1,
-                   table_rows: torch.Tensor | None = None, waves: int = 4) -> torch.Tensor:
+                   table_rows: torch.Tensor | None = None, waves: int = 4, merge_kernel: bool = False) -> torch.Tensor:
     """bfloat16 causal attention on the matrix cores for requests [seq_begin, seq_begin + n_seqs) of a
     step, whose new tokens are rows [token_begin, token_begin + n_tokens) of q and out and bring at most
     `max_new` tokens each.  `split_waves` (with `waves` = 4 or 8 and `num_splits`) spreads each request's keys
     over the waves of a workgroup and over workgroups: the arrangement for single decoded tokens.  Without
     it the 4 waves of a workgroup take neighbouring tokens and share each tile of keys through LDS; `num_splits`
-    then shares the keys of such a block of tokens out to several workgroups (short portions, long prefixes)."""
+    then shares the keys of such a block of tokens out to several workgroups (short portions, long prefixes).
+    The shares of workgroups are added up, in the order of the splits, by a second kernel, or for decoding with up
+    to 16 splits by the workgroup of each group that finishes last (`merge_kernel=True` asks for the second kernel
+    there too: the same bits)."""
     dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, table_rows)
     _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
     if not attention_mfma_supported(q.dtype, head_dim, block_size):
@@ -505,7 +524,9 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
         raise ValueError("8 waves take head_dim up to 160 (wider heads would not fit the registers)")
     if n_seqs == 0 or n_tokens == 0:
         return out
-    ws_o = ws_ml = None
+    ws_o = ws_ml = arrive = None
+    if num_splits > 1 and split_waves and not merge_kernel:
+        arrive = _arrival_counters(dev)
     if num_splits > 1:
         ws_o = torch.empty((q.shape[0] * n_heads * num_splits * head_dim,), dtype=torch.float32, device=dev)
         ws_ml = torch.empty((q.shape[0] * n_heads * num_splits * 2,), dtype=torch.float32, device=dev)
@@ -517,7 +538,8 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
         c_int(n_seqs), c_int(max_new), c_int(token_begin), c_int(n_tokens), c_int(n_heads), c_int(n_kv_heads),
         c_int(head_dim), c_int(block_size), c_int(window), c_float(scale),
         c_int(1 if split_waves else 0),
-        c_int(num_splits), c_int(waves), _ptr(ws_o), _ptr(ws_ml), _stream(dev)), "attention_mfma")
+        c_int(num_splits), c_int(waves), _ptr(ws_o), _ptr(ws_ml), _ptr(arrive),
+        c_int(arrive.numel() if arrive is not None else 0), _stream(dev)), "attention_mfma")
     return out
 
 

@@ -148,10 +148,12 @@ class Attention(Mixer):
 
     def decode_arrangement(self, n_requests: int, max_context: int) -> tuple[int, int]:
         """(workgroups per request and KV head, waves per workgroup) for decoding.  The waves of a
-        workgroup take 32 keys at a time each and merge inside the kernel; workgroups that share a
-        request need a second kernel to merge, which costs more than a few extra tiles per wave.  So a
-        small batch first gets 8 waves, and is split over workgroups only when a wave would still
-        walk more than 4 tiles; once the batch alone fills the chip (256 workgroups) nothing is split."""
+        workgroup take 32 keys at a time each and merge in LDS; workgroups that share a request hand
+        their shares to the one that finishes last, through memory, which costs more (2 to 3
+        microseconds) than a few extra tiles per wave.  So a small batch first gets 8 waves, and is
+        split over workgroups only when a wave would still walk more than 4 tiles (measured: at a
+        context of 512 no split pays at any batch size, at 4,096 four to eight do up to batch 8); once
+        the batch alone fills the chip (256 workgroups) nothing is split."""
         g = self.num_heads // self.num_kv_heads
         groups = n_requests * self.num_kv_heads * -(-g // 16)
         reach = min(max_context, self.window) if self.window else max_context

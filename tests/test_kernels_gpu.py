@@ -490,7 +490,7 @@ def test_sample_rows_do_not_depend_on_the_batch_or_the_run(vocab):
 
 # ------------------------------------------------------------------ attention on the matrix cores
 def run_attention_mfma(nh, nkv, d, bs, lens, new, window=0, seed=0, craft=None, split_waves=False, num_splits=1,
-                       waves=4):
+                       waves=4, merge_kernel=False, repeat=1):
     """As `run_attention`, for the bfloat16 matrix-core kernel and its request-wise arguments."""
     dtype = torch.bfloat16
     qs = [rnd(s, nh, d, seed=seed + 3 * b) for b, s in enumerate(lens)]
@@ -510,9 +510,11 @@ def run_attention_mfma(nh, nkv, d, bs, lens, new, window=0, seed=0, craft=None, 
     q = torch.cat([torch.cat(q_rows), torch.full((cu[-1], 2 * nkv * d), float("nan"), dtype=dtype)], dim=1).contiguous().to(DEV)
     out = torch.empty(cu[-1], nh * d, dtype=dtype, device=DEV)
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)  # noqa: E731
-    ops().attention_mfma(out, q, k_pool.to(DEV), v_pool.to(DEV), tables.to(DEV), i32(cu), i32(lens), 0, len(lens),
-                         max(new), 0, cu[-1], nh, nkv, d, bs, window, None, split_waves=split_waves,
-                         num_splits=num_splits, waves=waves)
+    operands = (q, k_pool.to(DEV), v_pool.to(DEV), tables.to(DEV), i32(cu), i32(lens))
+    for _ in range(repeat):  # (launches in a row find the counters of the one before zero again)
+        out.fill_(float("nan"))
+        ops().attention_mfma(out, *operands, 0, len(lens), max(new), 0, cu[-1], nh, nkv, d, bs, window, None,
+                             split_waves=split_waves, num_splits=num_splits, waves=waves, merge_kernel=merge_kernel)
     got = out.float().cpu()
     assert torch.isfinite(got).all(), "read a slot that was never written"
     return got, torch.cat(refs)
@@ -559,6 +561,61 @@ def test_attention_mfma(case, arrangement):
     got, ref = run_attention_mfma(nh, nkv, d, bs, lens, new, window, seed=50, split_waves=split_waves,
                                   num_splits=num_splits, waves=waves)
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("case", [(8, 2, 64, 16, [300, 64, 129, 1, 17, 600, 33, 90], 4, 8), (32, 4, 64, 16, [520], 8, 8),
+                                  (64, 8, 128, 16, [700, 33], 2, 8), (3, 1, 32, 8, [1, 7, 40, 100], 3, 4),
+                                  (6, 2, 80, 8, [70, 19, 300], 16, 4), (4, 4, 256, 16, [257, 31], 5, 4),
+                                  (32, 1, 48, 8, [450, 2], 7, 8)])
+def test_decode_shares_added_up_by_the_last_workgroup(case):
+    """Decoding with the keys of a request shared out to workgroups: the shares are added up inside the kernel by
+    the workgroup of each column group that finishes last (data handed over past the L2 of its XCD, a counter per
+    group that is zero again afterwards).  The same bits as the second kernel gives, launch after launch, and when
+    the launch is replayed from a graph."""
+    nh, nkv, d, bs, lens, splits, waves = case
+    new = [1] * len(lens)
+    want, ref = run_attention_mfma(nh, nkv, d, bs, lens, new, seed=80, split_waves=True, num_splits=splits, waves=waves,
+                                   merge_kernel=True)
+    assert (want - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
+    got, _ = run_attention_mfma(nh, nkv, d, bs, lens, new, seed=80, split_waves=True, num_splits=splits, waves=waves, repeat=5)
+    assert torch.equal(got, want)
+    from llmserve.ops import library
+
+    assert int(library._arrival_counters(torch.device(DEV)).abs().sum()) == 0
+
+
+def test_decode_shares_added_up_inside_a_replayed_graph():
+    nh, nkv, d, bs, lens, splits = 8, 2, 64, 16, [300, 64, 129, 600], 4
+    dtype = torch.bfloat16
+    qs = [rnd(s, nh, d, seed=90 + 3 * b) for b, s in enumerate(lens)]
+    ks = [rnd(s, nkv, d, seed=91 + 3 * b) for b, s in enumerate(lens)]
+    vs = [rnd(s, nkv, d, seed=92 + 3 * b) for b, s in enumerate(lens)]
+    qs, ks, vs = ([t.to(dtype) for t in ts] for ts in (qs, ks, vs))
+    k_pool, v_pool, tables = make_paged(ks, vs, bs, dtype, seed=9)
+    q = torch.cat([qs[b][-1:].reshape(1, nh * d) for b in range(len(lens))]).contiguous().to(DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)  # noqa: E731
+    operands = (q, k_pool.to(DEV), v_pool.to(DEV), tables.to(DEV), i32(list(range(len(lens) + 1))), i32(lens))
+    out = torch.empty(len(lens), nh * d, dtype=dtype, device=DEV)
+
+    def launch(**kw):
+        ops().attention_mfma(out, *operands, 0, len(lens), 1, 0, len(lens), nh, nkv, d, bs, 0, None, split_waves=True,
+                             num_splits=splits, waves=8, **kw)
+
+    launch(merge_kernel=True)
+    want = out.clone()
+    launch()  # (the counters exist from here on: a graph cannot make them)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch()
+        launch()
+    for _ in range(4):
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+        launch()  # eager work between the replays
+        assert torch.equal(out, want)
 
 
 # The prompt kernel gives a wave two column groups (32 columns) up to head_dim 128, and pairs early with late blocks of
