@@ -497,7 +497,7 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
     then shares the keys of such a block of tokens out to several workgroups (short portions, long prefixes).
     The shares of workgroups are added up, in the order of the splits, by a second kernel, or for decoding with up
     to 16 splits by the workgroup of each group that finishes last (`merge_kernel=True` asks for the second kernel
-    there too: the same bits)."""
+    there too: the same bits).  (For prompt portions the last workgroup was tried as well: no faster.)"""
     dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, table_rows)
     _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
     if not attention_mfma_supported(q.dtype, head_dim, block_size):
