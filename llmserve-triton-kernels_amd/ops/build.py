@@ -1,7 +1,7 @@
 """Compiles the HIP sources under ``csrc/`` for gfx950 into shared libraries.
 
 One source file becomes one library, named after the file and a hash of everything that
-goes into it (the file, the shared headers, the compiler flags).  A library whose hash
+goes into it (the file, the headers of this folder it includes, the compiler flags).  A library whose hash
 matches is loaded as it is; a missing or stale one is compiled at the first call that
 needs it, so a fresh checkout works without a build step.  Libraries are written into
 ``lib/`` next to the sources; when that folder cannot be written, into a per-user folder
@@ -61,10 +61,26 @@ def _hipcc() -> str:
                      "the engine has no fallback without its compiled kernels")
 
 
+_INCLUDE = re.compile(r'^\s*#\s*include\s+"([^"]+)"', re.MULTILINE)
+
+
+def _inputs(name: str) -> list[Path]:
+    """The source file and the headers of this folder it includes, directly or through one another."""
+    found: dict[str, Path] = {}
+    todo = [CSRC_DIR / f"{name}.hip"]
+    while todo:
+        path = todo.pop()
+        if path.name in found or not path.exists():
+            continue
+        found[path.name] = path
+        todo += [CSRC_DIR / inc for inc in _INCLUDE.findall(path.read_text(errors="replace"))]
+    return [found[k] for k in sorted(found)]
+
+
 def _source_hash(name: str) -> str:
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    for p in sorted(CSRC_DIR.glob("*.h")) + [CSRC_DIR / f"{name}.hip"]:
+    for p in _inputs(name):
         h.update(p.name.encode())
         h.update(p.read_bytes())
     return h.hexdigest()[:12]

@@ -28,3 +28,21 @@ def test_library_names_change_with_the_flags(monkeypatch):
     before = build._source_hash("gemm")
     monkeypatch.setattr(build, "HIPCC_FLAGS", build.HIPCC_FLAGS + ["-DX=1"])
     assert build._source_hash("gemm") != before
+
+
+def test_library_names_follow_the_headers_a_source_includes(tmp_path, monkeypatch):
+    """A header counts for the sources that include it, directly or through another header, and for no other: a
+    change to one kernel's header must not make every built library stale."""
+    (tmp_path / "common.h").write_text("#pragma once\n")
+    (tmp_path / "wide.h").write_text('#include "deep.h"\n')
+    (tmp_path / "deep.h").write_text("// deep\n")
+    (tmp_path / "one.hip").write_text('#include "common.h"\n#include "wide.h"\n#include <vector>\n')
+    (tmp_path / "two.hip").write_text('  #  include "common.h"\n')
+    monkeypatch.setattr(build, "CSRC_DIR", tmp_path)
+    assert [p.name for p in build._inputs("one")] == ["common.h", "deep.h", "one.hip", "wide.h"]
+    assert [p.name for p in build._inputs("two")] == ["common.h", "two.hip"]
+    one, two = build._source_hash("one"), build._source_hash("two")
+    (tmp_path / "deep.h").write_text("// deeper\n")
+    assert build._source_hash("one") != one and build._source_hash("two") == two
+    (tmp_path / "common.h").write_text("#pragma once\n// more\n")
+    assert build._source_hash("two") != two
