@@ -224,13 +224,26 @@ def sync_costs(args) -> int:
         print(f"the probe failed with status {status}")
         return 1
     r = [round(float(v), 2) for v in results]
+    hand = (ctypes.c_float * 16)()
+    space = torch.zeros(1024 * 768 + 2048, dtype=torch.float32, device="cuda:0")
+    torch.cuda.synchronize()
+    status = lib.llms_probe_handover(hand, ctypes.c_void_p(space.data_ptr()))
+    if status != 0:
+        print(f"the probe failed with status {status}")
+        return 1
+    h = [round(float(v), 2) for v in hand]
+    cases = ["64_workgroups_in_pairs", "64_workgroups_in_eights", "256_workgroups_in_fours", "1024_workgroups_in_fours"]
+    handover = {name: {"stores_only": h[3 * i], "atomic_accesses_no_fence": h[3 * i + 1], "fences": h[3 * i + 2]}
+                for i, name in enumerate(cases)}
     line = {"metric": "microseconds per kernel boundary in a captured chain of launches", "value": r[1], "unit": "us",
             "n_gpus": 1, "steps": 0, "warmup": 0, "ms_per_step": 0.0, "higher_is_better": False, "scaling": "weak",
             "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"parallelism": "single-gpu"},
             "kernel_boundary_us": {"8_workgroups": r[0], "256_workgroups": r[1], "1024_workgroups": r[2]},
             "grid_barrier_us": {"64": r[3], "256": r[4], "512": r[5], "1024": r[6]},
             "grid_barrier_with_fences_us": {"64": r[7], "256": r[8], "512": r[9]},
-            "spin_limits_hit": r[10], "stale_reads": r[11]}
+            "spin_limits_hit": r[10], "stale_reads": r[11],
+            # a launch in which the last workgroup of every group reads what the others of the group wrote
+            "handover_us_per_launch": handover, "handover_stale_reads": h[12]}
     print(json.dumps(line))
     return 0
 

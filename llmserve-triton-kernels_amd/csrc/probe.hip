@@ -2,7 +2,8 @@
 // captured chain of dependent launches, and what a barrier over the whole grid costs inside one kernel (an atomic
 // counter and a bounded spin), with and without the release/acquire fences that make one workgroup's stores visible
 // to workgroups on other XCDs.  Every spin has a limit, so a mistake gives a count of failures, never a hang.
-// And what memory gives a kernel that only reads: a long stream, and a stream as short as one weight matrix of a
+// What it costs workgroups to hand data to one another inside a kernel without waiting for each other (the last
+// to arrive does the common work).  And what memory gives a kernel that only reads: a long stream, and a stream as short as one weight matrix of a
 // decode step, which is the floor for any product that must read that matrix in a launch of its own.
 #include "common.h"
 
@@ -82,6 +83,59 @@ __global__ __launch_bounds__(256) void probe_read_flat_kernel(const char* __rest
             acc ^= __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4*>(buf + p * 4096 + i * 1024 + lane * 16));
     }
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[0] = acc.x;
+}
+
+// What it costs workgroups to hand data to one another inside a kernel, the way the decode attention adds its
+// shares up: groups of S workgroups; each writes 512 floats, is counted at its group's counter, and the last to be
+// counted reads the 512 floats of every member and checks them (a stale value is counted), then sets the counter
+// back to zero.  MODE 0: the stores alone.  MODE 1: stores and loads are relaxed atomic accesses at agent scope
+// (written through, read past the L2 of the reader's XCD), ordered by a wait for the stores, no fence.  MODE 2:
+// plain stores and loads with __threadfence() on both sides, the textbook way.  Nobody waits for anybody.
+template <int MODE>
+__global__ __launch_bounds__(256) void probe_handover_kernel(float* data, unsigned* counters, unsigned* stale, int S, int round,
+                                                             float* out) {
+    __shared__ unsigned last;
+    const int wg = blockIdx.x, group = wg / S;
+    float* mine = data + (size_t)wg * 512;
+    const float v = (float)(round * 1000 + wg);
+    for (int i = threadIdx.x; i < 512; i += 256) {
+        if (MODE == 2) mine[i] = v + i;
+        else __hip_atomic_store(mine + i, v + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (MODE == 0) return;
+    if (MODE == 2) __threadfence();
+    else __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned before = __hip_atomic_fetch_add(counters + group, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last = before + 1 == (unsigned)S;
+        if (last) __hip_atomic_store(counters + group, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!last) return;
+    if (MODE == 2) __threadfence();
+    float got[8][2];  // (all loads asked for before the first is looked at; S <= 8)
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        const float* theirs = data + (size_t)(group * S + min(s, S - 1)) * 512;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            got[s][j] = MODE == 2 ? theirs[threadIdx.x + 256 * j]
+                                  : __hip_atomic_load(theirs + threadIdx.x + 256 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    float acc = 0.f;
+    unsigned bad = 0;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        const float want = (float)(round * 1000 + group * S + min(s, S - 1));
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if (got[s][j] != want + (float)(threadIdx.x + 256 * j)) ++bad;
+            acc += got[s][j];
+        }
+    }
+    if (bad) atomicAdd(stale, bad);
+    out[(size_t)group * 256 + threadIdx.x] = acc;
 }
 
 #define PROBE_CHECK(call)                                                                          \
@@ -166,6 +220,57 @@ int llms_probe_sync(float* results, void* scratch) {
     }
     results[10] = (float)total_fails[0];
     results[11] = (float)total_fails[1];
+    PROBE_CHECK(hipEventDestroy(a));
+    PROBE_CHECK(hipEventDestroy(b));
+    PROBE_CHECK(hipStreamDestroy(stream));
+    return LLMS_OK;
+}
+
+// results[3 * i + m]: microseconds per launch of probe_handover_kernel<m> (m = 0 stores only, 1 atomic accesses
+// without a fence, 2 fences) in a captured chain of 100 launches, for the i-th of the cases (workgroups, group
+// size) = (64, 2), (64, 8), (256, 4), (1024, 4); results[12]: stale values seen by any of them (must be 0).
+// `scratch`: 1,024 * 768 floats and 8,192 further bytes of device memory.  The caller has synchronized the device.
+int llms_probe_handover(float* results, void* scratch) {
+    hipStream_t stream;
+    PROBE_CHECK(hipStreamCreate(&stream));
+    float* data = static_cast<float*>(scratch);
+    float* out = data + 1024 * 512;
+    unsigned* counters = reinterpret_cast<unsigned*>(data + 1024 * 768);
+    unsigned* stale = counters + 1024;
+    PROBE_CHECK(hipMemsetAsync(counters, 0, 8192, stream));
+    hipEvent_t a, b;
+    PROBE_CHECK(hipEventCreate(&a));
+    PROBE_CHECK(hipEventCreate(&b));
+    const int cases[4][2] = {{64, 2}, {64, 8}, {256, 4}, {1024, 4}};
+    float ms = 0.f;
+    for (int i = 0; i < 4; ++i) {
+        for (int mode = 0; mode < 3; ++mode) {
+            const int grid = cases[i][0], S = cases[i][1];
+            hipGraph_t graph;
+            hipGraphExec_t exec;
+            PROBE_CHECK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+            for (int r = 0; r < 100; ++r) {
+                if (mode == 0) probe_handover_kernel<0><<<grid, 256, 0, stream>>>(data, counters, stale, S, r + 1, out);
+                else if (mode == 1) probe_handover_kernel<1><<<grid, 256, 0, stream>>>(data, counters, stale, S, r + 1, out);
+                else probe_handover_kernel<2><<<grid, 256, 0, stream>>>(data, counters, stale, S, r + 1, out);
+            }
+            PROBE_CHECK(hipStreamEndCapture(stream, &graph));
+            PROBE_CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+            PROBE_CHECK(hipGraphLaunch(exec, stream));
+            PROBE_CHECK(hipStreamSynchronize(stream));
+            PROBE_CHECK(hipEventRecord(a, stream));
+            for (int k = 0; k < 5; ++k) PROBE_CHECK(hipGraphLaunch(exec, stream));
+            PROBE_CHECK(hipEventRecord(b, stream));
+            PROBE_CHECK(hipStreamSynchronize(stream));
+            PROBE_CHECK(hipEventElapsedTime(&ms, a, b));
+            results[3 * i + mode] = ms * 1e3f / 500.f;
+            PROBE_CHECK(hipGraphExecDestroy(exec));
+            PROBE_CHECK(hipGraphDestroy(graph));
+        }
+    }
+    unsigned seen = 0;
+    PROBE_CHECK(hipMemcpy(&seen, stale, sizeof(seen), hipMemcpyDeviceToHost));
+    results[12] = (float)seen;
     PROBE_CHECK(hipEventDestroy(a));
     PROBE_CHECK(hipEventDestroy(b));
     PROBE_CHECK(hipStreamDestroy(stream));
