@@ -221,8 +221,8 @@ __device__ __forceinline__ void merge_shares(const AttnArgs& a, size_t item0, bo
     }
 }
 
-template <int DB>
-__global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const AttnArgs a) {
+template <int DB, int NW>  // blocks of 16 dimensions of a head; waves of the workgroup (4 or 8), which share the keys
+__global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
     constexpr int KS = (D + 31) / 32;  // k-steps of the score product
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE;
@@ -285,7 +285,7 @@ __global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const A
     const int per_split = (n_tiles + a.num_splits - 1) / a.num_splits;
     const int t_begin = split * per_split + wave;
     const int t_end = min(n_tiles, (split + 1) * per_split);
-    const int t_step = blockDim.x / LLMS_WAVE;  // 4 or 8 waves share the keys
+    constexpr int t_step = NW;
     // The request's page ids are held in registers, 64 blocks at a time (lane l: block blk_base + l), and
     // handed around with lane shuffles, so finding a key's page costs no memory access in the loop.
     const int bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
@@ -356,10 +356,11 @@ __global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const A
     // acc[m][r] = O^T[d = 16m + 4g + r][col]
     // ---- the waves' partial results meet in LDS: every wave leaves its own, then the blocks of 16 dimensions
     // are dealt to the waves, each of which adds the partial results up in the order of the waves
-    constexpr int NW = DB <= 10 ? 8 : 4;  // (what the launch bounds allow)
+    // (the number of waves is the kernel's own: with a count read at run time every step of the sums below was a
+    // branch and a wait of its own, 1.3 microseconds for what is now a few loads and one wait)
     __shared__ float sh_acc[NW][DB][LLMS_WAVE][4];
     __shared__ float sh_m[NW][16], sh_l[NW][16];
-    const int nw = blockDim.x / LLMS_WAVE;
+    constexpr int nw = NW;
 #pragma unroll
     for (int m = 0; m < DB; ++m)
         *reinterpret_cast<float4*>(sh_acc[wave][m][lane]) = make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
@@ -370,27 +371,24 @@ __global__ __launch_bounds__(DB <= 10 ? 512 : 256) void attn_mfma_kernel(const A
     __syncthreads();
     float m_tot = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < NW; ++w)
-        if (w < nw) m_tot = fmaxf(m_tot, sh_m[w][col]);
+    for (int w = 0; w < NW; ++w) m_tot = fmaxf(m_tot, sh_m[w][col]);
     const float m_safe = (m_tot == -INFINITY) ? 0.f : m_tot;
     float weight[NW], l_tot = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-        weight[w] = w < nw ? exp2_fast(sh_m[w][col] - m_safe) : 0.f;  // 0 for a wave that saw no key
-        if (w < nw) l_tot += sh_l[w][col] * weight[w];
+        weight[w] = exp2_fast(sh_m[w][col] - m_safe);  // 0 for a wave that saw no key
+        l_tot += sh_l[w][col] * weight[w];
     }
     const size_t item = ((size_t)(tok0 + c_tok) * a.n_heads + head) * a.num_splits + split;
     for (int m = wave; m < DB; m += nw) {
         float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
-            if (w < nw) {
-                const float4 p = *reinterpret_cast<const float4*>(sh_acc[w][m][lane]);
-                o.x += p.x * weight[w];
-                o.y += p.y * weight[w];
-                o.z += p.z * weight[w];
-                o.w += p.w * weight[w];
-            }
+            const float4 p = *reinterpret_cast<const float4*>(sh_acc[w][m][lane]);
+            o.x += p.x * weight[w];
+            o.y += p.y * weight[w];
+            o.z += p.z * weight[w];
+            o.w += p.w * weight[w];
         }
         if (!col_ok) continue;
         if (a.num_splits == 1) {
@@ -742,9 +740,10 @@ static int launch_prompt(int db, int cg, dim3 grid, bool paired, const AttnArgs&
 }
 
 static int launch_attn(int db, dim3 grid, int threads, const AttnArgs& a, hipStream_t stream) {
-#define ATT_CASE(N)                                             \
-    case N:                                                     \
-        attn_mfma_kernel<N><<<grid, threads, 0, stream>>>(a);   \
+#define ATT_CASE(N)                                                                                  \
+    case N:                                                                                          \
+        if (threads == 8 * LLMS_WAVE && N <= 10) attn_mfma_kernel<N, (N <= 10 ? 8 : 4)><<<grid, 8 * LLMS_WAVE, 0, stream>>>(a); \
+        else attn_mfma_kernel<N, 4><<<grid, 4 * LLMS_WAVE, 0, stream>>>(a);                          \
         break;
     switch (db) {
         ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
