@@ -17,9 +17,9 @@
 //     their operands straight from the cache (nothing goes through LDS on the way to the matrix instruction),
 //     and optionally to `num_splits` workgroups whose partial results a second kernel merges.
 //   attn_prompt_kernel (prompts): consecutive column groups of one request want the same keys and share
-//     each tile through LDS, one or two groups per wave; without a window, a block of late tokens and a block of
-//     early ones are paired, or (a short portion behind a long prefix) the keys of a block are shared out to
-//     `num_splits` workgroups.
+//     each tile through LDS, one or two groups per wave; without a window, each wave has a twin that takes every
+//     other tile for the same columns, or (a short portion behind a long prefix) the keys of a block are shared
+//     out to `num_splits` workgroups.
 // All merges run in a fixed order, so a token's result does not depend on the batch around it.
 //
 // Needs block_size % 8 == 0, head_dim % 16 == 0 and <= 256, 16-byte aligned rows.
@@ -101,61 +101,93 @@ __device__ __forceinline__ float column_sum(float x) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-// One tile of 32 keys for a wave's 16 columns: scores, online softmax, weighted values.
+// One tile of 32 keys for CG column groups of 16 columns that share the keys: scores, online softmax, weighted
+// values.
 //   kf[u][s]: key rows of score tile u (row i = key 8*(i/4) + 4u + i%4), k-step s;  vf[m]: the lane's 8 keys
 //   (jk .. jk+7) of value dimensions 16m + col, already zero where the key is outside the group's range;
-//   qf[s]: the lane's column of queries.  acc[m][r] = O^T[16m + 4g + r][col] and the running max (times log2 e)
-//   and sum of the column are updated in place.  MASKED = false: every key of the tile is visible to every
-//   column of the wave (the caller knows), which saves the comparisons.  The accumulators are rescaled only
-//   when some column's maximum grew: a factor of exactly 1 otherwise, so the result is the same.
+//   qf[cg][s]: the lane's column of queries.  acc[cg][m][r] = O^T[16m + 4g + r][col] and the running max (times
+//   log2 e) and sum of the column are updated in place.  MASKED = false: every key of the tile is visible to every
+//   column of the wave (the caller knows), which saves the comparisons.  The accumulators are rescaled only when
+//   some column's maximum grew: a factor of exactly 1 otherwise, so the result is the same.  The groups go through
+//   each stage side by side, not one group after the other: their chains (matrix product, maximum, exponentials,
+//   matrix product) do not depend on each other, and a wave that alternates between them waits less for each.
+template <int DB, int KS, bool MASKED, int CG>
+__device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (&m_run)[CG], float (&l_run)[CG],
+                                                   const uint4 (&kf)[2][KS], const uint4 (&vf)[DB], const uint4 (&qf)[CG][KS],
+                                                   int jk, const int (&lo_col)[CG], const int (&p_col)[CG], float scale_log2) {
+    f32x4 s_acc[CG][2];
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            s_acc[cg][u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; ++s)
+                s_acc[cg][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u][s]), as_bf16x8(qf[cg][s]), s_acc[cg][u], 0, 0, 0);
+        }
+    // the lane holds its column's scores for the keys jk .. jk+7; the other 24 keys sit in the 3 other lane groups
+    float sc[CG][8], m_new[CG], m_safe[CG];
+    bool grew = false;
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg) {
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            sc[cg][e] = s_acc[cg][e / 4][e % 4];
+            if (MASKED) {
+                const int key = jk + e;
+                if (!(key >= lo_col[cg] && key <= p_col[cg])) sc[cg][e] = -INFINITY;
+            }
+            tmax = fmaxf(tmax, sc[cg][e]);
+        }
+        tmax = column_max(tmax);
+        m_new[cg] = fmaxf(m_run[cg], tmax * scale_log2);  // (scale > 0)
+        m_safe[cg] = (MASKED && m_new[cg] == -INFINITY) ? 0.f : m_new[cg];
+        grew = grew || m_new[cg] > m_run[cg];
+    }
+    if (__builtin_amdgcn_ballot_w64(grew) != 0) {
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg) {
+            const float corr = exp2_fast(m_run[cg] - m_safe[cg]);  // 1 where the maximum stayed; 0 while the column has seen no key
+            l_run[cg] *= corr;
+#pragma unroll
+            for (int m = 0; m < DB; ++m)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[cg][m][r] *= corr;
+            m_run[cg] = m_new[cg];
+        }
+    }
+    uint4 pf[CG];
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg) {
+        float psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            sc[cg][e] = exp2_fast(fmaf(sc[cg][e], scale_log2, -m_safe[cg]));
+            psum += sc[cg][e];
+        }
+        l_run[cg] += column_sum(psum);
+        pf[cg] = make_uint4(pack_bf16(sc[cg][0], sc[cg][1]), pack_bf16(sc[cg][2], sc[cg][3]), pack_bf16(sc[cg][4], sc[cg][5]),
+                            pack_bf16(sc[cg][6], sc[cg][7]));
+    }
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+        for (int m = 0; m < DB; ++m)
+            acc[cg][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[m]), as_bf16x8(pf[cg]), acc[cg][m], 0, 0, 0);
+}
+
+// The same for one column group (decoding).
 template <int DB, int KS, bool MASKED>
 __device__ __forceinline__ void attend_tile(f32x4 (&acc)[DB], float& m_run, float& l_run, const uint4 (&kf)[2][KS],
                                             const uint4 (&vf)[DB], const uint4 (&qf)[KS], int jk, int lo_col, int p_col,
                                             float scale_log2) {
-    f32x4 s_acc[2];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        s_acc[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < KS; ++s)
-            s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u][s]), as_bf16x8(qf[s]), s_acc[u], 0, 0, 0);
-    }
-    // the lane holds its column's scores for the keys jk .. jk+7; the other 24 keys sit in the 3 other lane groups
-    float sc[8];
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        sc[e] = s_acc[e / 4][e % 4];
-        if (MASKED) {
-            const int key = jk + e;
-            if (!(key >= lo_col && key <= p_col)) sc[e] = -INFINITY;
-        }
-        tmax = fmaxf(tmax, sc[e]);
-    }
-    tmax = column_max(tmax);
-    const float m_new = fmaxf(m_run, tmax * scale_log2);  // (scale > 0)
-    const float m_safe = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
-    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-        const float corr = exp2_fast(m_run - m_safe);  // 0 while the column has seen no key
-        l_run *= corr;
-#pragma unroll
-        for (int m = 0; m < DB; ++m)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[m][r] *= corr;
-        m_run = m_new;
-    }
-    float psum = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        sc[e] = exp2_fast(fmaf(sc[e], scale_log2, -m_safe));
-        psum += sc[e];
-    }
-    l_run += column_sum(psum);
-    const uint4 pf = make_uint4(pack_bf16(sc[0], sc[1]), pack_bf16(sc[2], sc[3]), pack_bf16(sc[4], sc[5]),
-                                pack_bf16(sc[6], sc[7]));
-#pragma unroll
-    for (int m = 0; m < DB; ++m)
-        acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vf[m]), as_bf16x8(pf), acc[m], 0, 0, 0);
+    float m1[1] = {m_run}, l1[1] = {l_run};
+    const int lo1[1] = {lo_col}, p1[1] = {p_col};
+    attend_tile_groups<DB, KS, MASKED, 1>(reinterpret_cast<f32x4 (&)[1][DB]>(acc), m1, l1, kf, vf,
+                                          reinterpret_cast<const uint4 (&)[1][KS]>(qf), jk, lo1, p1, scale_log2);
+    m_run = m1[0];
+    l_run = l1[0];
 }
 
 // 8 bytes to or from memory past the caches that other XCDs do not see (an L2 belongs to one XCD): what one
@@ -436,7 +468,7 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
 }
 
 // Prompt portions: a block of WB * CG consecutive column groups of one request and KV head per workgroup, CG per
-// wave.  The WB waves walk the same keys, so each tile of 32 keys is fetched once per workgroup: every thread brings
+// wave.  The waves walk the same keys, so each tile of 32 keys is fetched once per workgroup: every thread brings
 // 16-byte pieces of the key rows and of the (page-transposed) value rows into LDS, double-buffered, and the waves
 // read their matrix operands from there.  Key rows are stored in the order the score product wants them (row
 // 16u + i holds key 8*(i/4) + 4u + i%4, padded by one chunk per row against bank conflicts); values keep their
@@ -444,61 +476,57 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
 // instead of 16: with head_dim 128 the LDS reads were what the loop waited for (twice the matrix instructions'
 // time), with head_dim 64 it was instruction issue, of which the reads and the loop's own work are a third.
 //
-// PAIRED (no window, and enough tokens that the paired launch still has a workgroup for every CU): the causal
-// triangle gives the last tokens of a prompt the most keys, and a workgroup with
-// few keys leaves its CU idle while others still run.  A workgroup then has 2 WB waves and takes two blocks of
-// tokens, number x from the front and number x from the back: the first WB waves the late block, the others the early
-// block, which sees a prefix of the same keys, stops multiplying when it has passed its own position, and
-// loads the tiles for all.  Every workgroup of a request then has the same work.
-template <int DB, bool PAIRED, int CG, int WB>
-__global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt_kernel(const AttnArgs a) {
+// TWIN (no window, no splits): the workgroup has 2 WB waves and a round of the loop brings two tiles; wave w and
+// its twin w + WB own the same columns, the one takes the first tile of every round, the other the second, and
+// the twin's sums are merged into the other's through LDS at the end, first tile first.  The causal triangle gives
+// the last tokens of a prompt the most keys: the chain of dependent rounds of the longest block is halved this way,
+// a SIMD always has two waves to switch between, and the blocks are handed out from the longest to the shortest
+// (blockIdx.y counts from the end of the prompt), so that a CU that was given a long one takes a short one next.
+template <int DB, bool TWIN, int CG, int WB>
+__global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
     constexpr int KS = (D + 31) / 32;
     constexpr int KCH = D / 8;          // 16-byte chunks of a key row
     constexpr int KROW = KCH + 1;       // padded row stride in chunks
-    constexpr int PIECES = 4 * D;       // chunks of the key tile (32 x KCH) = chunks of the value tile (D x 4)
-    constexpr int LT = WB * LLMS_WAVE;  // threads that bring the tiles in
-    constexpr int PER_THREAD = (PIECES + LT - 1) / LT;
-    __shared__ uint4 k_lds[2][32 * KROW];
-    __shared__ uint4 v_lds[2][D * 4];
+    constexpr int TW = TWIN ? 2 : 1;    // tiles per round of the loop
+    constexpr int PIECES = 4 * D;       // chunks of a key tile (32 x KCH) = chunks of a value tile (D x 4)
+    constexpr int LT = TW * WB * LLMS_WAVE;  // threads, all of which bring the tiles in
+    constexpr int PER_THREAD = (TW * PIECES + LT - 1) / LT;
+    constexpr int K_TILE = 32 * KROW, V_TILE = D * 4;  // chunks of a tile in LDS
+    // two buffers of TW key tiles, then two of TW value tiles; at the end the twins' sums pass through the same memory
+    __shared__ uint4 lds_raw[2 * TW * (K_TILE + V_TILE)];
+    uint4* const k_lds = lds_raw;                     // [buffer][tile of the round][row][chunk]
+    uint4* const v_lds = lds_raw + 2 * TW * K_TILE;   // [buffer][tile of the round][dimension][4 chunks of 8 keys]
     const int tid = threadIdx.x, wave = tid / LLMS_WAVE, lane = tid % LLMS_WAVE;
     const int col = lane % 16, g = lane / 16;
+    const int twin = __builtin_amdgcn_readfirstlane(wave / WB);  // which tile of a round this wave takes
 
     const int G = a.n_heads / a.n_kv_heads;
     const int HG = G < 16 ? G : 16, TPG = 16 / HG, HB = (G + HG - 1) / HG;
-    const int kvh = blockIdx.y / HB, hb = blockIdx.y % HB;
+    const int head_block = TWIN ? blockIdx.x : blockIdx.y;
+    const int kvh = head_block / HB, hb = head_block % HB;
     const int b = a.seq_begin + blockIdx.z;
     const int tok0 = a.cu_seqlens[b], n_new = a.cu_seqlens[b + 1] - tok0;
     const int ctx = a.context_lens[b];
     // (asked for together with the lengths: one trip to memory earlier than where the block table is first needed)
     const int table_row = a.table_rows ? a.table_rows[b] : b;
-    // wg_first: first token (within the request's new tokens) of the block whose keys the workgroup walks;
-    // my_first: of the block this wave works for
-    int wg_first, my_first;
-    bool wave_on = true;
     const int BLK = WB * CG * TPG;  // tokens of a block: WB waves with CG column groups each
-    if (PAIRED) {
+    int wg_first;                   // first token (within the request's new tokens) of the workgroup's block
+    if (TWIN) {
         const int blocks = (n_new + BLK - 1) / BLK;
-        const int late = blocks - 1 - (int)blockIdx.x, early = blockIdx.x;
-        if (late < early || ctx <= 0) return;
-        wg_first = late * BLK;
-        my_first = (wave < WB ? late : early) * BLK;
-        wave_on = wave < WB || early != late;  // (the middle block of an odd number is its own partner)
+        if ((int)blockIdx.y >= blocks || ctx <= 0) return;
+        wg_first = (blocks - 1 - (int)blockIdx.y) * BLK;
     } else {
-        wg_first = my_first = ((int)blockIdx.x / a.num_splits) * BLK;
+        wg_first = ((int)blockIdx.x / a.num_splits) * BLK;
         if (wg_first >= n_new || ctx <= 0) return;
     }
-    // Without pairing the keys of a block may be shared out to num_splits workgroups (blockIdx.x % num_splits), whose
+    // Without twins the keys of a block may be shared out to num_splits workgroups (blockIdx.x % num_splits), whose
     // partial results attn_merge adds up: a short portion with a long prefix has few blocks and many keys.
-    const int n_splits = PAIRED ? 1 : a.num_splits, split = PAIRED ? 0 : (int)blockIdx.x % a.num_splits;
-    // The tiles are brought in by the waves that have time for it: those of the early block, which stop
-    // multiplying half way on average (without pairing, by everyone).
-    const bool loader = !PAIRED || tid >= LT;
-    const int ltid = PAIRED ? tid - LT : tid;
+    const int n_splits = TWIN ? 1 : a.num_splits, split = TWIN ? 0 : (int)blockIdx.x % a.num_splits;
 
     // this wave's CG column groups: consecutive tokens, the same heads
-    const int w_first = my_first + (wave % WB) * CG * TPG;
-    wave_on = wave_on && w_first < n_new;
+    const int w_first = wg_first + (wave % WB) * CG * TPG;
+    const bool wave_on = w_first < n_new;
     const int c_head_in = hb * HG + col % HG, head = kvh * G + c_head_in;
     int c_tok[CG], p_col[CG], lo_col[CG];
     bool col_ok[CG];
@@ -514,7 +542,7 @@ __global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt
     const int p_min = ctx - n_new + wg_first;
     const int lo_min = (a.window > 0 && p_min - a.window + 1 > 0) ? p_min - a.window + 1 : 0;
     const int j_begin = lo_min & ~31;
-    const int n_tiles = (p_max - j_begin) / 32 + 1;
+    const int n_rounds = ((p_max - j_begin) / 32 + TW) / TW;  // of TW tiles each
 
     const uint4 zero = make_uint4(0, 0, 0, 0);
     uint4 qf[CG][KS];
@@ -545,97 +573,153 @@ __global__ __launch_bounds__((PAIRED ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt
     const int w_last = min(w_first + CG * TPG, n_new) - 1;
     const int w_pmin = ctx - n_new + w_first, w_pmax = ctx - n_new + w_last;
     const int w_lo_max = (a.window > 0 && w_pmax - a.window + 1 > 0) ? w_pmax - a.window + 1 : 0;
-    const int bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
-    auto block_of = [&](int key) { return bs_shift >= 0 ? key >> bs_shift : key / a.block_size; };
-    const int last_blk = block_of(p_max);
-    int blk_base = 0, pages_reg = 0;
-    auto load_pages = [&](int base) {
-        blk_base = base;
-        pages_reg = table[min(base + lane, last_blk)];
-    };
+    // key / block_size by one multiply with ceil(2^32 / block_size): exact below 2^32 / block_size keys (the
+    // entry point refuses longer block tables)
+    const uint32_t bs_magic = 0xFFFFFFFFu / (uint32_t)a.block_size + 1u;
+    auto block_of = [&](int key) { return (int)__umulhi((uint32_t)key, bs_magic); };
 
-    // this thread's pieces of a tile: key piece c -> key c / KCH, chunk c % KCH; value piece c -> dimension c / 4,
-    // keys 8*(c % 4) .. +7.  Addresses are clamped to the last key of the workgroup (which exists); value pieces
-    // are zeroed outside [lo_min, p_max] on their way into LDS (not earlier: that would wait for the load).
+    // this thread's pieces of a round: piece c belongs to tile c / PIECES of the round; within the tile, key piece
+    // c' -> key c' / KCH, chunk c' % KCH; value piece c' -> dimension c' / 4, keys 8*(c' % 4) .. +7.  Keys are
+    // clamped to the last key of the workgroup (which exists), so every round can be asked for, also one past the
+    // last; value pieces are zeroed outside [lo_min, p_max] on their way into LDS (not earlier: that would wait
+    // for the load).  The page of a piece is read from the block table a round before the piece itself is asked
+    // for, and that a round before it goes into LDS: three rounds in flight, nothing waited for inside the loop.
     uint4 kreg[PER_THREAD], vreg[PER_THREAD];
-    auto load_tile = [&](int j0) {
-        const int blk_first = block_of(j0);
-        if (blk_first < blk_base || block_of(min(j0 + 31, p_max)) >= blk_base + LLMS_WAVE) load_pages(blk_first);
+    int k_page[PER_THREAD], v_page[PER_THREAD];
+    auto k_key_of = [&](int i, int j0) {
+        const int c_all = tid + LT * i;
+        return c_all < TW * PIECES ? min(j0 + 32 * (c_all / PIECES) + (c_all % PIECES) / KCH, p_max) : p_max;
+    };
+    auto v_key_of = [&](int i, int j0) {  // the first of the piece's 8 keys
+        const int c_all = tid + LT * i;
+        return c_all < TW * PIECES ? min(j0 + 32 * (c_all / PIECES) + 8 * (c_all % 4), p_max & ~7) : p_max & ~7;
+    };
+    auto ask_pages = [&](int j0) {
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
-            const int c = ltid + LT * i;
-            const bool piece_ok = c < PIECES;  // (D < 64: the upper threads have no piece)
-            {
-                const int key = min(j0 + (piece_ok ? c / KCH : 0), p_max), ch = piece_ok ? c % KCH : 0;
-                const int blk = block_of(key);
-                const int page = __shfl(pages_reg, blk - blk_base, LLMS_WAVE);
-                kreg[i] = *reinterpret_cast<const uint4*>(page_ptr(k_base, page, page_stride) +
-                                                           (uint32_t)((key - blk * a.block_size) * D + 8 * ch));
-            }
-            {
-                const int d = piece_ok ? c / 4 : 0, kc = piece_ok ? c % 4 : 0;
-                const int jk = j0 + 8 * kc, jc = min(jk, p_max & ~7);
-                const int blk = block_of(jc);
-                const int page = __shfl(pages_reg, blk - blk_base, LLMS_WAVE);
-                vreg[i] = *reinterpret_cast<const uint4*>(page_ptr(v_base, page, page_stride) +
-                                                           (uint32_t)(d * a.block_size + jc - blk * a.block_size));
-            }
+            k_page[i] = table[block_of(k_key_of(i, j0))];
+            v_page[i] = table[block_of(v_key_of(i, j0))];
         }
     };
-    auto store_tile = [&](int buf, int j0) {
-        const bool inside = j0 >= lo_min && j0 + 31 <= p_max;  // (uniform)
+    auto load_round = [&](int j0) {  // after ask_pages(j0)
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
-            const int c = ltid + LT * i;
-            if (c < PIECES) {
+            const int c_all = tid + LT * i;
+            const int c = c_all < TW * PIECES ? c_all % PIECES : 0;  // (D < 64: the upper threads have no piece)
+            const int key = k_key_of(i, j0), jc = v_key_of(i, j0);
+            kreg[i] = *reinterpret_cast<const uint4*>(page_ptr(k_base, k_page[i], page_stride) +
+                                                       (uint32_t)((key - block_of(key) * a.block_size) * D + 8 * (c % KCH)));
+            vreg[i] = *reinterpret_cast<const uint4*>(page_ptr(v_base, v_page[i], page_stride) +
+                                                       (uint32_t)((c / 4) * a.block_size + jc - block_of(jc) * a.block_size));
+        }
+    };
+    auto store_round = [&](int buf, int j0) {
+        const bool inside = j0 >= lo_min && j0 + 32 * TW - 1 <= p_max;  // (uniform)
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) {
+            const int c_all = tid + LT * i;
+            if (c_all < TW * PIECES) {
+                const int c = c_all % PIECES, tile = c_all / PIECES;
                 if (!inside) {
-                    const int jk = j0 + 8 * (c % 4);
+                    const int jk = j0 + 32 * tile + 8 * (c % 4);
                     vreg[i] = keep_elements(vreg[i], lo_min - jk, p_max + 1 - jk);
                 }
                 const int kl = c / KCH, ch = c % KCH;                    // key kl = 8a + 4u + b2 of the tile
                 const int row = ((kl >> 2) & 1) * 16 + (kl >> 3) * 4 + (kl & 3);  // -> row 16u + 4a + b2
-                k_lds[buf][row * KROW + ch] = kreg[i];
-                v_lds[buf][c] = vreg[i];                                  // [dimension][4 chunks of 8 keys]
+                k_lds[(buf * TW + tile) * K_TILE + row * KROW + ch] = kreg[i];
+                v_lds[(buf * TW + tile) * V_TILE + c] = vreg[i];
             }
         }
     };
 
-    const int per_split = (n_tiles + n_splits - 1) / n_splits;
-    const int t_lo = split * per_split, t_hi = min(n_tiles, t_lo + per_split);  // this workgroup's tiles (maybe none)
-    if (loader && t_lo < t_hi) {
-        load_pages(block_of(j_begin + 32 * t_lo));
-        load_tile(j_begin + 32 * t_lo);
-        store_tile(0, j_begin + 32 * t_lo);
-        if (t_lo + 1 < t_hi) load_tile(j_begin + 32 * (t_lo + 1));
-    }
+    const int per_split = (n_rounds + n_splits - 1) / n_splits;
+    const int r_lo = split * per_split, r_hi = min(n_rounds, r_lo + per_split);  // this workgroup's rounds (maybe none)
+    auto first_key = [&](int r) { return j_begin + 32 * TW * r; };
+    ask_pages(first_key(r_lo));
+    load_round(first_key(r_lo));
+    ask_pages(first_key(r_lo + 1));
+    store_round(0, first_key(r_lo));
+    // The queries have arrived by now (they were asked for before the first round, which has just been stored).
+    // Saying so here, outside the loop, keeps the wait for them out of it: inside, a wait for loads from memory
+    // would also wait for the round that is being fetched ahead.
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            asm volatile("" : "+v"(qf[cg][s].x), "+v"(qf[cg][s].y), "+v"(qf[cg][s].z), "+v"(qf[cg][s].w));
+    load_round(first_key(r_lo + 1));
+    ask_pages(first_key(r_lo + 2));
     __syncthreads();
-    for (int t = t_lo; t < t_hi; ++t) {
-        const int buf = (t - t_lo) & 1, j0 = j_begin + 32 * t;
-        if (wave_on && j0 <= w_pmax) {  // (a tile beyond the wave's last position adds nothing)
+    for (int r = r_lo; r < r_hi; ++r) {
+        const int buf = (r - r_lo) & 1, j0 = j_begin + 32 * (TW * r + twin);  // this wave's tile of the round
+        const bool busy = wave_on && j0 <= w_pmax;  // (a tile beyond the wave's last position adds nothing)
         uint4 kf[2][KS], vf[DB];
+        if (busy) {
+            const uint4* kt = k_lds + (buf * TW + twin) * K_TILE;
+            const uint4* vt = v_lds + (buf * TW + twin) * V_TILE;
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int s = 0; s < KS; ++s) {
-                const int ch = 4 * s + g;
-                kf[u][s] = k_lds[buf][(16 * u + col) * KROW + (ch < KCH ? ch : 0)];  // (beyond head_dim the queries are zero)
-            }
+                for (int s = 0; s < KS; ++s) {
+                    const int ch = 4 * s + g;
+                    kf[u][s] = kt[(16 * u + col) * KROW + (ch < KCH ? ch : 0)];  // (beyond head_dim the queries are zero)
+                }
 #pragma unroll
-        for (int m = 0; m < DB; ++m) vf[m] = v_lds[buf][(16 * m + col) * 4 + g];
-        const bool all_seen = j0 >= w_lo_max && j0 + 31 <= w_pmin;  // (uniform over the wave; columns without a token are discarded)
-#pragma unroll
-        for (int cg = 0; cg < CG; ++cg) {  // the same keys and values for each of the wave's column groups
-            if (all_seen)
-                attend_tile<DB, KS, false>(acc[cg], m_run[cg], l_run[cg], kf, vf, qf[cg], j0 + 8 * g, lo_col[cg], p_col[cg], scale_log2);
-            else
-                attend_tile<DB, KS, true>(acc[cg], m_run[cg], l_run[cg], kf, vf, qf[cg], j0 + 8 * g, lo_col[cg], p_col[cg], scale_log2);
+            for (int m = 0; m < DB; ++m) vf[m] = vt[(16 * m + col) * 4 + g];
         }
+        // the next round into the other buffer (last read before the previous barrier), the round after that asked
+        // for, and the pages of the one after that: by the twins while the fragments are on their way from LDS, by
+        // the others after their tile, so that the two waves of a SIMD are not at the same stage at the same time
+        // (one multiplies while the other computes exponentials)
+        auto fetch_ahead = [&]() {
+            if (r + 1 < r_hi) store_round(buf ^ 1, first_key(r + 1));
+            load_round(first_key(r + 2));
+            ask_pages(first_key(r + 3));
+        };
+        if (!TWIN || twin == 1) fetch_ahead();
+        if (busy) {
+            const bool all_seen = j0 >= w_lo_max && j0 + 31 <= w_pmin;  // (uniform over the wave; columns without a token are discarded)
+            // the same keys and values for each of the wave's column groups
+            if (all_seen) attend_tile_groups<DB, KS, false, CG>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
+            else attend_tile_groups<DB, KS, true, CG>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
         }
-        if (loader && t + 1 < t_hi) {
-            store_tile(buf ^ 1, j0 + 32);  // last read two tiles ago, before the previous barrier
-            if (t + 2 < t_hi) load_tile(j_begin + 32 * (t + 2));
-        }
+        if (TWIN && twin == 0) fetch_ahead();
         __syncthreads();
+    }
+    if constexpr (TWIN) {
+        // The twin's share (second tile of every round) joins the first wave's, one column group at a time:
+        // [item][twin wave][lane] floats in the memory of the tiles, which nobody reads any more.
+        float* share = reinterpret_cast<float*>(lds_raw);
+        constexpr int ITEMS = 4 * DB + 2;
+        const int slot = (wave % WB) * LLMS_WAVE + lane;
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg) {
+            if (cg > 0) __syncthreads();  // (the group before has been read)
+            if (twin == 1) {
+                share[slot] = m_run[cg];
+                share[WB * LLMS_WAVE + slot] = l_run[cg];
+#pragma unroll
+                for (int m = 0; m < DB; ++m)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) share[(2 + 4 * m + r) * WB * LLMS_WAVE + slot] = acc[cg][m][r];
+            }
+            __syncthreads();
+            if (twin == 0) {
+                const float m_b = share[slot], l_b = share[WB * LLMS_WAVE + slot];
+                const float m_tot = fmaxf(m_run[cg], m_b);
+                const float w_a = m_run[cg] == -INFINITY ? 0.f : exp2_fast(m_run[cg] - m_tot);
+                const float w_b = m_b == -INFINITY ? 0.f : exp2_fast(m_b - m_tot);
+                l_run[cg] = l_run[cg] * w_a + l_b * w_b;
+                m_run[cg] = m_tot;
+#pragma unroll
+                for (int m = 0; m < DB; ++m)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        acc[cg][m][r] = acc[cg][m][r] * w_a + share[(2 + 4 * m + r) * WB * LLMS_WAVE + slot] * w_b;
+            }
+        }
+        static_assert(ITEMS * WB * LLMS_WAVE * sizeof(float) <= sizeof(lds_raw), "the twins' shares must fit the tiles' memory");
+        if (twin == 1) return;
     }
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg) {
@@ -710,8 +794,8 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(bf16* __restrict__ out,
 #define PROMPT_FULL_CHIP 256  // workgroups below which one column group per wave is kept
 
 template <int DB, int CG>
-static void launch_prompt_cg(dim3 grid, bool paired, const AttnArgs& a, hipStream_t stream) {
-    if (paired) attn_prompt_kernel<DB, true, CG, PROMPT_WB><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
+static void launch_prompt_cg(dim3 grid, bool twin, const AttnArgs& a, hipStream_t stream) {
+    if (twin) attn_prompt_kernel<DB, true, CG, PROMPT_WB><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
     else attn_prompt_kernel<DB, false, CG, PROMPT_WB><<<grid, PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
 }
 
@@ -723,11 +807,11 @@ static void launch_merge(void* out, int out_stride, const float* ws_o, const flo
         (bf16*)out, out_stride, ws_o, ws_ml, token_begin, n_heads, head_dim, num_splits);
 }
 
-static int launch_prompt(int db, int cg, dim3 grid, bool paired, const AttnArgs& a, hipStream_t stream) {
+static int launch_prompt(int db, int cg, dim3 grid, bool twin, const AttnArgs& a, hipStream_t stream) {
 #define ATT_CASE(N)                                                                       \
     case N:                                                                               \
-        if (cg == 2 && PROMPT_CG_MAX(N) == 2) launch_prompt_cg<N, PROMPT_CG_MAX(N)>(grid, paired, a, stream); \
-        else launch_prompt_cg<N, 1>(grid, paired, a, stream);                             \
+        if (cg == 2 && PROMPT_CG_MAX(N) == 2) launch_prompt_cg<N, PROMPT_CG_MAX(N)>(grid, twin, a, stream); \
+        else launch_prompt_cg<N, 1>(grid, twin, a, stream);                             \
         break;
     switch (db) {
         ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
@@ -810,23 +894,25 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
             launch_merge(out, out_stride, ws_o, ws_ml, token_begin, n_tokens, n_heads, head_dim, num_splits, stream);
         }
     } else {
-        bool paired = window == 0 && head_dim <= 192 && num_splits == 1;  // early and late blocks of tokens in one workgroup
-        // (8 waves of wider heads would not fit the registers)
+        // twins (8 waves, two tiles a round) where a workgroup per CU is left that way; wider heads would not fit
+        // the registers of 8 waves, a window or splits have their own arrangement
+        LLMS_REQUIRE((unsigned long long)max_blocks * block_size * block_size <= 0xFFFFFFFFull,
+                     "attention_mfma: block table too long for this page size (keys * block_size must stay below 2^32)");
+        bool twin = window == 0 && head_dim <= 192 && num_splits == 1;
         auto grid_for = [&](int cg) {
             const int per_block = PROMPT_WB * cg;  // column groups of a block of tokens
-            dim3 grid((groups + per_block - 1) / per_block * num_splits, n_kv_heads * HB, n_seqs);
-            if (paired) grid.x = (grid.x + 1) / 2;
-            return grid;
+            return dim3((groups + per_block - 1) / per_block * num_splits, n_kv_heads * HB, n_seqs);
         };
         auto workgroups = [](dim3 g) { return (long long)g.x * g.y * g.z; };
         int cg = PROMPT_CG_MAX(head_dim / 16);
         dim3 grid = grid_for(cg);
         if (cg == 2 && workgroups(grid) < PROMPT_FULL_CHIP) grid = grid_for(cg = 1);
-        if (paired && workgroups(grid) < PROMPT_FULL_CHIP) {  // a short portion: workgroups for more CUs matter more
-            paired = false;                                    // than equal work for each
-            grid = grid_for(cg);
+        if (twin && workgroups(grid) < PROMPT_FULL_CHIP) twin = false;  // a short portion: workgroups for more CUs matter more
+        if (twin) {  // heads in x, blocks of tokens in y from the last one: the order in which workgroups are handed out
+            LLMS_REQUIRE(grid.x <= 65535, "attention_mfma: too many tokens per request for one launch");
+            grid = dim3(grid.y, grid.x, grid.z);
         }
-        if (int e = launch_prompt(head_dim / 16, cg, grid, paired, a, stream)) return e;
+        if (int e = launch_prompt(head_dim / 16, cg, grid, twin, a, stream)) return e;
         if (num_splits > 1) {
             hipError_t e1 = hipGetLastError();
             if (e1 != hipSuccess) {
