@@ -85,12 +85,20 @@ __device__ __forceinline__ const bf16* page_ptr(const bf16* base, int page, uint
 // (v_permlane32_swap, v_permlane16_swap: the upper half / the odd rows of 16 lanes of one operand change
 // places with the lower half / the even rows of the other), which stay in the vector unit; a lane shuffle
 // would go through LDS four times per tile.
+// (the maximum as the instruction itself: fmaxf would first pass each swapped value, whose origin the compiler
+// cannot see, through an instruction of its own that quiets a signalling NaN, four more per tile and column group)
+__device__ __forceinline__ float max_of_swapped(unsigned a, unsigned b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
 __device__ __forceinline__ float column_max(float x) {
     const unsigned xi = __float_as_uint(x);
     const auto a = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
-    const unsigned mi = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+    const unsigned mi = __float_as_uint(max_of_swapped(a[0], a[1]));
     const auto b = __builtin_amdgcn_permlane16_swap(mi, mi, false, false);
-    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+    return max_of_swapped(b[0], b[1]);
 }
 
 __device__ __forceinline__ float column_sum(float x) {
@@ -111,6 +119,7 @@ __device__ __forceinline__ float column_sum(float x) {
 //   some column's maximum grew: a factor of exactly 1 otherwise, so the result is the same.  The groups go through
 //   each stage side by side, not one group after the other: their chains (matrix product, maximum, exponentials,
 //   matrix product) do not depend on each other, and a wave that alternates between them waits less for each.
+#define STALE_MAX 8.f  // by how much (in powers of two) a column's maximum may pass the reference before a rescale
 template <int DB, int KS, bool MASKED, int CG>
 __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (&m_run)[CG], float (&l_run)[CG],
                                                    const uint4 (&kf)[2][KS], const uint4 (&vf)[DB], const uint4 (&qf)[CG][KS],
@@ -142,13 +151,17 @@ __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (
         }
         tmax = column_max(tmax);
         m_new[cg] = fmaxf(m_run[cg], tmax * scale_log2);  // (scale > 0)
-        m_safe[cg] = (MASKED && m_new[cg] == -INFINITY) ? 0.f : m_new[cg];
-        grew = grew || m_new[cg] > m_run[cg];
+        grew = grew || m_new[cg] > m_run[cg] + STALE_MAX;   // (also a column's first key: -inf + x = -inf)
     }
+    // m_run is the reference the weights are taken against, not necessarily the maximum: while no column's
+    // maximum has passed its reference by more than STALE_MAX (a factor of 2^STALE_MAX in the weights and sums,
+    // far inside the range of 32-bit and bfloat16 numbers, and the same relative precision), nothing is rescaled.
+    // The quotient at the end does not depend on the reference.
     if (__builtin_amdgcn_ballot_w64(grew) != 0) {
 #pragma unroll
         for (int cg = 0; cg < CG; ++cg) {
-            const float corr = exp2_fast(m_run[cg] - m_safe[cg]);  // 1 where the maximum stayed; 0 while the column has seen no key
+            const float m_ref = (MASKED && m_new[cg] == -INFINITY) ? 0.f : m_new[cg];
+            const float corr = exp2_fast(m_run[cg] - m_ref);  // 1 where the maximum stayed; 0 while the column has seen no key
             l_run[cg] *= corr;
 #pragma unroll
             for (int m = 0; m < DB; ++m)
@@ -157,14 +170,16 @@ __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (
             m_run[cg] = m_new[cg];
         }
     }
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg) m_safe[cg] = (MASKED && m_run[cg] == -INFINITY) ? 0.f : m_run[cg];
     uint4 pf[CG];
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg) {
-        float psum = 0.f;
+        float psum;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             sc[cg][e] = exp2_fast(fmaf(sc[cg][e], scale_log2, -m_safe[cg]));
-            psum += sc[cg][e];
+            psum = e == 0 ? sc[cg][0] : psum + sc[cg][e];
         }
         l_run[cg] += column_sum(psum);
         pf[cg] = make_uint4(pack_bf16(sc[cg][0], sc[cg][1]), pack_bf16(sc[cg][2], sc[cg][3]), pack_bf16(sc[cg][4], sc[cg][5]),
@@ -489,9 +504,6 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt_k
     constexpr int KCH = D / 8;          // 16-byte chunks of a key row
     constexpr int KROW = KCH + 1;       // padded row stride in chunks
     constexpr int TW = TWIN ? 2 : 1;    // tiles per round of the loop
-    constexpr int PIECES = 4 * D;       // chunks of a key tile (32 x KCH) = chunks of a value tile (D x 4)
-    constexpr int LT = TW * WB * LLMS_WAVE;  // threads, all of which bring the tiles in
-    constexpr int PER_THREAD = (TW * PIECES + LT - 1) / LT;
     constexpr int K_TILE = 32 * KROW, V_TILE = D * 4;  // chunks of a tile in LDS
     // two buffers of TW key tiles, then two of TW value tiles; at the end the twins' sums pass through the same memory
     __shared__ uint4 lds_raw[2 * TW * (K_TILE + V_TILE)];
@@ -578,56 +590,51 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt_k
     const uint32_t bs_magic = 0xFFFFFFFFu / (uint32_t)a.block_size + 1u;
     auto block_of = [&](int key) { return (int)__umulhi((uint32_t)key, bs_magic); };
 
-    // this thread's pieces of a round: piece c belongs to tile c / PIECES of the round; within the tile, key piece
-    // c' -> key c' / KCH, chunk c' % KCH; value piece c' -> dimension c' / 4, keys 8*(c' % 4) .. +7.  Keys are
-    // clamped to the last key of the workgroup (which exists), so every round can be asked for, also one past the
-    // last; value pieces are zeroed outside [lo_min, p_max] on their way into LDS (not earlier: that would wait
-    // for the load).  The page of a piece is read from the block table a round before the piece itself is asked
-    // for, and that a round before it goes into LDS: three rounds in flight, nothing waited for inside the loop.
-    uint4 kreg[PER_THREAD], vreg[PER_THREAD];
-    int k_page[PER_THREAD], v_page[PER_THREAD];
-    auto k_key_of = [&](int i, int j0) {
-        const int c_all = tid + LT * i;
-        return c_all < TW * PIECES ? min(j0 + 32 * (c_all / PIECES) + (c_all % PIECES) / KCH, p_max) : p_max;
-    };
-    auto v_key_of = [&](int i, int j0) {  // the first of the piece's 8 keys
-        const int c_all = tid + LT * i;
-        return c_all < TW * PIECES ? min(j0 + 32 * (c_all / PIECES) + 8 * (c_all % 4), p_max & ~7) : p_max & ~7;
-    };
-    auto ask_pages = [&](int j0) {
-#pragma unroll
-        for (int i = 0; i < PER_THREAD; ++i) {
-            k_page[i] = table[block_of(k_key_of(i, j0))];
-            v_page[i] = table[block_of(v_key_of(i, j0))];
-        }
-    };
+    // A round is 4 TW groups of 8 consecutive keys, one per wave: inside a page the key rows of a group are one
+    // contiguous piece of 16 D bytes, and its values are 16 bytes per dimension, so everything a wave asks for in a
+    // round lies in one page.  The page, the group's place in it and the two base addresses are therefore the same
+    // for all lanes and are worked out by the scalar unit; a lane adds its constant offset.  Groups are clamped to
+    // the one that holds the workgroup's last key (which exists), so every round can be asked for, also one past
+    // the last: key rows past the last key may hold anything (their scores are masked), values outside
+    // [lo_min, p_max] are zeroed on their way into LDS (not earlier: that would wait for the load).  The page is
+    // read from the block table a round before the group is asked for, and that a round before it goes into LDS:
+    // three rounds in flight, nothing waited for inside the loop.
+    static_assert(WB == 4, "a wave per group of 8 keys: 4 to a tile");
+    constexpr int PER_LANE = (D + LLMS_WAVE - 1) / LLMS_WAVE;  // 16-byte pieces of a group per lane (keys and values alike)
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    uint4 kreg[PER_LANE], vreg[PER_LANE];
+    int page_ahead = 0;
+    auto group_key_of = [&](int j0) { return min(j0 + 8 * wave_s, p_max & ~7); };  // first key of this wave's group
+    // (the block table does not change while the kernel runs: read as constant memory, which is what lets the
+    // scalar unit fetch it; as an ordinary load it would come back through the vector memory queue, and moving it
+    // to a scalar register would wait for the key and value pieces queued before it)
+    typedef const int __attribute__((address_space(4))) * ConstInts;
+    const ConstInts table_c = (ConstInts)(uintptr_t)table;
+    auto ask_pages = [&](int j0) { page_ahead = table_c[block_of(group_key_of(j0))]; };
     auto load_round = [&](int j0) {  // after ask_pages(j0)
+        const int jg = group_key_of(j0), in_page = jg - block_of(jg) * a.block_size;
+        const bf16* kg = page_ptr(k_base, page_ahead, page_stride) + (uint32_t)(in_page * D);
+        const bf16* vg = page_ptr(v_base, page_ahead, page_stride) + (uint32_t)in_page;
 #pragma unroll
-        for (int i = 0; i < PER_THREAD; ++i) {
-            const int c_all = tid + LT * i;
-            const int c = c_all < TW * PIECES ? c_all % PIECES : 0;  // (D < 64: the upper threads have no piece)
-            const int key = k_key_of(i, j0), jc = v_key_of(i, j0);
-            kreg[i] = *reinterpret_cast<const uint4*>(page_ptr(k_base, k_page[i], page_stride) +
-                                                       (uint32_t)((key - block_of(key) * a.block_size) * D + 8 * (c % KCH)));
-            vreg[i] = *reinterpret_cast<const uint4*>(page_ptr(v_base, v_page[i], page_stride) +
-                                                       (uint32_t)((c / 4) * a.block_size + jc - block_of(jc) * a.block_size));
+        for (int i = 0; i < PER_LANE; ++i) {
+            const int p = min(lane + LLMS_WAVE * i, D - 1);  // (D % 64 != 0: the upper lanes repeat the last piece)
+            kreg[i] = *reinterpret_cast<const uint4*>(kg + 8 * p);
+            vreg[i] = *reinterpret_cast<const uint4*>(vg + (uint32_t)(p * a.block_size));
         }
     };
     auto store_round = [&](int buf, int j0) {
-        const bool inside = j0 >= lo_min && j0 + 32 * TW - 1 <= p_max;  // (uniform)
+        const int jk = j0 + 8 * wave_s;                       // (not clamped: what the group stands for)
+        const bool inside = jk >= lo_min && jk + 7 <= p_max;  // (the same for the wave)
+        const int tile = wave_s / 4, kg4 = wave_s % 4;
 #pragma unroll
-        for (int i = 0; i < PER_THREAD; ++i) {
-            const int c_all = tid + LT * i;
-            if (c_all < TW * PIECES) {
-                const int c = c_all % PIECES, tile = c_all / PIECES;
-                if (!inside) {
-                    const int jk = j0 + 32 * tile + 8 * (c % 4);
-                    vreg[i] = keep_elements(vreg[i], lo_min - jk, p_max + 1 - jk);
-                }
-                const int kl = c / KCH, ch = c % KCH;                    // key kl = 8a + 4u + b2 of the tile
-                const int row = ((kl >> 2) & 1) * 16 + (kl >> 3) * 4 + (kl & 3);  // -> row 16u + 4a + b2
+        for (int i = 0; i < PER_LANE; ++i) {
+            const int p = lane + LLMS_WAVE * i;
+            if (p < D) {
+                if (!inside) vreg[i] = keep_elements(vreg[i], lo_min - jk, p_max + 1 - jk);
+                const int q = p / KCH, ch = p % KCH;             // key 8 kg4 + q of the tile = 8a + 4u + b2
+                const int row = (q >> 2) * 16 + kg4 * 4 + (q & 3);  // -> row 16u + 4a + b2
                 k_lds[(buf * TW + tile) * K_TILE + row * KROW + ch] = kreg[i];
-                v_lds[(buf * TW + tile) * V_TILE + c] = vreg[i];
+                v_lds[(buf * TW + tile) * V_TILE + p * 4 + kg4] = vreg[i];  // [dimension][4 chunks of 8 keys]
             }
         }
     };

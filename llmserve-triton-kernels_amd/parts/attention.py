@@ -133,10 +133,13 @@ class Attention(Mixer):
                                table_rows=batch.state_slots)
 
     def prompt_splits(self, n_requests: int, max_new: int, max_context: int) -> int:
-        """Workgroups that share the keys of one block of prompt tokens.  A long prompt has blocks enough to
-        fill the chip by itself; a short portion behind a long prefix has few blocks and many keys, and four
-        waves per CU wait for memory most of the time, so its keys are shared out until every CU has about four
-        workgroups, 8 tiles of keys each at least (a second kernel merges the shares)."""
+        """Workgroups that share the keys of one block of prompt tokens (a second kernel merges their shares).
+        Blocks enough for a workgroup of 8 waves on every CU need no sharing: there each wave has a twin that
+        takes every other tile of keys for the same tokens, and with two such workgroups per CU the long blocks
+        and the short ones even out.  With exactly one per CU sharing pays only behind a long prefix (measured:
+        from about 3,000 keys on).  A short portion behind a long prefix has few blocks and many keys: its keys
+        are shared out until the chip holds about two workgroups of 4 waves per CU, 8 tiles of keys each at
+        least."""
         if self.window:
             return 1
         g = self.num_heads // self.num_kv_heads
@@ -144,7 +147,11 @@ class Attention(Mixer):
         blocks = -(-max_new // (4 * (16 // hg)))  # of 4 waves with one column group each
         workgroups = blocks * self.num_kv_heads * -(-g // hg) * n_requests
         tiles = -(-max_context // 32)
-        return max(1, min(1024 // max(workgroups, 1), tiles // 8, 8))
+        if workgroups >= 512:
+            return 1
+        if workgroups >= 256:
+            return 4 if tiles >= 96 else 1
+        return max(1, min(512 // max(workgroups, 1), tiles // 8, 8))
 
     def decode_arrangement(self, n_requests: int, max_context: int) -> tuple[int, int]:
         """(workgroups per request and KV head, waves per workgroup) for decoding.  The waves of a
