@@ -26,6 +26,7 @@
 #include "common.h"
 #include "attention_mfma.h"
 
+#include <algorithm>
 #include <mutex>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -71,6 +72,9 @@ struct AttnArgs {
     // zero between launches.  Non-null: the workgroups of a group count themselves here and the last to arrive adds
     // the shares up (no merge kernel).
     unsigned* arrive;
+    // prompts with twins: the first workgroup of every CU (the first `first_blocks` values of blockIdx.y) takes one
+    // of the longest blocks of tokens, shortest of them first; the rest follow from the longest remaining one down
+    int first_blocks;
 };
 
 // 2^x by the hardware's own instruction.  Scores are kept in units of log2(e) (scale_log2 = scale * log2 e), so
@@ -120,10 +124,13 @@ __device__ __forceinline__ float column_sum(float x) {
 //   each stage side by side, not one group after the other: their chains (matrix product, maximum, exponentials,
 //   matrix product) do not depend on each other, and a wave that alternates between them waits less for each.
 #define STALE_MAX 8.f  // by how much (in powers of two) a column's maximum may pass the reference before a rescale
-template <int DB, int KS, bool MASKED, int CG>
+//   fill_values(): called once the score products are issued, may bring vf in then (it is read after the softmax):
+//   what it asks LDS for arrives while the vector unit is busy, and does not stand in the way of the key rows.
+template <int DB, int KS, bool MASKED, int CG, class FillValues>
 __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (&m_run)[CG], float (&l_run)[CG],
-                                                   const uint4 (&kf)[2][KS], const uint4 (&vf)[DB], const uint4 (&qf)[CG][KS],
-                                                   int jk, const int (&lo_col)[CG], const int (&p_col)[CG], float scale_log2) {
+                                                   const uint4 (&kf)[2][KS], uint4 (&vf)[DB], const uint4 (&qf)[CG][KS],
+                                                   int jk, const int (&lo_col)[CG], const int (&p_col)[CG], float scale_log2,
+                                                   FillValues fill_values) {
     f32x4 s_acc[CG][2];
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg)
@@ -134,6 +141,7 @@ __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (
             for (int s = 0; s < KS; ++s)
                 s_acc[cg][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[u][s]), as_bf16x8(qf[cg][s]), s_acc[cg][u], 0, 0, 0);
         }
+    fill_values();
     // the lane holds its column's scores for the keys jk .. jk+7; the other 24 keys sit in the 3 other lane groups
     float sc[CG][8], m_new[CG], m_safe[CG];
     bool grew = false;
@@ -199,8 +207,8 @@ __device__ __forceinline__ void attend_tile(f32x4 (&acc)[DB], float& m_run, floa
                                             float scale_log2) {
     float m1[1] = {m_run}, l1[1] = {l_run};
     const int lo1[1] = {lo_col}, p1[1] = {p_col};
-    attend_tile_groups<DB, KS, MASKED, 1>(reinterpret_cast<f32x4 (&)[1][DB]>(acc), m1, l1, kf, vf,
-                                          reinterpret_cast<const uint4 (&)[1][KS]>(qf), jk, lo1, p1, scale_log2);
+    attend_tile_groups<DB, KS, MASKED, 1>(reinterpret_cast<f32x4 (&)[1][DB]>(acc), m1, l1, kf, const_cast<uint4 (&)[DB]>(vf),
+                                          reinterpret_cast<const uint4 (&)[1][KS]>(qf), jk, lo1, p1, scale_log2, [] {});
     m_run = m1[0];
     l_run = l1[0];
 }
@@ -498,7 +506,7 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
 // a SIMD always has two waves to switch between, and the blocks are handed out from the longest to the shortest
 // (blockIdx.y counts from the end of the prompt), so that a CU that was given a long one takes a short one next.
 template <int DB, bool TWIN, int CG, int WB>
-__global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt_kernel(const AttnArgs a) {
+__global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) ? 4 : 1) void attn_prompt_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
     constexpr int KS = (D + 31) / 32;
     constexpr int KCH = D / 8;          // 16-byte chunks of a key row
@@ -525,9 +533,13 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt_k
     const int BLK = WB * CG * TPG;  // tokens of a block: WB waves with CG column groups each
     int wg_first;                   // first token (within the request's new tokens) of the workgroup's block
     if (TWIN) {
-        const int blocks = (n_new + BLK - 1) / BLK;
-        if ((int)blockIdx.y >= blocks || ctx <= 0) return;
-        wg_first = (blocks - 1 - (int)blockIdx.y) * BLK;
+        // rank 0: the last block of the prompt, which sees the most keys.  Workgroups are handed out in the order
+        // of blockIdx.y: the first on every CU get the longest blocks, and the CU that was given the shortest of
+        // these gets the longest of the rest
+        const int blocks = (n_new + BLK - 1) / BLK, by = blockIdx.y;
+        const int rank = by < a.first_blocks ? a.first_blocks - 1 - by : by;
+        if (rank >= blocks || ctx <= 0) return;
+        wg_first = (blocks - 1 - rank) * BLK;
     } else {
         wg_first = ((int)blockIdx.x / a.num_splits) * BLK;
         if (wg_first >= n_new || ctx <= 0) return;
@@ -660,10 +672,20 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt_k
     for (int r = r_lo; r < r_hi; ++r) {
         const int buf = (r - r_lo) & 1, j0 = j_begin + 32 * (TW * r + twin);  // this wave's tile of the round
         const bool busy = wave_on && j0 <= w_pmax;  // (a tile beyond the wave's last position adds nothing)
+        // the next round into the other buffer (last read before the previous barrier), the round after that asked
+        // for, and the pages of the one after that: by the twins before they read their fragments from LDS, by the
+        // others after their tile, so that the two waves of a SIMD are not at the same stage at the same time (one
+        // multiplies while the other computes exponentials) and the reads of the one half of the waves have LDS to
+        // themselves while the other half still fetches
+        auto fetch_ahead = [&]() {
+            if (r + 1 < r_hi) store_round(buf ^ 1, first_key(r + 1));
+            load_round(first_key(r + 2));
+            ask_pages(first_key(r + 3));
+        };
+        if (TWIN && twin == 1) fetch_ahead();
         uint4 kf[2][KS], vf[DB];
         if (busy) {
             const uint4* kt = k_lds + (buf * TW + twin) * K_TILE;
-            const uint4* vt = v_lds + (buf * TW + twin) * V_TILE;
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -671,24 +693,18 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE) void attn_prompt_k
                     const int ch = 4 * s + g;
                     kf[u][s] = kt[(16 * u + col) * KROW + (ch < KCH ? ch : 0)];  // (beyond head_dim the queries are zero)
                 }
-#pragma unroll
-            for (int m = 0; m < DB; ++m) vf[m] = vt[(16 * m + col) * 4 + g];
         }
-        // the next round into the other buffer (last read before the previous barrier), the round after that asked
-        // for, and the pages of the one after that: by the twins while the fragments are on their way from LDS, by
-        // the others after their tile, so that the two waves of a SIMD are not at the same stage at the same time
-        // (one multiplies while the other computes exponentials)
-        auto fetch_ahead = [&]() {
-            if (r + 1 < r_hi) store_round(buf ^ 1, first_key(r + 1));
-            load_round(first_key(r + 2));
-            ask_pages(first_key(r + 3));
-        };
-        if (!TWIN || twin == 1) fetch_ahead();
+        if (!TWIN) fetch_ahead();  // (while the fragments are on their way)
         if (busy) {
             const bool all_seen = j0 >= w_lo_max && j0 + 31 <= w_pmin;  // (uniform over the wave; columns without a token are discarded)
-            // the same keys and values for each of the wave's column groups
-            if (all_seen) attend_tile_groups<DB, KS, false, CG>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
-            else attend_tile_groups<DB, KS, true, CG>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2);
+            // the same keys and values for each of the wave's column groups; the values are asked for after the keys' products
+            const uint4* vt = v_lds + (buf * TW + twin) * V_TILE;
+            auto read_values = [&]() {
+#pragma unroll
+                for (int m = 0; m < DB; ++m) vf[m] = vt[(16 * m + col) * 4 + g];
+            };
+            if (all_seen) attend_tile_groups<DB, KS, false, CG>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2, read_values);
+            else attend_tile_groups<DB, KS, true, CG>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2, read_values);
         }
         if (TWIN && twin == 0) fetch_ahead();
         __syncthreads();
@@ -830,6 +846,22 @@ static int launch_prompt(int db, int cg, dim3 grid, bool twin, const AttnArgs& a
     return LLMS_OK;
 }
 
+// CUs of the current device (asked once per device).
+static int compute_units(int* out) {
+    static int cached[64];
+    int dev = -1;
+    LLMS_HIP_CHECK(hipGetDevice(&dev));
+    LLMS_REQUIRE(dev >= 0 && dev < 64, "attention_mfma: device index out of range");
+    if (cached[dev] == 0) {
+        int n = 0;
+        LLMS_HIP_CHECK(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+        LLMS_REQUIRE(n > 0, "attention_mfma: the device reports no compute units");
+        cached[dev] = n;
+    }
+    *out = cached[dev];
+    return LLMS_OK;
+}
+
 static int launch_attn(int db, dim3 grid, int threads, const AttnArgs& a, hipStream_t stream) {
 #define ATT_CASE(N)                                                                                  \
     case N:                                                                                          \
@@ -885,7 +917,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     const int groups = (max_new + TPG - 1) / TPG;
     AttnArgs a = {(bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pool, (const bf16*)v_pool,
                   block_tables, table_rows, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
-                  window, scale, num_splits, ws_o, ws_ml, nullptr};
+                  window, scale, num_splits, ws_o, ws_ml, nullptr, 0};
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
     LLMS_REQUIRE(arrive == nullptr || ((uintptr_t)arrive % 4 == 0 && n_arrive > 0), "attention_mfma: bad counters");
     if (split_waves > 0) {
@@ -913,11 +945,19 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
         auto workgroups = [](dim3 g) { return (long long)g.x * g.y * g.z; };
         int cg = PROMPT_CG_MAX(head_dim / 16);
         dim3 grid = grid_for(cg);
-        if (cg == 2 && workgroups(grid) < PROMPT_FULL_CHIP) grid = grid_for(cg = 1);
+        if (cg == 2 && workgroups(grid) < PROMPT_FULL_CHIP * (twin && head_dim <= 64 ? 2 : 1)) grid = grid_for(cg = 1);
         if (twin && workgroups(grid) < PROMPT_FULL_CHIP) twin = false;  // a short portion: workgroups for more CUs matter more
-        if (twin) {  // heads in x, blocks of tokens in y from the last one: the order in which workgroups are handed out
+        if (twin) {  // heads in x, blocks of tokens in y: the order in which workgroups are handed out
             LLMS_REQUIRE(grid.x <= 65535, "attention_mfma: too many tokens per request for one launch");
             grid = dim3(grid.y, grid.x, grid.z);
+            int cus = 0;
+            if (int e = compute_units(&cus)) return e;
+            // The first workgroup of every CU: the longest blocks, shortest of them first; then from the longest
+            // remaining block down.  Where a CU holds one workgroup, the CU that is free first takes the longest of
+            // the rest; where it holds two (head_dim up to 64: the registers of 16 waves and two sets of tiles fit),
+            // the second lands on the CUs in the order of the first (measured), so each CU gets a long and a
+            // short one that add up to the same.
+            a.first_blocks = n_seqs == 1 ? (int)std::min<long long>(grid.y, cus / grid.x) : 0;
         }
         if (int e = launch_prompt(head_dim / 16, cg, grid, twin, a, stream)) return e;
         if (num_splits > 1) {
