@@ -540,9 +540,9 @@ MFMA_CASES = [  # nh, nkv, d, bs, lens, new, window
 ]
 
 
-# split_waves: False = the prompt kernel (tiles shared through LDS, early and late blocks paired when there is
-# no window and the launch is large; with splits, the keys of a block shared out to workgroups), True = the waves
-# (4 or 8) share the keys, optionally split over workgroups
+# split_waves: False = the prompt kernel (tiles shared through LDS; without a window and in a large launch every wave
+# has a twin that takes every other tile for the same columns; with splits, the keys of a block shared out to
+# workgroups), True = the waves (4 or 8) share the keys, optionally split over workgroups
 @pytest.mark.parametrize("arrangement", [(False, 1, 4), (False, 2, 4), (False, 5, 4), (True, 1, 4), (True, 2, 4), (True, 5, 4),
                                          (True, 1, 8), (True, 3, 8)])
 @pytest.mark.parametrize("case", MFMA_CASES)
@@ -618,15 +618,16 @@ def test_decode_shares_added_up_inside_a_replayed_graph():
         assert torch.equal(out, want)
 
 
-# The prompt kernel gives a wave two column groups (32 columns) up to head_dim 128, and pairs early with late blocks of
-# tokens, once the launch has a workgroup for each of the 256 CUs; the cases above are too small for that.
+# The prompt kernel gives a wave two column groups (32 columns) up to head_dim 128, and every wave a twin for every
+# other tile of keys, once the launch has a workgroup for each of the 256 CUs (two each for two column groups up to
+# head_dim 64); the cases above are too small for that.
 WIDE_LAUNCH_CASES = [  # nh, nkv, d, bs, lens, new, window
     (16, 16, 32, 8, [260, 200, 131, 97, 260, 33, 1, 17], [260, 200, 131, 97, 260, 33, 1, 17], 0),  # a second group without tokens
     (16, 4, 64, 16, [520, 300, 77, 515, 512, 511, 2, 64], [520, 300, 77, 100, 512, 31, 2, 64], 0),  # portions beside whole prompts
-    (16, 16, 32, 8, [300, 290, 280, 31, 300, 47], [300, 290, 280, 31, 300, 16], 50),               # a window: no pairing
+    (16, 16, 32, 8, [300, 290, 280, 31, 300, 47], [300, 290, 280, 31, 300, 16], 50),               # a window: no twins
     (16, 16, 128, 16, [300, 129, 128, 127, 33, 290, 150, 257], [300, 129, 128, 127, 33, 290, 7, 257], 0),
     (24, 8, 80, 8, [330, 190, 1, 64, 200, 326, 65, 200], [330, 190, 1, 64, 200, 3, 65, 200], 0),
-    (16, 16, 160, 8, [300, 150, 17, 290, 300, 64, 300, 1], [300, 150, 17, 290, 300, 64, 300, 1], 0),  # one group, paired
+    (16, 16, 160, 8, [300, 150, 17, 290, 300, 64, 300, 1], [300, 150, 17, 290, 300, 64, 300, 1], 0),  # one group, twins
 ]
 
 
@@ -637,9 +638,55 @@ def test_attention_mfma_launches_that_fill_the_chip(case):
     hg = min(g, 16)
     groups = -(-max(new) // (16 // hg))
     blocks = -(-groups // (8 if d <= 128 else 4))
-    workgroups = (blocks if window else -(-blocks // 2)) * nkv * -(-g // hg) * len(lens)
-    assert workgroups >= 256, "this case would run with one column group per wave and without pairing"
+    workgroups = blocks * nkv * -(-g // hg) * len(lens)
+    assert workgroups >= 256, "this case would run without twins"
     got, ref = run_attention_mfma(nh, nkv, d, bs, lens, new, window, seed=55)
+    assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
+
+
+# One long prompt, or a long portion behind a prefix: every wave has a twin, and the blocks of tokens are handed out
+# in an order of their own (the first workgroup of every CU takes one of the longest, shortest of these first).
+# One or two column groups per wave, one or two workgroups per CU, pages of 8, 16, 24 and 32 (the block index is one
+# multiply with a rounded-up reciprocal), a prompt that ends in the middle of a block, of a tile and of a page.
+LONG_PROMPT_CASES = [  # nh, nkv, d, bs, len, new
+    (32, 4, 64, 16, 2048, 2048),   # two column groups, two workgroups per CU, every CU's first workgroup in the fold
+    (32, 4, 64, 16, 2093, 1500),   # the same behind a prefix, ends off every boundary
+    (16, 16, 32, 8, 2100, 2100),   # one column group (too few blocks for two), 16 tokens per group
+    (16, 16, 128, 32, 1100, 1100), # head_dim 128: one workgroup per CU
+    (24, 8, 48, 24, 1571, 1571),   # pages of 24 keys, 3 heads per KV head
+    (8, 8, 64, 16, 4111, 4111),    # more workgroups than run at once
+]
+
+
+@pytest.mark.parametrize("case", LONG_PROMPT_CASES)
+def test_attention_mfma_one_long_prompt(case):
+    nh, nkv, d, bs, length, new = case
+    got, ref = run_attention_mfma(nh, nkv, d, bs, [length], [new], 0, seed=57)
+    assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
+
+
+def test_attention_mfma_long_prompt_finds_one_far_key_per_token():
+    """Every query of a long prompt looks for one key of its own, far back or near, among two thousand: a block of
+    tokens that took the wrong keys, a tile that its twin skipped or a page read twice would miss some."""
+    length, nh, nkv, d = 2048, 32, 4, 64
+    gen = torch.Generator().manual_seed(58)
+    wanted = [int(torch.randint(0, t + 1, (1,), generator=gen)) for t in range(length)]  # key of token t, <= t
+
+    def craft(qs, ks, vs):
+        # dimension 0..10 of a key spell its index in +-1; a query spells the index it wants, scaled up, so that
+        # the wanted key scores 11 * 40 and every other at most 9 * 40 (55 against 45 after the scaling by 1/8)
+        bits = lambda i: torch.tensor([1.0 if (i >> b) & 1 else -1.0 for b in range(11)])  # noqa: E731
+        for t in range(length):
+            ks[0][t, :, :11] = bits(t)
+            qs[0][t, :, :11] = 40.0 * bits(wanted[t])
+            vs[0][t] = 0.0
+            vs[0][t, :, 0] = float(t % 128)
+        ks[0][:, :, 11:] *= 0.1
+
+    got, ref = run_attention_mfma(nh, nkv, d, 16, [length], [length], 0, seed=59, craft=craft)
+    value = got.view(length, nh, d)[:, :, 0]
+    want = torch.tensor([float(w % 128) for w in wanted]).unsqueeze(1).expand(length, nh)
+    assert (value - want).abs().max() <= 0.51, "a token did not find its key"
     assert (got - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
 
 
