@@ -919,6 +919,8 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
                   block_tables, table_rows, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
                   window, scale, num_splits, ws_o, ws_ml, nullptr, 0};
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
+    LLMS_REQUIRE((unsigned long long)max_blocks * block_size * block_size <= 0xFFFFFFFFull,
+                 "attention_mfma: block table too long for this page size (keys * block_size must stay below 2^32)");
     LLMS_REQUIRE(arrive == nullptr || ((uintptr_t)arrive % 4 == 0 && n_arrive > 0), "attention_mfma: bad counters");
     if (split_waves > 0) {
         dim3 grid(groups * num_splits, n_kv_heads * HB, n_seqs);
@@ -935,8 +937,6 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     } else {
         // twins (8 waves, two tiles a round) where a workgroup per CU is left that way; wider heads would not fit
         // the registers of 8 waves, a window or splits have their own arrangement
-        LLMS_REQUIRE((unsigned long long)max_blocks * block_size * block_size <= 0xFFFFFFFFull,
-                     "attention_mfma: block table too long for this page size (keys * block_size must stay below 2^32)");
         bool twin = window == 0 && head_dim <= 192 && num_splits == 1;
         auto grid_for = [&](int cg) {
             const int per_block = PROMPT_WB * cg;  // column groups of a block of tokens
