@@ -493,8 +493,9 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
     step, whose new tokens are rows [token_begin, token_begin + n_tokens) of q and out and bring at most
     `max_new` tokens each.  `split_waves` (with `waves` = 4 or 8 and `num_splits`) spreads each request's keys
     over the waves of a workgroup and over workgroups: the arrangement for single decoded tokens.  Without
-    it the 4 waves of a workgroup take neighbouring tokens and share each tile of keys through LDS; `num_splits`
-    then shares the keys of such a block of tokens out to several workgroups (short portions, long prefixes).
+    it the 4 waves of a block of tokens take neighbouring tokens and share each tile of keys through LDS (in a
+    large launch without a window each has a twin wave that takes every other tile); `num_splits` instead
+    shares the keys of such a block of tokens out to several workgroups (short portions, long prefixes).
     The shares of workgroups are added up, in the order of the splits, by a second kernel, or for decoding with up
     to 16 splits by the workgroup of each group that finishes last (`merge_kernel=True` asks for the second kernel
     there too: the same bits).  (For prompt portions the last workgroup was tried as well: no faster.)"""
