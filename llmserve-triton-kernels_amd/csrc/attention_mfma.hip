@@ -117,15 +117,16 @@ __device__ __forceinline__ float column_sum(float x) {
 // values.
 //   kf[u][s]: key rows of score tile u (row i = key 8*(i/4) + 4u + i%4), k-step s;  vf[m]: the lane's 8 keys
 //   (jk .. jk+7) of value dimensions 16m + col, already zero where the key is outside the group's range;
-//   qf[cg][s]: the lane's column of queries.  acc[cg][m][r] = O^T[16m + 4g + r][col] and the running max (times
-//   log2 e) and sum of the column are updated in place.  MASKED = false: every key of the tile is visible to every
-//   column of the wave (the caller knows), which saves the comparisons.  The accumulators are rescaled only when
-//   some column's maximum grew: a factor of exactly 1 otherwise, so the result is the same.  The groups go through
-//   each stage side by side, not one group after the other: their chains (matrix product, maximum, exponentials,
-//   matrix product) do not depend on each other, and a wave that alternates between them waits less for each.
-#define STALE_MAX 8.f  // by how much (in powers of two) a column's maximum may pass the reference before a rescale
+//   qf[cg][s]: the lane's column of queries.  acc[cg][m][r] = O^T[16m + 4g + r][col], the column's reference
+//   for its weights (times log2 e; its running maximum or a little less) and the sum of its weights are updated in
+//   place; the sum as the lane's own share of it (the caller adds the four lanes of a column up once, at the end:
+//   column_sum).  MASKED = false: every key of the tile is visible to every column of the wave (the caller
+//   knows), which saves the comparisons.  The groups go through each stage side by side, not one group after the
+//   other: their chains (matrix product, maximum, exponentials, matrix product) do not depend on each other, and
+//   a wave that alternates between them waits less for each.
 //   fill_values(): called once the score products are issued, may bring vf in then (it is read after the softmax):
 //   what it asks LDS for arrives while the vector unit is busy, and does not stand in the way of the key rows.
+#define STALE_MAX 8.f  // by how much (in powers of two) a column's maximum may pass the reference before a rescale
 template <int DB, int KS, bool MASKED, int CG, class FillValues>
 __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (&m_run)[CG], float (&l_run)[CG],
                                                    const uint4 (&kf)[2][KS], uint4 (&vf)[DB], const uint4 (&qf)[CG][KS],
@@ -143,7 +144,7 @@ __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (
         }
     fill_values();
     // the lane holds its column's scores for the keys jk .. jk+7; the other 24 keys sit in the 3 other lane groups
-    float sc[CG][8], m_new[CG], m_safe[CG];
+    float sc[CG][8], t_max[CG], m_safe[CG];
     bool grew = false;
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg) {
@@ -157,25 +158,26 @@ __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (
             }
             tmax = fmaxf(tmax, sc[cg][e]);
         }
-        tmax = column_max(tmax);
-        m_new[cg] = fmaxf(m_run[cg], tmax * scale_log2);  // (scale > 0)
-        grew = grew || m_new[cg] > m_run[cg] + STALE_MAX;   // (also a column's first key: -inf + x = -inf)
+        t_max[cg] = tmax;  // of the lane's 8 keys
+        grew = grew || tmax * scale_log2 > m_run[cg] + STALE_MAX;  // (scale > 0; also a column's first key: -inf + x = -inf)
     }
-    // m_run is the reference the weights are taken against, not necessarily the maximum: while no column's
-    // maximum has passed its reference by more than STALE_MAX (a factor of 2^STALE_MAX in the weights and sums,
-    // far inside the range of 32-bit and bfloat16 numbers, and the same relative precision), nothing is rescaled.
-    // The quotient at the end does not depend on the reference.
+    // m_run is the reference the weights are taken against, not necessarily the maximum: while no score has passed
+    // its column's reference by more than STALE_MAX (a factor of 2^STALE_MAX in the weights and sums, far inside
+    // the range of 32-bit and bfloat16 numbers, and the same relative precision), nothing is rescaled, and the
+    // maximum over the column's four lanes is not even formed.  The quotient at the end does not depend on the
+    // reference.
     if (__builtin_amdgcn_ballot_w64(grew) != 0) {
 #pragma unroll
         for (int cg = 0; cg < CG; ++cg) {
-            const float m_ref = (MASKED && m_new[cg] == -INFINITY) ? 0.f : m_new[cg];
+            const float m_new = fmaxf(m_run[cg], column_max(t_max[cg]) * scale_log2);
+            const float m_ref = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
             const float corr = exp2_fast(m_run[cg] - m_ref);  // 1 where the maximum stayed; 0 while the column has seen no key
             l_run[cg] *= corr;
 #pragma unroll
             for (int m = 0; m < DB; ++m)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc[cg][m][r] *= corr;
-            m_run[cg] = m_new[cg];
+            m_run[cg] = m_new;
         }
     }
 #pragma unroll
@@ -189,7 +191,7 @@ __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (
             sc[cg][e] = exp2_fast(fmaf(sc[cg][e], scale_log2, -m_safe[cg]));
             psum = e == 0 ? sc[cg][0] : psum + sc[cg][e];
         }
-        l_run[cg] += column_sum(psum);
+        l_run[cg] += psum;  // (the lane's share: the four lanes of a column are added up once, by whoever reads the sum)
         pf[cg] = make_uint4(pack_bf16(sc[cg][0], sc[cg][1]), pack_bf16(sc[cg][2], sc[cg][3]), pack_bf16(sc[cg][4], sc[cg][5]),
                             pack_bf16(sc[cg][6], sc[cg][7]));
     }
@@ -419,6 +421,7 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
 #pragma unroll
     for (int m = 0; m < DB; ++m)
         *reinterpret_cast<float4*>(sh_acc[wave][m][lane]) = make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+    l_run = column_sum(l_run);  // (until here every lane kept its own share of its column's sum)
     if (g == 0) {
         sh_m[wave][col] = m_run;
         sh_l[wave][col] = l_run;
@@ -709,6 +712,8 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
         if (TWIN && twin == 0) fetch_ahead();
         __syncthreads();
     }
+#pragma unroll
+    for (int cg = 0; cg < CG; ++cg) l_run[cg] = column_sum(l_run[cg]);  // (every lane kept its own share of its column's sum)
     if constexpr (TWIN) {
         // The twin's share (second tile of every round) joins the first wave's, one column group at a time:
         // [item][twin wave][lane] floats in the memory of the tiles, which nobody reads any more.
