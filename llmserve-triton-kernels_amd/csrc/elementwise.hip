@@ -289,6 +289,44 @@ __global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restri
             *reinterpret_cast<uint4*>(dst + half) = make_uint4(rb[0], rb[1], rb[2], rb[3]);
         }
     }
+    // Values.  A page holds them transposed (a dimension's keys side by side), so a token alone leaves in 2-byte
+    // stores.  Eight tokens that lie side by side in one page (a prompt's: slots lead .. lead + 7, the first a
+    // multiple of 8) are stored by the workgroup of the first of them instead, 8 x 8 pieces turned in registers,
+    // 16 bytes per store.  Every workgroup of such a group finds the same answer from the same eight slots.
+    const int lead = n & ~7;
+    bool side_by_side = false;
+    if (slots && lead + 7 < n_tokens && block_size % 8 == 0 && ((uintptr_t)v_pool % 16) == 0) {
+        const int s0 = slots[lead];
+        side_by_side = s0 >= 0 && s0 % 8 == 0;
+#pragma unroll
+        for (int j = 1; j < 8; ++j) side_by_side = side_by_side && slots[lead + j] == s0 + j;
+    }
+    if (side_by_side) {
+        if (n != lead) return;
+        const int page8 = slot / block_size, off8 = slot % block_size;  // (n == lead: its own slot)
+        const bf16* v0 = row + (size_t)(n_heads + n_kv_heads) * head_dim;
+        for (int t = threadIdx.x; t < n_kv_heads * head_dim / 8; t += blockDim.x) {
+            uint32_t in[8][4];  // [token][pair of dimensions]
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint4 vv = *reinterpret_cast<const uint4*>(v0 + (size_t)j * row_width + 8 * t);
+                in[j][0] = vv.x; in[j][1] = vv.y; in[j][2] = vv.z; in[j][3] = vv.w;
+            }
+            const int kvh = (8 * t) / head_dim, d = (8 * t) % head_dim;
+            bf16* dst = v_pool + (((size_t)page8 * n_kv_heads + kvh) * head_dim + d) * block_size + off8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {  // dimension d + i: the 8 tokens' values, two to a word
+                uint32_t w[4];
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const uint32_t a = in[2 * m][i / 2], b = in[2 * m + 1][i / 2];
+                    w[m] = (i & 1) ? ((a >> 16) | (b & 0xffff0000u)) : ((a & 0xffffu) | (b << 16));
+                }
+                *reinterpret_cast<uint4*>(dst + (size_t)i * block_size) = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+        return;
+    }
     if (slot >= 0) {
         const bf16* v = row + (size_t)(n_heads + n_kv_heads) * head_dim;
         for (int t = threadIdx.x; t < n_kv_heads * head_dim / 8; t += blockDim.x) {

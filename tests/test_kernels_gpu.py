@@ -103,6 +103,52 @@ def test_rmsnorm_tiny_inputs_feel_eps():
         assert torch.allclose(out.cpu(), plain_llama.rms_norm(x, w, eps), atol=1e-6)
 
 
+@pytest.mark.parametrize("nh,nkv,d,bs", [(4, 2, 16, 16), (8, 8, 64, 8), (16, 2, 128, 32), (6, 3, 48, 24), (4, 4, 32, 4)])
+def test_rope_store_prompt_tokens_side_by_side(nh, nkv, d, bs):
+    """A prompt's tokens lie side by side in their pages: eight of them that start at a multiple of 8 are stored by
+    one workgroup, 16 bytes per dimension.  Runs that start off such a boundary, break in the middle (another page,
+    a token without a slot), or end before eight, and a second request behind the first, leave as single values:
+    every slot must hold its own token's values and nothing else may change."""
+    dtype = torch.bfloat16
+    pages = 16
+    # request a: 29 tokens from slot 3 of page 2 on through pages 5 and 1 (pages need not follow each other)
+    # request b: 16 tokens from the start of page 7, the 12th without a slot; then 5 scattered single tokens
+    def run(page_list, first, count):
+        out, page_i, off = [], 0, first
+        for _ in range(count):
+            out.append(page_list[page_i] * bs + off)
+            off += 1
+            if off == bs:
+                page_i, off = page_i + 1, 0
+        return out
+    slots = run([2, 5, 1, 9, 10, 11, 0, 4], 3, 29) + run([7, 3, 6, 8], 0, 16)  # (12 of the 16 pages at most)
+    slots[29 + 11] = -1
+    free = sorted(set(range(pages * bs)) - set(slots))
+    assert len(free) >= 8
+    slots += [free[0], free[-1], free[len(free) // 2], -1, free[1]]
+    n = len(slots)
+    width = (nh + 2 * nkv) * d
+    qkv = rnd(n, width, seed=16).to(dtype)
+    positions = torch.arange(n, dtype=torch.int32)
+    inv_freq = 1.0 / (1e4 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    k_pool = torch.full((pages, nkv, bs, d), 7.0, dtype=dtype, device=DEV)
+    v_pool = torch.full((pages, nkv, d, bs), 7.0, dtype=dtype, device=DEV)
+    dev_qkv = qkv.clone().to(DEV)
+    ops().rope_store(dev_qkv, inv_freq.to(DEV), positions.to(DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                     k_pool, v_pool, nh, nkv, d, bs)
+    v = qkv[:, (nh + nkv) * d:].view(n, nkv, d)
+    vp = v_pool.cpu()
+    written = torch.zeros(pages, bs, dtype=torch.bool)
+    for i, sl in enumerate(slots):
+        if sl < 0:
+            continue
+        page, off = divmod(sl, bs)
+        written[page, off] = True
+        assert torch.equal(vp[page, :, :, off], v[i]), f"token {i} (slot {sl})"
+    assert (vp.permute(0, 3, 1, 2)[~written] == 7).all()
+    assert torch.equal(dev_qkv.cpu()[:, (nh + nkv) * d:], qkv[:, (nh + nkv) * d:])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,bs,theta", [(4, 2, 16, 16, 1e4), (3, 1, 32, 8, 5e5), (8, 8, 64, 4, 1e4),
                                                (5, 5, 48, 1, 1e6), (16, 2, 128, 32, 1e4)])
