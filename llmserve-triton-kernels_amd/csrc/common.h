@@ -95,8 +95,14 @@ __device__ __forceinline__ float block_sum(float v, float* lds /* >= 16 floats *
     __syncthreads();
     if (lane == 0) lds[wave] = v;
     __syncthreads();
+    // (all 16 places are read at once and those of waves that do not exist left out: a loop up to nwaves would
+    // wait for LDS once per wave)
+    float part[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) part[i] = lds[i];
     float t = 0.f;
-    for (int i = 0; i < nwaves; ++i) t += lds[i];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) t += i < nwaves ? part[i] : 0.f;
     return t;
 }
 
@@ -107,7 +113,11 @@ __device__ __forceinline__ float block_max(float v, float* lds) {
     __syncthreads();
     if (lane == 0) lds[wave] = v;
     __syncthreads();
-    float t = lds[0];
-    for (int i = 1; i < nwaves; ++i) t = fmaxf(t, lds[i]);
+    float part[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) part[i] = lds[i];
+    float t = part[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) t = fmaxf(t, i < nwaves ? part[i] : part[0]);
     return t;
 }
