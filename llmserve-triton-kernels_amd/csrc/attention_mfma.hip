@@ -506,8 +506,9 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
 // its twin w + WB own the same columns, the one takes the first tile of every round, the other the second, and
 // the twin's sums are merged into the other's through LDS at the end, first tile first.  The causal triangle gives
 // the last tokens of a prompt the most keys: the chain of dependent rounds of the longest block is halved this way,
-// a SIMD always has two waves to switch between, and the blocks are handed out from the longest to the shortest
-// (blockIdx.y counts from the end of the prompt), so that a CU that was given a long one takes a short one next.
+// a SIMD always has two waves to switch between (four up to head_dim 64, where two workgroups share a CU), and the
+// blocks are handed out in an order (see `rank` below) in which a CU that was given a long one gets a short one
+// beside or after it.
 template <int DB, bool TWIN, int CG, int WB>
 __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) ? 4 : 1) void attn_prompt_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
