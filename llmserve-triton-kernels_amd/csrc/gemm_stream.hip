@@ -338,8 +338,10 @@ __global__ __launch_bounds__(ST_WAVES* LLMS_WAVE) void gemm_slices_kernel(const 
 }
 
 // A launch with a workgroup or less per CU gets chunks of 512 (16 KB in flight per wave: all a lone workgroup can
-// do for its CU), a larger one chunks of 128 (eight workgroups per CU, no rounds); up to four workgroups per CU
-// these have 8 waves, which doubles what the launch has in flight (down_proj at batch 8: 7.0 to 6.8 microseconds).
+// do for its CU), a larger one chunks of 128 (eight workgroups per CU, no rounds); up to three workgroups per CU
+// and 16 rows these have 8 waves, which doubles what the launch has in flight (TinyLlama's down_proj: 7.4 to 6.5
+// microseconds at batch 1, 7.5 to 7.2 at batch 8; with more workgroups or more rows the same was slower: the
+// 7B shape's o_proj with 1,024 workgroups 9.0 to 9.8).
 #define ST_FEW_WORKGROUPS 256
 
 template <typename TOut, int EPI>
@@ -347,7 +349,7 @@ static void launch_stream(unsigned tiles, const StreamArgs& a, hipStream_t strea
     const dim3 grid(tiles, a.k_splits);
     if ((long long)tiles * a.k_splits <= ST_FEW_WORKGROUPS)
         gemm_stream_kernel<TOut, EPI, 512, 4><<<grid, 4 * LLMS_WAVE, 0, stream>>>(a);
-    else if ((long long)tiles * a.k_splits <= 4 * ST_FEW_WORKGROUPS)
+    else if ((long long)tiles * a.k_splits <= 3 * ST_FEW_WORKGROUPS && a.M <= 16)
         gemm_stream_kernel<TOut, EPI, 128, 8><<<grid, 8 * LLMS_WAVE, 0, stream>>>(a);
     else
         gemm_stream_kernel<TOut, EPI, 128, 4><<<grid, 4 * LLMS_WAVE, 0, stream>>>(a);
