@@ -28,9 +28,13 @@
 
 #include <algorithm>
 #include <mutex>
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+// 16 bytes on their way from memory to LDS, as a vector the compiler keeps in registers (an array of two uint4, a
+// struct, that is filled in one place and emptied in another it copied through memory)
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 
@@ -618,7 +622,13 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
     static_assert(WB == 4, "a wave per group of 8 keys: 4 to a tile");
     constexpr int PER_LANE = (D + LLMS_WAVE - 1) / LLMS_WAVE;  // 16-byte pieces of a group per lane (keys and values alike)
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
-    uint4 kreg[PER_LANE], vreg[PER_LANE];
+    // Rounds between asking for a group and putting it into LDS: one where the keys of a KV head stay in L2, two
+    // with wide heads (a head's keys and values are then megabytes, the trip goes to memory and takes longer than a
+    // round); each round in flight has registers of its own.
+    constexpr int AHEAD = DB > 4 ? 2 : 1;
+    u32x4 kreg0[PER_LANE], vreg0[PER_LANE], kreg1[PER_LANE], vreg1[PER_LANE];  // (the second set only with AHEAD == 2)
+    constexpr std::integral_constant<int, 0> SET0{};
+    constexpr std::integral_constant<int, 1> SET1{};
     int page_ahead = 0;
     auto group_key_of = [&](int j0) { return min(j0 + 8 * wave_s, p_max & ~7); };  // first key of this wave's group
     // (the block table does not change while the kernel runs: read as constant memory, which is what lets the
@@ -627,18 +637,24 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
     typedef const int __attribute__((address_space(4))) * ConstInts;
     const ConstInts table_c = (ConstInts)(uintptr_t)table;
     auto ask_pages = [&](int j0) { page_ahead = table_c[block_of(group_key_of(j0))]; };
-    auto load_round = [&](int j0) {  // after ask_pages(j0)
+    // (the register set is named by a type, std::integral_constant<int, 0 or 1>: an array passed by reference would
+    // be kept in memory by the compiler)
+    auto load_round = [&](int j0, auto set) __attribute__((always_inline)) {  // after ask_pages(j0)
+        auto& kreg = *[&]() { if constexpr (decltype(set)::value == 1) return &kreg1; else return &kreg0; }();
+        auto& vreg = *[&]() { if constexpr (decltype(set)::value == 1) return &vreg1; else return &vreg0; }();
         const int jg = group_key_of(j0), in_page = jg - block_of(jg) * a.block_size;
         const bf16* kg = page_ptr(k_base, page_ahead, page_stride) + (uint32_t)(in_page * D);
         const bf16* vg = page_ptr(v_base, page_ahead, page_stride) + (uint32_t)in_page;
 #pragma unroll
         for (int i = 0; i < PER_LANE; ++i) {
             const int p = min(lane + LLMS_WAVE * i, D - 1);  // (D % 64 != 0: the upper lanes repeat the last piece)
-            kreg[i] = *reinterpret_cast<const uint4*>(kg + 8 * p);
-            vreg[i] = *reinterpret_cast<const uint4*>(vg + (uint32_t)(p * a.block_size));
+            kreg[i] = *reinterpret_cast<const u32x4*>(kg + 8 * p);
+            vreg[i] = *reinterpret_cast<const u32x4*>(vg + (uint32_t)(p * a.block_size));
         }
     };
-    auto store_round = [&](int buf, int j0) {
+    auto store_round = [&](int buf, int j0, auto set) __attribute__((always_inline)) {
+        auto& kreg = *[&]() { if constexpr (decltype(set)::value == 1) return &kreg1; else return &kreg0; }();
+        auto& vreg = *[&]() { if constexpr (decltype(set)::value == 1) return &vreg1; else return &vreg0; }();
         const int jk = j0 + 8 * wave_s;                       // (not clamped: what the group stands for)
         const bool inside = jk >= lo_min && jk + 7 <= p_max;  // (the same for the wave)
         const int tile = wave_s / 4, kg4 = wave_s % 4;
@@ -646,11 +662,12 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
         for (int i = 0; i < PER_LANE; ++i) {
             const int p = lane + LLMS_WAVE * i;
             if (p < D) {
-                if (!inside) vreg[i] = keep_elements(vreg[i], lo_min - jk, p_max + 1 - jk);
+                uint4 values = make_uint4(vreg[i][0], vreg[i][1], vreg[i][2], vreg[i][3]);
+                if (!inside) values = keep_elements(values, lo_min - jk, p_max + 1 - jk);
                 const int q = p / KCH, ch = p % KCH;             // key 8 kg4 + q of the tile = 8a + 4u + b2
                 const int row = (q >> 2) * 16 + kg4 * 4 + (q & 3);  // -> row 16u + 4a + b2
-                k_lds[(buf * TW + tile) * K_TILE + row * KROW + ch] = kreg[i];
-                v_lds[(buf * TW + tile) * V_TILE + p * 4 + kg4] = vreg[i];  // [dimension][4 chunks of 8 keys]
+                *reinterpret_cast<u32x4*>(&k_lds[(buf * TW + tile) * K_TILE + row * KROW + ch]) = kreg[i];
+                v_lds[(buf * TW + tile) * V_TILE + p * 4 + kg4] = values;  // [dimension][4 chunks of 8 keys]
             }
         }
     };
@@ -658,33 +675,39 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
     const int per_split = (n_rounds + n_splits - 1) / n_splits;
     const int r_lo = split * per_split, r_hi = min(n_rounds, r_lo + per_split);  // this workgroup's rounds (maybe none)
     auto first_key = [&](int r) { return j_begin + 32 * TW * r; };
+    // round r_lo + i is fetched into register set i % AHEAD and goes into LDS buffer i % 2
     ask_pages(first_key(r_lo));
-    load_round(first_key(r_lo));
+    load_round(first_key(r_lo), SET0);
     ask_pages(first_key(r_lo + 1));
-    store_round(0, first_key(r_lo));
+    if (AHEAD == 2) {
+        load_round(first_key(r_lo + 1), SET1);
+        ask_pages(first_key(r_lo + 2));
+    }
+    store_round(0, first_key(r_lo), SET0);
     // The queries have arrived by now (they were asked for before the first round, which has just been stored).
     // Saying so here, outside the loop, keeps the wait for them out of it: inside, a wait for loads from memory
-    // would also wait for the round that is being fetched ahead.
+    // would also wait for the rounds that are being fetched ahead.
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
         for (int s = 0; s < KS; ++s)
             asm volatile("" : "+v"(qf[cg][s].x), "+v"(qf[cg][s].y), "+v"(qf[cg][s].z), "+v"(qf[cg][s].w));
-    load_round(first_key(r_lo + 1));
-    ask_pages(first_key(r_lo + 2));
+    load_round(first_key(r_lo + AHEAD), SET0);
+    ask_pages(first_key(r_lo + AHEAD + 1));
     __syncthreads();
-    for (int r = r_lo; r < r_hi; ++r) {
-        const int buf = (r - r_lo) & 1, j0 = j_begin + 32 * (TW * r + twin);  // this wave's tile of the round
+    // One round: `buf` is its LDS buffer, `set` names the registers that hold the round after it.
+    auto one_round = [&](int r, int buf, auto set) __attribute__((always_inline)) {
+        const int j0 = j_begin + 32 * (TW * r + twin);  // this wave's tile of the round
         const bool busy = wave_on && j0 <= w_pmax;  // (a tile beyond the wave's last position adds nothing)
-        // the next round into the other buffer (last read before the previous barrier), the round after that asked
-        // for, and the pages of the one after that: by the twins before they read their fragments from LDS, by the
-        // others after their tile, so that the two waves of a SIMD are not at the same stage at the same time (one
-        // multiplies while the other computes exponentials) and the reads of the one half of the waves have LDS to
-        // themselves while the other half still fetches
+        // the next round into the other buffer (last read before the previous barrier), a later one asked for, and the
+        // pages of the one after that: by the twins before they read their fragments from LDS, by the others after
+        // their tile, so that the two waves of a SIMD are not at the same stage at the same time (one multiplies
+        // while the other computes exponentials) and the reads of the one half of the waves have LDS to themselves
+        // while the other half still fetches
         auto fetch_ahead = [&]() {
-            if (r + 1 < r_hi) store_round(buf ^ 1, first_key(r + 1));
-            load_round(first_key(r + 2));
-            ask_pages(first_key(r + 3));
+            if (r + 1 < r_hi) store_round(buf ^ 1, first_key(r + 1), set);
+            load_round(first_key(r + 1 + AHEAD), set);
+            ask_pages(first_key(r + 2 + AHEAD));
         };
         if (TWIN && twin == 1) fetch_ahead();
         uint4 kf[2][KS], vf[DB];
@@ -712,6 +735,12 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
         }
         if (TWIN && twin == 0) fetch_ahead();
         __syncthreads();
+    };
+    // two rounds per turn, so that buffers and register sets are known by name: round r_lo + i goes into LDS from
+    // set i % AHEAD, which then takes round i + AHEAD
+    for (int r = r_lo; r < r_hi; r += 2) {
+        one_round(r, 0, std::integral_constant<int, AHEAD - 1>{});
+        if (r + 1 < r_hi) one_round(r + 1, 1, SET0);
     }
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg) l_run[cg] = column_sum(l_run[cg]);  // (every lane kept its own share of its column's sum)
