@@ -113,7 +113,8 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(TOut* __restrict__ C, co
     const int tid = threadIdx.x, wave = tid / LLMS_WAVE, lane = tid % LLMS_WAVE;
     const int wm = (wave % 2) * 64, wn = (wave / 2) * 64;
     const int l32 = lane % 32, g = lane / 32;
-    const uint4 zero = make_uint4(0, 0, 0, 0);
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;  // a struct (uint4) held in an array is copied
+    const u32x4 zero = {0, 0, 0, 0};                              // through private memory by the compiler
 
     f32x16 acc[2][2];
 #pragma unroll
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(TOut* __restrict__ C, co
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     // staging: 512 chunks of 8 elements per operand tile, two per thread
-    uint4 ra[2], rb[2];
+    u32x4 ra[2], rb[2];
     const int crow[2] = {tid / 4, (tid + 256) / 4};
     const int ckc = (tid % 4) * 8;
     auto load_global = [&](int k0) {
@@ -132,15 +133,15 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(TOut* __restrict__ C, co
         for (int c = 0; c < 2; ++c) {
             const int k = k0 + ckc;
             const int am = m0 + crow[c], wn_ = n0 + crow[c];
-            ra[c] = (am < M && k < K) ? *reinterpret_cast<const uint4*>(A + (size_t)am * lda + k) : zero;
-            rb[c] = (wn_ < N && k < K) ? *reinterpret_cast<const uint4*>(W + (size_t)wn_ * K + k) : zero;
+            ra[c] = (am < M && k < K) ? *reinterpret_cast<const u32x4*>(A + (size_t)am * lda + k) : zero;
+            rb[c] = (wn_ < N && k < K) ? *reinterpret_cast<const u32x4*>(W + (size_t)wn_ * K + k) : zero;
         }
     };
     auto store_lds = [&](int buf) {
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
-            *reinterpret_cast<uint4*>(&As[buf][crow[c] * TL_LD + ckc]) = ra[c];
-            *reinterpret_cast<uint4*>(&Bs[buf][crow[c] * TL_LD + ckc]) = rb[c];
+            *reinterpret_cast<u32x4*>(&As[buf][crow[c] * TL_LD + ckc]) = ra[c];
+            *reinterpret_cast<u32x4*>(&Bs[buf][crow[c] * TL_LD + ckc]) = rb[c];
         }
     };
 
