@@ -225,32 +225,76 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const float* __restrict__
 // bfloat16, head_dim % 16 == 0: the token's head_dim/2 sines and cosines are computed once per workgroup (the angle
 // depends on the token and on i only; computed per element they cost more than the kernel's memory traffic); a
 // thread takes 8 consecutive pairs (i .. i+7 and their partners at + head_dim/2) of one head with 16-byte loads and
-// stores; values leave in 16-byte reads and single stores (transposed in the page).
+// stores.  A workgroup is a chain of trips to memory (slot and position, the row, the run's slots, the values), so
+// the row's first pieces are asked for before the angles are worked out, and a head's pieces while the head
+// before it is rotated.
+//
+// Values: a page holds them transposed (a dimension's keys side by side), so a token alone leaves them in 2-byte
+// stores.  G tokens (16, or 8 where the page size is no multiple of 16; 0: never) that lie side by side in one page,
+// the first at a multiple of G, are a run: the run's workgroups share its KV heads out, and for a head a workgroup
+// brings the G tokens' values through LDS, so that every thread stores 16 bytes of one dimension and a wave's
+// stores are one contiguous piece where the page is G tokens wide.  Every workgroup of a run finds the same answer
+// from the same G slots.
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+#define ROPE_TILE_PAD 8  // elements between the rows of the LDS tile, so that a row starts at a multiple of 16 bytes
+
+template <int G>
 __global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restrict__ qkv, const float* __restrict__ inv_freq,
                                                                   const int* __restrict__ positions,
                                                                   const int* __restrict__ slots, bf16* __restrict__ k_pool,
                                                                   bf16* __restrict__ v_pool, int n_tokens, int n_heads,
                                                                   int n_kv_heads, int head_dim, int block_size) {
-    // Workgroups go round the 8 XCDs; 16 consecutive tokens (whose values are neighbours in a page's rows, 2 bytes
-    // each) go to one XCD, so that its L2 collects them into whole pieces before they are written back.
+    // Workgroups go round the 8 XCDs; 16 consecutive tokens go to one XCD, so that what they write into the same
+    // lines of a page meets in one L2.
     const int xcd = blockIdx.x % 8, place = blockIdx.x / 8;
     const int n = (place / 16) * 128 + xcd * 16 + place % 16;
     if (n >= n_tokens) return;
+    const int tid = threadIdx.x;
     const int half = head_dim / 2, chunks = half / 8;
     const int row_width = (n_heads + 2 * n_kv_heads) * head_dim;
     bf16* row = qkv + (size_t)n * row_width;
     const int slot = slots ? slots[n] : -1;
     const int page = slot >= 0 ? slot / block_size : 0;
     const int off = slot >= 0 ? slot % block_size : 0;
-    const int c = threadIdx.x % chunks, h0 = threadIdx.x / chunks, h_step = blockDim.x / chunks;
-    // the token's head_dim/2 angles once per workgroup (their sines and cosines are most of this kernel's arithmetic)
-    extern __shared__ float angles[];  // [half] sines, [half] cosines
+    const int c = tid % chunks, h0 = tid / chunks, h_step = blockDim.x / chunks;
+    const int rot_heads = n_heads + n_kv_heads;
+    const bool rotates = h0 < h_step && h0 < rot_heads;  // (threads past the last whole group of `chunks` have no head)
+    u32x4 av = {0, 0, 0, 0}, bv = {0, 0, 0, 0};
+    if (rotates) {
+        const bf16* x = row + (size_t)h0 * head_dim + 8 * c;
+        av = *reinterpret_cast<const u32x4*>(x);
+        bv = *reinterpret_cast<const u32x4*>(x + half);
+    }
+
+    extern __shared__ float angles[];  // [half] sines, [half] cosines, then the tile of values [G][head_dim + pad]
+    __shared__ int run_found;
+    // is this token part of a run?  (lead: the run's first token; the same for all of the workgroup)
+    const int lead = n - (G > 0 ? off % G : 0);
+    const bool may_run = G > 0 && slot >= 0 && lead >= 0 && lead + G <= n_tokens;
+    if (tid < 64) {  // (the first wave)
+        bool follows = true;
+        if (may_run && tid < G) follows = slots[lead + tid] == slot - off % (G > 0 ? G : 1) + tid;
+        const bool all_follow = __ballot(follows) == __ballot(true);
+        if (tid == 0) run_found = may_run && all_follow;
+    }
     if (inv_freq) {
         const float pos = (float)positions[n];
-        for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &angles[i], &angles[half + i]);
-        __syncthreads();
+        for (int i = tid; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &angles[i], &angles[half + i]);
     }
-    if (h0 < h_step) {
+    __syncthreads();
+    const bool in_run = run_found != 0;
+
+    // the values of the run's first head for this workgroup, asked for before the rotation
+    constexpr int GG = G > 0 ? G : 1;
+    const int pieces = head_dim / 8;  // 16-byte pieces of a head
+    const int my_head = n - lead;      // this workgroup takes the run's KV heads my_head, my_head + G, ...
+    const bf16* v_lead = qkv + (size_t)lead * row_width + (size_t)(n_heads + n_kv_heads) * head_dim;
+    u32x4 v_first = {0, 0, 0, 0};
+    if (in_run && my_head < n_kv_heads && tid < GG * pieces)
+        v_first = *reinterpret_cast<const u32x4*>(v_lead + (size_t)(tid / pieces) * row_width + (size_t)my_head * head_dim +
+                                                  8 * (tid % pieces));
+
+    if (rotates) {
         float sn[8], cs[8];
         if (inv_freq) {
 #pragma unroll
@@ -259,84 +303,79 @@ __global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restri
                 cs[e] = angles[half + 8 * c + e];
             }
         }
-        const int rot_heads = n_heads + n_kv_heads;
         for (int h = h0; h < rot_heads; h += h_step) {
-            const bool is_key = h >= n_heads;
-            if (is_key && k_pool != nullptr && slot < 0) continue;  // a key with nowhere to go
-            bf16* x = row + (size_t)h * head_dim + 8 * c;
-            const uint4 av = *reinterpret_cast<const uint4*>(x), bv = *reinterpret_cast<const uint4*>(x + half);
-            const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
-            uint32_t ra[4] = {aw[0], aw[1], aw[2], aw[3]}, rb[4] = {bw[0], bw[1], bw[2], bw[3]};
-            if (inv_freq) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float lo_a[2], lo_b[2];
-#pragma unroll
-                    for (int u = 0; u < 2; ++u) {
-                        const float a = bf16_bits_to_f32((uint16_t)(u ? aw[j] >> 16 : aw[j] & 0xffffu));
-                        const float b = bf16_bits_to_f32((uint16_t)(u ? bw[j] >> 16 : bw[j] & 0xffffu));
-                        lo_a[u] = a * cs[2 * j + u] - b * sn[2 * j + u];
-                        lo_b[u] = b * cs[2 * j + u] + a * sn[2 * j + u];
-                    }
-                    ra[j] = pack_bf16x2(lo_a[0], lo_a[1]);
-                    rb[j] = pack_bf16x2(lo_b[0], lo_b[1]);
-                }
+            u32x4 a_next = {0, 0, 0, 0}, b_next = {0, 0, 0, 0};
+            if (h + h_step < rot_heads) {
+                const bf16* x_next = row + (size_t)(h + h_step) * head_dim + 8 * c;
+                a_next = *reinterpret_cast<const u32x4*>(x_next);
+                b_next = *reinterpret_cast<const u32x4*>(x_next + half);
             }
-            bf16* dst = x;
-            if (is_key && k_pool != nullptr)
-                dst = k_pool + (((size_t)page * n_kv_heads + (h - n_heads)) * block_size + off) * head_dim + 8 * c;
-            *reinterpret_cast<uint4*>(dst) = make_uint4(ra[0], ra[1], ra[2], ra[3]);
-            *reinterpret_cast<uint4*>(dst + half) = make_uint4(rb[0], rb[1], rb[2], rb[3]);
+            const bool is_key = h >= n_heads;
+            if (!(is_key && k_pool != nullptr && slot < 0)) {  // (else: a key with nowhere to go)
+                u32x4 ra = av, rb = bv;
+                if (inv_freq) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        float lo_a[2], lo_b[2];
+#pragma unroll
+                        for (int u = 0; u < 2; ++u) {
+                            const float a = bf16_bits_to_f32((uint16_t)(u ? av[j] >> 16 : av[j] & 0xffffu));
+                            const float b = bf16_bits_to_f32((uint16_t)(u ? bv[j] >> 16 : bv[j] & 0xffffu));
+                            lo_a[u] = a * cs[2 * j + u] - b * sn[2 * j + u];
+                            lo_b[u] = b * cs[2 * j + u] + a * sn[2 * j + u];
+                        }
+                        ra[j] = pack_bf16x2(lo_a[0], lo_a[1]);
+                        rb[j] = pack_bf16x2(lo_b[0], lo_b[1]);
+                    }
+                }
+                bf16* dst = row + (size_t)h * head_dim + 8 * c;
+                if (is_key && k_pool != nullptr)
+                    dst = k_pool + (((size_t)page * n_kv_heads + (h - n_heads)) * block_size + off) * head_dim + 8 * c;
+                *reinterpret_cast<u32x4*>(dst) = ra;
+                *reinterpret_cast<u32x4*>(dst + half) = rb;
+            }
+            av = a_next;
+            bv = b_next;
         }
     }
-    // Values.  A page holds them transposed (a dimension's keys side by side), so a token alone leaves in 2-byte
-    // stores.  Eight tokens that lie side by side in one page (a prompt's: slots lead .. lead + 7, the first a
-    // multiple of 8) are stored by the workgroup of the first of them instead, 8 x 8 pieces turned in registers,
-    // 16 bytes per store.  Every workgroup of such a group finds the same answer from the same eight slots.
-    const int lead = n & ~7;
-    bool side_by_side = false;
-    if (slots && lead + 7 < n_tokens && block_size % 8 == 0 && ((uintptr_t)v_pool % 16) == 0) {
-        const int s0 = slots[lead];
-        side_by_side = s0 >= 0 && s0 % 8 == 0;
-#pragma unroll
-        for (int j = 1; j < 8; ++j) side_by_side = side_by_side && slots[lead + j] == s0 + j;
-    }
-    if (side_by_side) {
-        if (n != lead) return;
-        const int page8 = slot / block_size, off8 = slot % block_size;  // (n == lead: its own slot)
-        const bf16* v0 = row + (size_t)(n_heads + n_kv_heads) * head_dim;
-        for (int t = threadIdx.x; t < n_kv_heads * head_dim / 8; t += blockDim.x) {
-            uint32_t in[8][4];  // [token][pair of dimensions]
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint4 vv = *reinterpret_cast<const uint4*>(v0 + (size_t)j * row_width + 8 * t);
-                in[j][0] = vv.x; in[j][1] = vv.y; in[j][2] = vv.z; in[j][3] = vv.w;
+
+    if constexpr (G > 0) if (in_run) {
+        uint16_t* tile = reinterpret_cast<uint16_t*>(angles + head_dim);
+        const int pitch = head_dim + ROPE_TILE_PAD;
+        constexpr int PARTS = G / 8;  // 16-byte pieces of a dimension's G tokens
+        for (int kvh = my_head; kvh < n_kv_heads; kvh += GG) {  // (the same number of turns for the whole workgroup)
+            for (int t = tid; t < GG * pieces; t += blockDim.x) {
+                const int j = t / pieces, piece = t % pieces;
+                const u32x4 vv = (kvh == my_head && t == tid)
+                                     ? v_first
+                                     : *reinterpret_cast<const u32x4*>(v_lead + (size_t)j * row_width +
+                                                                       (size_t)kvh * head_dim + 8 * piece);
+                *reinterpret_cast<u32x4*>(&tile[j * pitch + 8 * piece]) = vv;
             }
-            const int kvh = (8 * t) / head_dim, d = (8 * t) % head_dim;
-            bf16* dst = v_pool + (((size_t)page8 * n_kv_heads + kvh) * head_dim + d) * block_size + off8;
+            __syncthreads();
+            bf16* head = v_pool + ((size_t)page * n_kv_heads + kvh) * head_dim * block_size + (off - off % GG);
+            for (int t = tid; t < head_dim * PARTS; t += blockDim.x) {
+                const int d = t / PARTS, part = t % PARTS;
+                u32x4 w;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {  // dimension d + i: the 8 tokens' values, two to a word
-                uint32_t w[4];
-#pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    const uint32_t a = in[2 * m][i / 2], b = in[2 * m + 1][i / 2];
-                    w[m] = (i & 1) ? ((a >> 16) | (b & 0xffff0000u)) : ((a & 0xffffu) | (b << 16));
-                }
-                *reinterpret_cast<uint4*>(dst + (size_t)i * block_size) = make_uint4(w[0], w[1], w[2], w[3]);
+                for (int m = 0; m < 4; ++m)
+                    w[m] = (uint32_t)tile[(8 * part + 2 * m) * pitch + d] |
+                           ((uint32_t)tile[(8 * part + 2 * m + 1) * pitch + d] << 16);
+                *reinterpret_cast<u32x4*>(head + (size_t)d * block_size + 8 * part) = w;
             }
+            __syncthreads();
         }
         return;
     }
     if (slot >= 0) {
         const bf16* v = row + (size_t)(n_heads + n_kv_heads) * head_dim;
-        for (int t = threadIdx.x; t < n_kv_heads * head_dim / 8; t += blockDim.x) {
-            const uint4 vv = *reinterpret_cast<const uint4*>(v + 8 * t);
-            const uint32_t vw[4] = {vv.x, vv.y, vv.z, vv.w};
+        for (int t = tid; t < n_kv_heads * head_dim / 8; t += blockDim.x) {
+            const u32x4 vv = *reinterpret_cast<const u32x4*>(v + 8 * t);
             const int kvh = (8 * t) / head_dim, d = (8 * t) % head_dim;
             bf16* dst = v_pool + (((size_t)page * n_kv_heads + kvh) * head_dim + d) * block_size + off;
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-                dst[(size_t)e * block_size].bits = (uint16_t)(e & 1 ? vw[e / 2] >> 16 : vw[e / 2] & 0xffffu);
+                dst[(size_t)e * block_size].bits = (uint16_t)(e & 1 ? vv[e / 2] >> 16 : vv[e / 2] & 0xffffu);
         }
     }
 }
@@ -450,9 +489,18 @@ int llms_rope_store(int dtype, void* qkv, const float* inv_freq, const int* posi
     if (dtype == 1 && head_dim % 16 == 0 && head_dim <= 4096 && ((uintptr_t)qkv % 16) == 0 &&
         (k_pool == nullptr || ((uintptr_t)k_pool % 16) == 0)) {
         const unsigned grid = (unsigned)((n_tokens + 127) / 128 * 128);
-        rope_store_bf16_vec_kernel<<<grid, 256, head_dim * sizeof(float), stream>>>(
-            (bf16*)qkv, inv_freq, positions, slots, (bf16*)k_pool, (bf16*)v_pool, n_tokens, n_heads, n_kv_heads, head_dim,
-            block_size);
+        // runs of tokens whose values go through LDS: as long as the page size allows, and the tile fits
+        const bool runs = slots && ((uintptr_t)v_pool % 16) == 0 && head_dim <= 1024;
+        const int run = !runs ? 0 : block_size % 16 == 0 ? 16 : block_size % 8 == 0 ? 8 : 0;
+        const size_t lds = head_dim * sizeof(float) + (size_t)run * (head_dim + ROPE_TILE_PAD) * sizeof(uint16_t);
+#define LLMS_ROPE_LAUNCH(G)                                                                                       \
+    rope_store_bf16_vec_kernel<G><<<grid, 256, lds, stream>>>((bf16*)qkv, inv_freq, positions, slots, (bf16*)k_pool, \
+                                                              (bf16*)v_pool, n_tokens, n_heads, n_kv_heads, head_dim, \
+                                                              block_size)
+        if (run == 16) LLMS_ROPE_LAUNCH(16);
+        else if (run == 8) LLMS_ROPE_LAUNCH(8);
+        else LLMS_ROPE_LAUNCH(0);
+#undef LLMS_ROPE_LAUNCH
         LLMS_LAUNCH_CHECK();
     }
     DISPATCH_DTYPE(dtype, rope_store_kernel<T><<<n_tokens, 256, 0, stream>>>(
