@@ -103,12 +103,14 @@ def test_rmsnorm_tiny_inputs_feel_eps():
         assert torch.allclose(out.cpu(), plain_llama.rms_norm(x, w, eps), atol=1e-6)
 
 
-@pytest.mark.parametrize("nh,nkv,d,bs", [(4, 2, 16, 16), (8, 8, 64, 8), (16, 2, 128, 32), (6, 3, 48, 24), (4, 4, 32, 4)])
+@pytest.mark.parametrize("nh,nkv,d,bs", [(4, 2, 16, 16), (8, 8, 64, 8), (16, 2, 128, 32), (6, 3, 48, 24), (4, 4, 32, 4),
+                                         (2, 20, 16, 16), (20, 20, 32, 64)])
 def test_rope_store_prompt_tokens_side_by_side(nh, nkv, d, bs):
-    """A prompt's tokens lie side by side in their pages: eight of them that start at a multiple of 8 are stored by
-    one workgroup, 16 bytes per dimension.  Runs that start off such a boundary, break in the middle (another page,
-    a token without a slot), or end before eight, and a second request behind the first, leave as single values:
-    every slot must hold its own token's values and nothing else may change."""
+    """A prompt's tokens lie side by side in their pages: 16 of them (8 where the page size is no multiple of 16) whose
+    first slot is a multiple of that are a run, whose workgroups share the KV heads out (fewer heads than tokens,
+    and more) and store 16 bytes per dimension.  Runs that start off such a boundary (in the page, and in the batch),
+    break in the middle (another page, a token without a slot), or end early, and a second request behind the first,
+    leave as single values: every slot must hold its own token's values and nothing else may change."""
     dtype = torch.bfloat16
     pages = 16
     # request a: 29 tokens from slot 3 of page 2 on through pages 5 and 1 (pages need not follow each other)
