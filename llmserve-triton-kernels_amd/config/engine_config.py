@@ -25,7 +25,9 @@ class EngineConfig:
     max_prefill_chunk: int | None = None  # longest portion of one prompt in one step
     max_model_len: int | None = None  # defaults to the model's max_position_embeddings
     seed: int = 0
-    use_graphs: bool = True  # replay steps from captured HIP graphs (decode-only steps; others when the host was their limit)
+    # replay steps from captured HIP graphs: decode-only steps, and steps with portions of prompts that are small
+    # enough for the host's launches to be their limit (a rule by sizes; a bucket of sizes is captured at its second use)
+    use_graphs: bool = True
 
     def validate(self) -> None:
         if self.dtype not in DTYPE_NAMES:
