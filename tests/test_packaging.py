@@ -31,3 +31,15 @@ def test_top_level_names():
 
     for name in ("LLM", "EngineConfig", "SamplingParams", "GenerationResult"):
         assert getattr(llmserve, name).__name__ == name
+
+
+def test_bench_refuses_more_than_one_gpu_with_one_line():
+    """The measurement program runs one GPU: asked for more it says so in one line and exits with 2, before it
+    touches a device."""
+    import subprocess
+    import sys
+
+    done = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2", "--steps", "1", "--warmup", "0"],
+                          capture_output=True, text=True, timeout=120)
+    assert done.returncode == 2
+    assert len(done.stdout.strip().splitlines()) == 1 and "--gpus 2" in done.stdout
