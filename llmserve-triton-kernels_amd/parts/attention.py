@@ -138,8 +138,10 @@ class Attention(Mixer):
         takes every other tile of keys for the same tokens, and with two such workgroups per CU the long blocks
         and the short ones even out.  With exactly one per CU sharing pays only behind a long prefix (measured:
         from about 3,000 keys on).  A short portion behind a long prefix has few blocks and many keys: its keys
-        are shared out until the chip holds about two workgroups of 4 waves per CU, 8 tiles of keys each at
-        least."""
+        are shared out, 8 tiles of keys a workgroup at least (16 where the blocks alone are half a chip), up to
+        about two workgroups of 4 waves per CU, and not in more than 4 once the blocks alone are a quarter of a
+        chip (measured on portions of 16 to 256 tokens behind 256 to 4,032 keys, at head sizes 64 and 128: the
+        merge kernel's work grows with blocks times shares)."""
         if self.window:
             return 1
         g = self.num_heads // self.num_kv_heads
@@ -151,7 +153,9 @@ class Attention(Mixer):
             return 1
         if workgroups >= 256:
             return 4 if tiles >= 96 else 1
-        return max(1, min(512 // max(workgroups, 1), tiles // 8, 8))
+        per_share = 16 if workgroups >= 128 else 8
+        most = 4 if workgroups >= 64 else 8
+        return max(1, min(512 // max(workgroups, 1), tiles // per_share, most))
 
     def decode_arrangement(self, n_requests: int, max_context: int) -> tuple[int, int]:
         """(workgroups per request and KV head, waves per workgroup) for decoding.  The waves of a
