@@ -851,10 +851,17 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(bf16* __restrict__ out,
 #define PROMPT_WB 4  // waves per block of tokens (2 was tried with 2 column groups each: slower)
 #define PROMPT_FULL_CHIP 256  // workgroups below which one column group per wave is kept
 
+#define PROMPT_TWIN_MAX_DB 12  // widest head (in blocks of 16 dimensions) whose 8 waves with twins fit the registers
+
 template <int DB, int CG>
 static void launch_prompt_cg(dim3 grid, bool twin, const AttnArgs& a, hipStream_t stream) {
-    if (twin) attn_prompt_kernel<DB, true, CG, PROMPT_WB><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
-    else attn_prompt_kernel<DB, false, CG, PROMPT_WB><<<grid, PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
+    if constexpr (DB <= PROMPT_TWIN_MAX_DB) {  // (wider heads are never given twins, so those kernels are not built)
+        if (twin) {
+            attn_prompt_kernel<DB, true, CG, PROMPT_WB><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
+            return;
+        }
+    }
+    attn_prompt_kernel<DB, false, CG, PROMPT_WB><<<grid, PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
 }
 
 // Few tokens (decoding): small workgroups, so that the merge reaches many CUs; many tokens: 256 threads each.
@@ -972,7 +979,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     } else {
         // twins (8 waves, two tiles a round) where a workgroup per CU is left that way; wider heads would not fit
         // the registers of 8 waves, a window or splits have their own arrangement
-        bool twin = window == 0 && head_dim <= 192 && num_splits == 1;
+        bool twin = window == 0 && head_dim <= 16 * PROMPT_TWIN_MAX_DB && num_splits == 1;
         auto grid_for = [&](int cg) {
             const int per_block = PROMPT_WB * cg;  // column groups of a block of tokens
             return dim3((groups + per_block - 1) / per_block * num_splits, n_kv_heads * HB, n_seqs);

@@ -46,3 +46,32 @@ def test_library_names_follow_the_headers_a_source_includes(tmp_path, monkeypatc
     assert build._source_hash("one") != one and build._source_hash("two") == two
     (tmp_path / "common.h").write_text("#pragma once\n// more\n")
     assert build._source_hash("two") != two
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None and not build.Path("/opt/rocm/bin/hipcc").exists(),
+                    reason="hipcc is needed to compile")
+@pytest.mark.parametrize("name,kernels,most_bytes", [
+    ("gemm_stream", ("gemm_stream_kernel", "gemm_slices_kernel"), 0),
+    ("attention_mfma", ("attn_prompt_kernel", "attn_mfma_kernel"), 64),
+])
+def test_streaming_kernels_hold_what_they_fetch_in_registers(tmp_path, name, kernels, most_bytes):
+    """What a lane has fetched and not yet used must stay in registers.  The compiler may lower an array of a
+    struct (uint4) that one place fills and another empties to copies through the lane's private memory, which puts
+    a wait behind every load: twice the time, and no numerics test sees it.  The kernels' private segment (in the
+    code object's metadata) is empty, or holds the few registers spilt by the kernels that are compiled for two
+    workgroups per CU."""
+    import re
+    import subprocess
+
+    flags = [f for f in build.HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    out = tmp_path / f"{name}.s"
+    subprocess.run([build._hipcc(), *flags, f"-I{build.CSRC_DIR}", "-S", "--cuda-device-only",
+                    str(build.CSRC_DIR / f"{name}.hip"), "-o", str(out)], check=True, capture_output=True, timeout=600)
+    text = out.read_text()
+    sizes = {}
+    for block in text.split("  - .agpr_count:")[1:]:  # one block of metadata per kernel
+        kernel = re.search(r"\.name:\s+(\S+)", block).group(1)
+        sizes[kernel] = int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", block).group(1))
+    checked = {k: v for k, v in sizes.items() if any(want in k for want in kernels)}
+    assert checked, sorted(sizes)
+    assert {k: v for k, v in checked.items() if v > most_bytes} == {}
