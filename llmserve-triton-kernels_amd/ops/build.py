@@ -41,7 +41,7 @@ HIPCC_FLAGS = [
 # built when something is first sampled).
 GROUPS = {
     "float32": ("elementwise", "gemm", "attention"),
-    "bfloat16": ("elementwise", "gemm", "attention", "gemm_stream", "attention_mfma"),
+    "bfloat16": ("elementwise", "gemm", "attention", "gemm_stream", "gemm_decode", "attention_mfma"),
 }
 
 

@@ -377,6 +377,116 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
     return parts if k_splits != 1 else out
 
 
+_cu_count: dict[int, int] = {}
+
+
+def compute_units(dev: torch.device) -> int:
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    if index not in _cu_count:
+        _cu_count[index] = torch.cuda.get_device_properties(index).multi_processor_count
+    return _cu_count[index]
+
+
+GEMM_DECODE_MAX_ROWS = 16
+GEMM_DECODE_MAX_K = 16 * 3 * 128  # 16 waves with up to three chunks of 128 each
+_GEMM_DECODE_LDS_FOR_ROWS = 160 * 1024 - 16 * 4096 - 1024  # what the waves' tiles leave of a compute unit's LDS
+
+
+def gemm_decode_fits(m: int, k: int) -> bool:
+    """Whether m rows of k elements fit ops.gemm_decode: the rows (8 of them up to 8 rows, else 16) stay in LDS."""
+    if not (0 < m <= GEMM_DECODE_MAX_ROWS and 0 < k <= GEMM_DECODE_MAX_K):
+        return False
+    return (8 if m <= 8 else 16) * (-(-k // 128) * 256 + 16) <= _GEMM_DECODE_LDS_FOR_ROWS
+
+
+def gemm_decode_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ops.gemm_decode takes x [M, K] against w [N, K]."""
+    return x.dtype == torch.bfloat16 and gemm_decode_fits(x.shape[0], x.shape[1]) and gemm_bf16_supported(x, w)
+
+
+def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, *,
+                norm: tuple[torch.Tensor, float] | None = None, swiglu: bool = False, rope: dict | None = None,
+                residual: torch.Tensor | None = None) -> torch.Tensor:
+    """The product for up to 16 bfloat16 rows with one workgroup per compute unit, and what surrounds it fused in.
+
+    norm = (weight [K], eps): the rows of x are replaced by RMSNorm(x) * weight on the way in.
+    plain:     out[M, N] = x w^T (+ bias), bfloat16 or float32.
+    swiglu:    w = [gate; up] ([2I, K]); out[M, I] = silu(gate) * up.
+    rope = dict(n_heads, n_kv_heads, head_dim, inv_freq | None, positions, slots | None, k_pool, v_pool,
+               block_size): w = [q; k; v]; out[M, n_heads * head_dim] = rotated q; rotated k and v are stored at
+               the tokens' cache slots.
+    residual:  residual[M, N] += x w^T (+ bias) in place (32-bit sum of the rounded product and the row, rounded
+               once); `out` is not used and `residual` is returned."""
+    dev = _dev(out, x, w, bias, residual, norm[0] if norm else None)
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise ValueError("x must be 2-d with unit inner stride")
+    _rows(w, "w", x.shape[1])
+    m, k = x.shape
+    n = w.shape[0]
+    if not 0 < m <= GEMM_DECODE_MAX_ROWS:
+        raise ValueError(f"gemm_decode takes 1..{GEMM_DECODE_MAX_ROWS} rows")
+    if not gemm_decode_fits(m, k):
+        raise ValueError(f"gemm_decode keeps the rows of x in LDS: {m} rows of K = {k} do not fit (K up to "
+                         f"{GEMM_DECODE_MAX_K}, and up to 2,944 with more than 8 rows)")
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise ValueError("gemm_decode takes bfloat16 operands")
+    if not gemm_bf16_supported(x, w):
+        raise ValueError(f"gemm_decode needs K ({k}) and the row stride of x ({x.stride(0)}) to be multiples of 8 "
+                         "and 16-byte aligned operands")
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous bfloat16 vector of N elements")
+    if sum((swiglu, rope is not None, residual is not None)) > 1:
+        raise ValueError("one epilogue at a time")
+    norm_weight, eps = None, 0.0
+    if norm is not None:
+        norm_weight, eps = norm
+        if norm_weight.dtype != torch.bfloat16 or norm_weight.numel() != k or not norm_weight.is_contiguous() \
+                or norm_weight.data_ptr() % 16:
+            raise ValueError("the norm's weight must be a contiguous, 16-byte aligned bfloat16 vector of K elements")
+    epilogue, inter, cols = 0, 0, n
+    r = dict(n_heads=0, n_kv_heads=0, head_dim=0, block_size=0, inv_freq=None, positions=None, slots=None,
+             k_pool=None, v_pool=None)
+    if swiglu:
+        if n % 2 or bias is not None:
+            raise ValueError("the gated epilogue needs an even number of weight rows and no bias")
+        epilogue, inter, cols = 1, n // 2, n // 2
+    elif rope is not None:
+        r.update(rope)
+        nh, nkv, d = r["n_heads"], r["n_kv_heads"], r["head_dim"]
+        if d % 2 or n != (nh + 2 * nkv) * d:
+            raise ValueError("the rotary epilogue needs an even head_dim and N = (heads + 2 kv heads) * head_dim")
+        _i32(r["positions"], "positions", m)
+        if r["inv_freq"] is not None:
+            _f32(r["inv_freq"], "inv_freq", d // 2)
+        if r["slots"] is not None:
+            _i32(r["slots"], "slots", m)
+            bs, kp, vp = r["block_size"], r["k_pool"], r["v_pool"]
+            pages = kp.shape[0]
+            if (tuple(kp.shape) != (pages, nkv, bs, d) or tuple(vp.shape) != (pages, nkv, d, bs)
+                    or not kp.is_contiguous() or not vp.is_contiguous() or kp.dtype != x.dtype or vp.dtype != x.dtype):
+                raise ValueError("pools do not have the cache layout [pages, kv, block, D] / [pages, kv, D, block]")
+        _dev(x, r["inv_freq"], r["positions"], r["slots"], r["k_pool"], r["v_pool"])
+        epilogue, cols = 2, nh * d
+    elif residual is not None:
+        if (residual.dim() != 2 or residual.stride(1) != 1 or tuple(residual.shape) != (m, n)
+                or residual.dtype != torch.bfloat16):
+            raise ValueError(f"residual must be a bfloat16 [{m}, {n}] tensor with unit inner stride")
+        epilogue = 3
+    if epilogue != 3:
+        if out is None or out.dim() != 2 or out.stride(1) != 1 or tuple(out.shape) != (m, cols):
+            raise ValueError(f"out must be 2-d [{m}, {cols}] with unit inner stride")
+        if out.dtype != torch.bfloat16 and not (epilogue == 0 and out.dtype == torch.float32):
+            raise ValueError("gemm_decode stores bfloat16 (the plain epilogue also float32)")
+    _check(load("gemm_decode").llms_gemm_decode(
+        c_int(1 if epilogue == 3 else _code(out)), c_int(epilogue), _ptr(None if epilogue == 3 else out),
+        c_int(0 if epilogue == 3 else out.stride(0)), _ptr(x), c_int(x.stride(0)), _ptr(w), _ptr(bias),
+        _ptr(norm_weight), c_float(eps), c_int(m), c_int(n), c_int(k), c_int(inter), c_int(r["n_heads"]),
+        c_int(r["n_kv_heads"]), c_int(r["head_dim"]), c_int(r["block_size"]), _ptr(r["inv_freq"]), _ptr(r["positions"]),
+        _ptr(r["slots"]), _ptr(r["k_pool"]), _ptr(r["v_pool"]), _ptr(residual),
+        c_int(residual.stride(0) if residual is not None else 0), c_int(compute_units(dev)), _stream(dev)), "gemm_decode")
+    return residual if epilogue == 3 else out
+
+
 SLICE_K = 512  # what one workgroup of gemm_slices takes of K
 
 

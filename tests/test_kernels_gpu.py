@@ -345,6 +345,132 @@ def test_gemm_stream_rotary_epilogue(nh, nkv, d, bs, theta, bias, m):
     assert torch.equal(q3, q) and (k3 == 7).all() and (v3 == 7).all()
 
 
+# ------------------------------------------------------------------ gemm_decode: one workgroup per compute unit
+@pytest.mark.parametrize("m,n,k", [(1, 16, 64), (3, 333, 96), (16, 2056, 2048), (7, 100, 5632), (9, 48, 176),
+                                   (8, 32000, 2048), (5, 2048, 4096), (8, 24, 5888), (2, 5000, 8), (12, 40, 2944)])
+def test_gemm_decode_plain(m, n, k):
+    x, w, b = rnd(m, k, seed=11).bfloat16(), rnd(n, k, seed=12).bfloat16(), rnd(n, seed=13).bfloat16()
+    ref = x.double() @ w.double().t() + b.double()
+    buf = torch.full((m * n + 64,), 7.0, device=DEV)
+    out = ops().gemm_decode(buf[32:-32].view(m, n), x.to(DEV), w.to(DEV), b.to(DEV))
+    assert (out.cpu().double() - ref).abs().max() <= 2e-6 * math.sqrt(k) * float(ref.abs().max())
+    assert torch.all(buf[:32] == 7.0) and torch.all(buf[-32:] == 7.0)
+    out = ops().gemm_decode(torch.empty(m, n, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV))
+    ref = x.double() @ w.double().t()
+    assert (out.float().cpu().double() - ref).abs().max() <= 2.0 ** -8 * float(ref.abs().max())
+    # rows of a larger tensor: the stride of x is not K
+    wide = torch.cat([x, rnd(m, 8, seed=33).bfloat16()], dim=1).to(DEV)
+    assert torch.equal(ops().gemm_decode(torch.empty(m, n, dtype=torch.bfloat16, device=DEV), wide[:, :k], w.to(DEV)), out)
+
+
+def test_gemm_decode_refuses_what_it_cannot_take():
+    x, w = rnd(17, 64).bfloat16().to(DEV), rnd(32, 64).bfloat16().to(DEV)
+    with pytest.raises(ValueError, match="1..16"):
+        ops().gemm_decode(torch.empty(17, 32, dtype=torch.bfloat16, device=DEV), x, w)
+    for rows, big in ((2, ops().GEMM_DECODE_MAX_K + 8), (9, 3072)):
+        with pytest.raises(ValueError, match="do not fit"):
+            ops().gemm_decode(torch.empty(rows, 32, dtype=torch.bfloat16, device=DEV), rnd(rows, big).bfloat16().to(DEV),
+                              rnd(32, big).bfloat16().to(DEV))
+    with pytest.raises(ValueError, match="one epilogue"):
+        ops().gemm_decode(torch.empty(2, 16, dtype=torch.bfloat16, device=DEV), x[:2], w, swiglu=True,
+                          residual=torch.empty(2, 32, dtype=torch.bfloat16, device=DEV))
+    assert not ops().gemm_decode_supported(x, w) and ops().gemm_decode_supported(x[:16], w)
+
+
+@pytest.mark.parametrize("m,n,k,eps", [(1, 64, 64, 1e-5), (8, 2560, 2048, 1e-5), (16, 333, 96, 1e-6), (5, 100, 4096, 1e-5),
+                                       (3, 48, 5888 - 8, 1e-6), (13, 200, 2560, 1e-5)])
+def test_gemm_decode_norms_its_rows_on_the_way_in(m, n, k, eps):
+    """RMSNorm in the prologue: the same as the norm kernel followed by the product (the sum of squares is added up
+    in another order, so the normed rows may differ by one rounding)."""
+    x = rnd(m, k, seed=41, scale=3.0).bfloat16()
+    nw = (1 + 0.1 * rnd(k, seed=42)).bfloat16()
+    w = rnd(n, k, seed=43, scale=0.1).bfloat16()
+    normed = plain_llama.rms_norm(x, nw, eps)
+    ref = normed.double() @ w.double().t()
+    out = ops().gemm_decode(torch.empty(m, n, device=DEV), x.to(DEV), w.to(DEV), norm=(nw.to(DEV), eps))
+    # a normed element may be rounded the other way: 2^-8 of it, times its weight, summed over K at random signs
+    tol = 2.0 ** -8 * float(normed.float().abs().max()) * float(w.float().abs().max()) * math.sqrt(k)
+    assert (out.cpu().double() - ref).abs().max() <= tol
+    # against the norm kernel and the plain product of this library
+    y = ops().rmsnorm(torch.empty(m, k, dtype=torch.bfloat16, device=DEV), x.to(DEV), nw.to(DEV), eps)
+    two = ops().gemm_decode(torch.empty(m, n, device=DEV), y, w.to(DEV))
+    assert (out - two).abs().max() <= tol
+    assert (out != two).float().mean() < 0.5  # mostly the same bits
+
+
+@pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96), (8, 1000, 4096), (3, 22, 2048)])
+def test_gemm_decode_gated_epilogue(m, inter, k):
+    """silu(gate) * up in the epilogue: the same bits as the product followed by the activation kernel."""
+    x = rnd(m, k, seed=16).bfloat16()
+    w = torch.cat([rnd(inter, k, seed=17, scale=0.2), rnd(inter, k, seed=18, scale=0.2)]).bfloat16()
+    g, u = plain_llama.linear(x, w[:inter]), plain_llama.linear(x, w[inter:])
+    ref = (plain_llama.silu(g) * u).float()
+    out = ops().gemm_decode(torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV), swiglu=True)
+    assert (out.float().cpu() - ref).abs().max() <= 2.0 ** -7 * float(ref.abs().max())
+    gu = ops().gemm_decode(torch.empty(m, 2 * inter, dtype=torch.bfloat16, device=DEV), x.to(DEV), w.to(DEV))
+    act = ops().silu_mul(torch.empty(m, inter, dtype=torch.bfloat16, device=DEV), gu)
+    assert torch.equal(act, out)
+
+
+@pytest.mark.parametrize("nh,nkv,d,bs,theta,bias,m", [(4, 2, 16, 16, 1e4, False, 5), (3, 1, 32, 8, 5e5, True, 5),
+                                                      (32, 4, 64, 16, 1e4, False, 8), (2, 2, 48, 8, None, True, 16),
+                                                      (5, 5, 128, 16, 1e4, True, 3), (6, 3, 80, 16, 1e6, False, 1)])
+def test_gemm_decode_rotary_epilogue(nh, nkv, d, bs, theta, bias, m):
+    """q/k/v projection with the rotation and the cache store in the epilogue: the same bits as the
+    projection followed by the rotation kernel."""
+    k, pages = 96, 12
+    n = (nh + 2 * nkv) * d
+    x, w = rnd(m, k, seed=23).bfloat16().to(DEV), rnd(n, k, seed=24, scale=0.3).bfloat16().to(DEV)
+    b = rnd(n, seed=25).bfloat16().to(DEV) if bias else None
+    gen = torch.Generator().manual_seed(35)
+    positions = torch.randint(0, 4096, (m,), generator=gen).to(torch.int32)
+    positions[0] = 0
+    positions = positions.to(DEV)
+    slots = torch.randperm(bs * pages, generator=gen)[:m].to(torch.int32)
+    slots[m // 2] = -1
+    slots = slots.to(DEV)
+    inv_freq = (1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV) if theta else None
+    pools = lambda: (torch.full((pages, nkv, bs, d), 7.0, dtype=torch.bfloat16, device=DEV),  # noqa: E731
+                     torch.full((pages, nkv, d, bs), 7.0, dtype=torch.bfloat16, device=DEV))
+    k1, v1 = pools()
+    qkv = ops().gemm_decode(torch.empty(m, n, dtype=torch.bfloat16, device=DEV), x, w, b)
+    ops().rope_store(qkv, inv_freq, positions, slots, k1, v1, nh, nkv, d, bs)
+    k2, v2 = pools()
+    rope = dict(n_heads=nh, n_kv_heads=nkv, head_dim=d, inv_freq=inv_freq, positions=positions, slots=slots,
+                k_pool=k2, v_pool=v2, block_size=bs)
+    q = ops().gemm_decode(torch.empty(m, nh * d, dtype=torch.bfloat16, device=DEV), x, w, b, rope=rope)
+    assert torch.equal(q, qkv[:, : nh * d]) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert (k2 != 7).any() and (v2 != 7).any() or m == 1
+    k3, v3 = pools()  # without slots only q is produced
+    q3 = ops().gemm_decode(torch.empty(m, nh * d, dtype=torch.bfloat16, device=DEV), x, w, b, rope=dict(rope, slots=None, k_pool=k3, v_pool=v3))
+    assert torch.equal(q3, q) and (k3 == 7).all() and (v3 == 7).all()
+
+
+@pytest.mark.parametrize("m,n,k,bias", [(1, 64, 64, False), (8, 2048, 2048, False), (8, 2048, 5632, True), (16, 333, 176, True),
+                                        (5, 4096, 4096, False), (11, 90, 2900 - 4, True)])
+def test_gemm_decode_residual_epilogue(m, n, k, bias):
+    """residual += x w^T: the rounded product added to the row in 32-bit and rounded once, as the norm kernel adds a
+    delta (same bits as product, then that kernel's residual output)."""
+    x, w = rnd(m, k, seed=51).bfloat16().to(DEV), rnd(n, k, seed=52, scale=0.1).bfloat16().to(DEV)
+    b = rnd(n, seed=53).bfloat16().to(DEV) if bias else None
+    wide = rnd(m, n + 8, seed=54, scale=2.0).bfloat16().to(DEV)
+    res = wide[:, :n]  # (a view: the row stride is not N)
+    before = res.clone()
+    delta = ops().gemm_decode(torch.empty(m, n, dtype=torch.bfloat16, device=DEV), x, w, b)
+    want = (before.float() + delta.float()).bfloat16()
+    got = ops().gemm_decode(None, x, w, b, residual=res)
+    assert got is res and torch.equal(res, want)
+    assert torch.equal(wide[:, n:].cpu(), rnd(m, n + 8, seed=54, scale=2.0).bfloat16()[:, n:])
+
+
+def test_gemm_decode_rows_do_not_depend_on_the_batch():
+    a, w = rnd(16, 2048, seed=14).bfloat16().to(DEV), rnd(320, 2048, seed=15).bfloat16().to(DEV)
+    nw = (1 + 0.1 * rnd(2048, seed=4)).bfloat16().to(DEV)
+    full = ops().gemm_decode(torch.empty(16, 320, device=DEV), a, w, norm=(nw, 1e-5))
+    one = ops().gemm_decode(torch.empty(1, 320, device=DEV), a[9:10].contiguous(), w, norm=(nw, 1e-5))
+    assert torch.equal(full[9:10], one)
+
+
 def test_gemm_bf16_rows_do_not_depend_on_the_batch():
     """A row's result is the same bits whatever else is in the batch (same kernel)."""
     a, w = rnd(40, 2048, seed=14).bfloat16().to(DEV), rnd(320, 2048, seed=15).bfloat16().to(DEV)
