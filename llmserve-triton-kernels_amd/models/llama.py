@@ -23,7 +23,8 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
     for i in range(cfg.num_hidden_layers):
         p = f"model.layers.{i}."
         layers.append(LayerSpec(
-            mixer=mixer, feed_forward=feed_forward, mixer_norm=norm, feed_forward_norm=norm, block="prenorm",
+            block="prenorm",
+            parts={"mixer": mixer, "feed_forward": feed_forward, "mixer_norm": norm, "feed_forward_norm": norm},
             weights={"mixer": p + "self_attn.", "feed_forward": p + "mlp.",
                      "mixer_norm": p + "input_layernorm.", "feed_forward_norm": p + "post_attention_layernorm."}))
     return ModelSpec(

@@ -16,8 +16,8 @@ import math
 import torch
 
 from ..ops import library as ops
-from .linear import few_rows, linear, linear_partial_sums
-from .registry import POSITION_ENCODINGS, DeferredNorm, Mixer, register_mixer
+from .linear import decode_product, few_rows, linear, linear_partial_sums
+from .registry import ADDED_IN_PLACE, POSITION_ENCODINGS, DeferredNorm, Mixer, register_mixer
 from .spec import PagedCacheSpec, ParamInfo
 
 
@@ -70,11 +70,11 @@ class Attention(Mixer):
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         view = batch.groups[cache.group_id]
         slots = view.slots if cache.store else None
-        to_a_norm = isinstance(x, DeferredNorm)  # the caller hands the result to a norm, which takes partial sums
+        deferred = x if isinstance(x, DeferredNorm) else None  # (then the result goes to a norm, which takes partial sums)
         q = self.project_few_rows(x, batch, cache, slots)
         if q is None:
-            if isinstance(x, DeferredNorm):
-                x = x.materialize()
+            if deferred is not None:
+                x = deferred.materialize()
             q = linear(x, self.qkv_weight, self.qkv_bias)  # q, k and v side by side; q is read in place
             fused = getattr(self.position, "rotate_and_store", None)
             if fused is not None:
@@ -86,15 +86,20 @@ class Attention(Mixer):
                                    cache.block_size)
         out = torch.empty((q.shape[0], nh * d), dtype=q.dtype, device=q.device)
         self.attend(out, q, cache, view, batch)
-        return (linear_partial_sums(out, self.o_weight) if to_a_norm else None) or linear(out, self.o_weight)
+        if deferred is not None and deferred.may_add_in_place and decode_product(out, self.o_weight):
+            ops.gemm_decode(None, out, self.o_weight, residual=deferred.residual)  # the residual sum in the epilogue
+            return ADDED_IN_PLACE
+        return (linear_partial_sums(out, self.o_weight) if deferred is not None else None) or linear(out, self.o_weight)
 
     def _few_rows_unfit(self, rows) -> bool:
-        return (rows.dtype != torch.bfloat16 or not few_rows(rows.shape[0], self.qkv_weight) or self.head_dim % 16 != 0
-                or not ops.gemm_bf16_supported(rows, self.qkv_weight))
+        if rows.dtype != torch.bfloat16 or self.head_dim % 16 != 0 or not ops.gemm_bf16_supported(rows, self.qkv_weight):
+            return True
+        return not (decode_product(rows, self.qkv_weight) or few_rows(rows.shape[0], self.qkv_weight))
 
     def project_few_rows(self, x, batch, cache, slots):
-        """With few bfloat16 rows one kernel does the projection, the rotation and the cache store:
-        ops.gemm_stream.  Returns the rotated queries, or None when that kernel does not apply."""
+        """With few bfloat16 rows one kernel does the projection, the rotation and the cache store
+        (ops.gemm_decode, which also norms its rows on the way in, or ops.gemm_stream).  Returns the rotated
+        queries, or None when neither kernel applies."""
         deferred = isinstance(x, DeferredNorm)
         rows = x.residual if deferred else x
         m = rows.shape[0]
@@ -103,13 +108,20 @@ class Attention(Mixer):
         frequencies = getattr(self.position, "rotary_frequencies", None)
         if frequencies is None and not getattr(self.position, "identity", False):
             return None  # a position encoding this kernel does not know
-        if deferred:
+        decode = decode_product(rows, self.qkv_weight)
+        norm = x.fused() if deferred and decode else None
+        if norm is not None:
+            x.resolve(None)  # nothing is left to add: the kernel norms the residual rows as they are
+        elif deferred:
             rows = x.materialize()  # the residual sum and the norm by the norm's own kernel, the rest fused
         rope = dict(n_heads=self.num_heads, n_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                     inv_freq=frequencies() if frequencies is not None else None, positions=batch.positions,
                     slots=slots, k_pool=cache.k_pool, v_pool=cache.v_pool, block_size=cache.block_size)
         q = torch.empty((m, self.num_heads * self.head_dim), dtype=rows.dtype, device=rows.device)
-        ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias, rope=rope)
+        if decode:
+            ops.gemm_decode(q, rows, self.qkv_weight, self.qkv_bias, rope=rope, norm=norm)
+        else:
+            ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias, rope=rope)
         return q
 
     def attend(self, out, qkv, cache, view, batch):

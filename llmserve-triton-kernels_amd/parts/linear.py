@@ -1,7 +1,10 @@
 """y = x W^T (+ b) for the parts: picks the matrix product by dtype and shape.
 
 float32: the 32-bit multiply-add kernel, always (no reduced-precision matrix mode).
-bfloat16, few rows (decoding): the hand-written kernel that streams the weight once
+bfloat16, up to 16 rows whose K fits a compute unit's LDS: ops.gemm_decode, one workgroup per compute
+  unit, which also norms its rows on the way in and adds its result to the residual rows where the
+  parts ask for that (decode_product).
+bfloat16, few rows otherwise: the hand-written kernel that streams the weight once
   (ops.gemm_stream); it takes up to 64 rows, one workgroup per 16 rows and 16 weight rows, so
   beyond 16 rows the weights are re-read from L2 and it only pays for the smaller matrices.
   A product whose result goes to a norm may be left as 32-bit partial sums over shares of K, which
@@ -34,6 +37,14 @@ STREAM_MAX_ROWS = 64
 # beyond STREAM_ROWS: bytes of weight times blocks of 16 rows up to which the streaming kernel still beats
 # the library (measured on the TinyLlama shapes at 32 and 64 rows, with the epilogue it saves counted in)
 STREAM_REREAD_BYTES = 64e6
+
+
+DECODE_KERNEL = os.environ.get("LLMSERVE_DECODE_GEMM", "1") != "0"
+
+
+def decode_product(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether x [M, K] against weight goes to ops.gemm_decode (one workgroup per compute unit)."""
+    return DECODE_KERNEL and ops.gemm_decode_supported(x, weight)
 
 
 def few_rows(m: int, weight: torch.Tensor) -> bool:
@@ -102,6 +113,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     if m == 0:
         return out
     if x.dtype == torch.bfloat16 and ops.gemm_bf16_supported(x, weight):
+        if decode_product(x, weight):
+            return ops.gemm_decode(out, x, weight, bias)
         if few_rows(m, weight):
             return ops.gemm_stream(out, x, weight, bias)
         if OWN_KERNELS_ONLY:

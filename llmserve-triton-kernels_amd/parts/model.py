@@ -26,10 +26,14 @@ class Model:
         self.head = HEADS.build(spec.head, ctx)
         self.blocks = []
         self._sources = None
-        for layer in spec.layers:
-            self.blocks.append(BLOCKS.get(layer.block)(
-                MIXERS.build(layer.mixer, ctx), FEED_FORWARDS.build(layer.feed_forward, ctx),
-                NORMS.build(layer.mixer_norm, ctx), NORMS.build(layer.feed_forward_norm, ctx)))
+        families = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}
+        for index, layer in enumerate(spec.layers):
+            block = BLOCKS.get(layer.block)
+            if set(layer.parts) != set(block.ROLES) or set(layer.weights) != set(block.ROLES):
+                raise ValueError(f"layer {index}: the arrangement {layer.block!r} has the roles {sorted(block.ROLES)}; "
+                                 f"the spec names parts for {sorted(layer.parts)} and weights for {sorted(layer.weights)}")
+            self.blocks.append(block({role: families[family].build(layer.parts[role], ctx)
+                                      for role, family in block.ROLES.items()}))
 
     # ---- tensors -------------------------------------------------------------------------
     def _parts(self) -> list[tuple[str, Part]]:
@@ -37,9 +41,7 @@ class Model:
         w = self.spec.weights
         out = [(w["embedding"], self.embedding), (w["final_norm"], self.final_norm), (w["head"], self.head)]
         for layer, blk in zip(self.spec.layers, self.blocks):
-            out += [(layer.weights["mixer_norm"], blk.mixer_norm), (layer.weights["mixer"], blk.mixer),
-                    (layer.weights["feed_forward_norm"], blk.feed_forward_norm),
-                    (layer.weights["feed_forward"], blk.feed_forward)]
+            out += [(layer.weights[role], part) for role, part in blk.parts.items()]
         return out
 
     def param_infos(self) -> dict[str, ParamInfo]:
@@ -62,15 +64,18 @@ class Model:
     def graph_safe(self) -> bool:
         """Whether a decode-only step through this model may be captured as a HIP graph."""
         parts = [part for _, part in self._parts()]
-        parts += [getattr(blk.mixer, "position", None) for blk in self.blocks]
+        parts += [getattr(part, "position", None) for blk in self.blocks for part in blk.parts.values()]
         return all(p.graph_safe for p in parts if p is not None)
 
     def cache_specs(self) -> list:
         """What each entry of the schedule keeps between steps (None when its layer borrows
         another layer's cache).  A layer that runs twice keeps two caches, one per run: the keys
         of its second run are not those of its first."""
-        return [None if self.spec.layers[i].cache_from is not None else self.blocks[i].mixer.cache_spec()
-                for i in self.spec.schedule]
+        def own(i):
+            keeper = self.blocks[i].cache_part()
+            return None if self.spec.layers[i].cache_from is not None or keeper is None else keeper.cache_spec()
+
+        return [own(i) for i in self.spec.schedule]
 
     def cache_sources(self) -> list:
         """For each entry of the schedule the entry whose cache it reads instead of its own: the

@@ -18,9 +18,11 @@ Interfaces (x is always the flat batch of new tokens, [N, hidden], in the model 
   Block             forward(x, delta, batch, cache) -> (x, delta)   hidden state is x + delta
 
 A mixer or feed-forward that sets `accepts_deferred_norm` is handed a `DeferredNorm` instead of the
-normed tensor and may fold the residual sum and the norm into its own first kernel.  To such a caller
-it may also return `PartialSums` instead of y: 32-bit partial sums of its last product, which the next
-norm's kernel adds up as it adds the residual.
+normed tensor and may fold the residual sum and the norm into its own first kernel (a norm that is an
+RMSNorm offers `rms_params() -> (weight, eps)` for that).  To such a caller it may also return
+`PartialSums` instead of y: 32-bit partial sums of its last product, which the next norm's kernel adds
+up as it adds the residual; or, where the caller allows it, `ADDED_IN_PLACE` after adding y into the
+residual rows itself.
 """
 
 from __future__ import annotations
@@ -100,22 +102,42 @@ def as_tensor(delta):
     return delta.total() if isinstance(delta, PartialSums) else delta
 
 
+class AddedInPlace:
+    """What a part returns in the place of y when it has added y into the residual rows it was handed
+    (`DeferredNorm.residual`, after the input was consumed) by itself: nothing is left to add."""
+
+
+ADDED_IN_PLACE = AddedInPlace()
+
+
 class DeferredNorm:
     """The input of a mixer or feed-forward before it is computed: norm(residual + delta).
 
     The consumer either calls `materialize()` (the norm's own kernel: residual += delta in place, returns
     the normed tensor) or computes the same thing inside a kernel of its own and reports the summed
-    residual with `resolve(new_residual)`.  Afterwards `residual` is the summed residual stream."""
+    residual with `resolve(new_residual)`.  Afterwards `residual` is the summed residual stream.
 
-    def __init__(self, norm: "Norm", residual: torch.Tensor, delta: torch.Tensor | None):
+    `fused()` serves the second way where the norm is an RMSNorm: (weight, eps) when nothing is left to add,
+    so that a kernel which norms its rows on the way in can take `residual` as they are.
+    `may_add_in_place`: the caller will add the consumer's result to `residual` next and allows the
+    consumer to do that itself (in 32-bit, rounded once) and to return `ADDED_IN_PLACE`."""
+
+    def __init__(self, norm: "Norm", residual: torch.Tensor, delta: torch.Tensor | None, may_add_in_place: bool = False):
         self.norm = norm
         self.residual = residual
         self.delta = delta
+        self.may_add_in_place = may_add_in_place
         self.resolved = False
 
     @property
     def num_rows(self) -> int:
         return self.residual.shape[0]
+
+    def fused(self) -> "tuple[torch.Tensor, float] | None":
+        if self.delta is not None:
+            return None
+        params = getattr(self.norm, "rms_params", None)
+        return params() if params is not None else None
 
     def materialize(self) -> torch.Tensor:
         if self.resolved:
@@ -157,13 +179,25 @@ class FeedForward(Part):
 
 
 class Block:
-    """Arrangement of one layer's parts."""
+    """Arrangement of one layer's parts.
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
-        self.mixer = mixer
-        self.feed_forward = feed_forward
-        self.mixer_norm = mixer_norm
-        self.feed_forward_norm = feed_forward_norm
+    `ROLES` maps every role of the arrangement to the family its part is built from ("mixer",
+    "feed_forward" or "norm"); the model builds a part for each role from the layer's spec and hands them
+    over, and they are the block's attributes by role.  The part in the role "mixer", if the arrangement
+    has one, is the one that keeps a cache between steps."""
+
+    ROLES: dict[str, str] = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm",
+                             "feed_forward_norm": "norm"}
+
+    def __init__(self, parts: dict[str, Part]):
+        if set(parts) != set(self.ROLES):
+            raise ValueError(f"{type(self).__name__} has the roles {sorted(self.ROLES)}, got {sorted(parts)}")
+        self.parts = dict(parts)
+        for role, part in parts.items():
+            setattr(self, role, part)
+
+    def cache_part(self) -> "Mixer | None":
+        return self.parts.get("mixer")
 
     def forward(self, x, delta, batch, cache):
         raise NotImplementedError

@@ -26,6 +26,10 @@ class RMSNorm(Norm):
     def load(self, tensors):
         self.weight = tensors["weight"].contiguous()
 
+    def rms_params(self):
+        """(weight, eps): what a kernel that norms its rows on the way in needs."""
+        return self.weight, self.eps
+
     def forward(self, x):
         return ops.rmsnorm(torch.empty_like(x), x, self.weight, self.eps)
 

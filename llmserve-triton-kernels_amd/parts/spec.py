@@ -27,21 +27,26 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: a block arrangement of a mixer and a feed-forward with their norms.
+    """One layer: the parts of its block arrangement, by role.
 
-    `weights` maps each role ("mixer", "feed_forward", "mixer_norm", "feed_forward_norm")
-    to the checkpoint prefix of that part's tensors; a part's own tensor names are appended
-    to it.  `cache_from` names another layer whose cache this layer's mixer reads instead
-    of keeping one of its own (the cache of that layer's latest run earlier in the schedule).
+    The arrangement (`block`, a key of the block registry) declares which roles it has and which family
+    each role's part comes from (`Block.ROLES`: the reference's layer has "mixer", "feed_forward",
+    "mixer_norm" and "feed_forward_norm"; another arrangement may have a third norm or a second
+    feed-forward).  `parts` maps every role to its part, `weights` every role to the checkpoint prefix of
+    that part's tensors (a part's own tensor names are appended to it).  `cache_from` names another layer
+    whose cache this layer's mixer reads instead of keeping one of its own (the cache of that layer's
+    latest run earlier in the schedule).
     """
 
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: Mapping[str, PartSpec]
     weights: Mapping[str, str]
     block: str = "prenorm"
     cache_from: int | None = None
+
+    @property
+    def mixer(self) -> PartSpec | None:
+        """The part that keeps a cache between steps, if the arrangement has one."""
+        return self.parts.get("mixer")
 
 
 @dataclass(frozen=True)
@@ -75,6 +80,8 @@ class ModelSpec:
                 if first_use is not None and (first_own is None or first_own > first_use):
                     raise ValueError(f"layer {i} reads the cache of layer {src} before that layer has run")
                 a, b = self.layers[i].mixer, self.layers[src].mixer
+                if a is None or b is None:
+                    raise ValueError(f"layer {i} cannot read the cache of layer {src}: one of them has no mixer")
                 for key in ("num_kv_heads", "head_dim"):
                     if a.get(key) != b.get(key):
                         raise ValueError(f"layer {i} cannot read the cache of layer {src}: {key} differs")

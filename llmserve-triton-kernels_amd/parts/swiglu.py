@@ -9,8 +9,8 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .linear import few_rows, linear, linear_partial_sums
-from .registry import DeferredNorm, FeedForward, register_feed_forward
+from .linear import decode_product, few_rows, linear, linear_partial_sums
+from .registry import ADDED_IN_PLACE, DeferredNorm, FeedForward, register_feed_forward
 from .spec import ParamInfo
 
 
@@ -36,18 +36,27 @@ class SwiGLU(FeedForward):
         self.down = tensors["down_proj.weight"].contiguous()
 
     def forward(self, x):
-        m = x.num_rows if isinstance(x, DeferredNorm) else x.shape[0]
+        deferred = isinstance(x, DeferredNorm)  # the caller hands the result to a norm, which takes partial sums
+        rows = x.residual if deferred else x
+        m = rows.shape[0]
         dtype, device = self.gate_up.dtype, self.gate_up.device
         act = torch.empty((m, self.intermediate), dtype=dtype, device=device)
-        few = dtype == torch.bfloat16 and few_rows(m, self.gate_up) and self.intermediate % 8 == 0
-        to_a_norm = isinstance(x, DeferredNorm)  # the caller hands the result to a norm, which takes partial sums
-        if isinstance(x, DeferredNorm):
-            x = x.materialize()
-        if few and ops.gemm_bf16_supported(x, self.gate_up):
-            ops.gemm_stream(act, x, self.gate_up, swiglu=True)  # activation in the product's epilogue
+        if decode_product(rows, self.gate_up):
+            norm = x.fused() if deferred else None
+            if norm is not None:
+                x.resolve(None)  # nothing is left to add: the kernel norms the residual rows as they are
+            elif deferred:
+                rows = x.materialize()
+            ops.gemm_decode(act, rows, self.gate_up, swiglu=True, norm=norm)  # norm before, activation after the product
         else:
-            ops.silu_mul(act, linear(x, self.gate_up))
-        return self._down(act, to_a_norm)
-
-    def _down(self, act, to_a_norm):
-        return (linear_partial_sums(act, self.down) if to_a_norm else None) or linear(act, self.down)
+            if deferred:
+                rows = x.materialize()
+            few = dtype == torch.bfloat16 and few_rows(m, self.gate_up) and self.intermediate % 8 == 0
+            if few and ops.gemm_bf16_supported(rows, self.gate_up):
+                ops.gemm_stream(act, rows, self.gate_up, swiglu=True)  # activation in the product's epilogue
+            else:
+                ops.silu_mul(act, linear(rows, self.gate_up))
+        if deferred and x.may_add_in_place and decode_product(act, self.down):
+            ops.gemm_decode(None, act, self.down, residual=x.residual)  # the residual sum in the product's epilogue
+            return ADDED_IN_PLACE
+        return (linear_partial_sums(act, self.down) if deferred else None) or linear(act, self.down)

@@ -110,8 +110,9 @@ def test_spec_is_data_per_layer():
     layer = spec.layers[1]
     assert layer.mixer.kind == "attention" and layer.mixer["num_kv_heads"] == 1 and layer.mixer["head_dim"] == 32
     assert layer.mixer["position"].kind == "rope" and layer.mixer["position"]["theta"] == 500000.0
-    assert layer.feed_forward.kind == "swiglu" and layer.feed_forward["intermediate"] == 256
-    assert layer.mixer_norm["eps"] == 1e-6 and layer.weights["mixer"] == "model.layers.1.self_attn."
+    assert set(layer.parts) == set(layer.weights) == {"mixer", "feed_forward", "mixer_norm", "feed_forward_norm"}
+    assert layer.parts["feed_forward"].kind == "swiglu" and layer.parts["feed_forward"]["intermediate"] == 256
+    assert layer.parts["mixer_norm"]["eps"] == 1e-6 and layer.weights["mixer"] == "model.layers.1.self_attn."
     assert spec.head["tied"] is True
 
 

@@ -340,8 +340,8 @@ def register_toy():
             ffn = (PartSpec("soft_experts", {"hidden": h, "intermediate": inter, "experts": 3}) if i == 2
                    else PartSpec("swiglu", {"hidden": h, "intermediate": inter}))
             layers.append(LayerSpec(
-                mixer=mixer, feed_forward=ffn, mixer_norm=norm,
-                feed_forward_norm=norm, cache_from=0 if i == 3 else None,
+                parts={"mixer": mixer, "feed_forward": ffn, "mixer_norm": norm, "feed_forward_norm": norm},
+                cache_from=0 if i == 3 else None,
                 weights={"mixer": p + "mix.", "feed_forward": p + "ffn.", "mixer_norm": p + "n1.",
                          "feed_forward_norm": p + "n2."}))
         return ModelSpec(hidden_size=h, vocab_size=cfg.vocab_size, max_positions=128,
