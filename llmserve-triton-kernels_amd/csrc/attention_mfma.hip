@@ -363,9 +363,7 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
     // exists), so the number of loads in flight is known and the arithmetic of one tile overlaps the loads of
     // the next.  Key rows beyond p_max hold real keys whose scores the mask discards; values outside
     // [lo_min, p_max], which may be stale or never written, are zeroed after the load.
-    auto load_tile = [&](int j0, uint4 (&kf)[2][KS], uint4 (&vf)[DB]) {
-        const int blk_first = block_of(j0);
-        if (blk_first < blk_base || block_of(min(j0 + 31, p_max)) >= blk_base + LLMS_WAVE) load_pages(blk_first);
+    auto fetch_tile = [&](int j0, uint4 (&kf)[2][KS], uint4 (&vf)[DB]) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int key = min(j0 + 8 * (col / 4) + 4 * u + (col % 4), p_max);  // `col` is the row index i here
@@ -385,23 +383,13 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
 #pragma unroll
         for (int m = 0; m < DB; ++m) vf[m] = *reinterpret_cast<const uint4*>(vrow + (uint32_t)(16 * m * a.block_size));
     };
-
-    // the next tile's operands are requested before this tile's arithmetic starts
-    uint4 kf_next[2][KS], vf_next[DB];
-    if (t_begin < t_end) {
-        load_pages(block_of(j_begin + 32 * t_begin));
-        load_tile(j_begin + 32 * t_begin, kf_next, vf_next);
-    }
-    for (int t = t_begin; t < t_end; t += t_step) {
-        const int j0 = j_begin + 32 * t;
-        uint4 kf[2][KS], vf[DB];
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int s = 0; s < KS; ++s) kf[u][s] = kf_next[u][s];
-#pragma unroll
-        for (int m = 0; m < DB; ++m) vf[m] = vf_next[m];
-        if (t + t_step < t_end) load_tile(j_begin + 32 * (t + t_step), kf_next, vf_next);
+    auto load_tile = [&](int j0, uint4 (&kf)[2][KS], uint4 (&vf)[DB]) {
+        const int blk_first = block_of(j0);
+        if (blk_first < blk_base || block_of(min(j0 + 31, p_max)) >= blk_base + LLMS_WAVE) load_pages(blk_first);
+        fetch_tile(j0, kf, vf);
+    };
+    // scores, softmax and weighted values of the tile that starts at key j0
+    auto attend = [&](int j0, const uint4 (&kf)[2][KS], uint4 (&vf)[DB]) {
         // (queries beyond head_dim are zero, so a key chunk loaded from a clamped address adds nothing)
         const int jk = j0 + 8 * g;
         if (j0 >= lo_max && j0 + 31 <= p_min) {  // (uniform over the wave; columns without a token are discarded)
@@ -411,6 +399,43 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
 #pragma unroll
             for (int m = 0; m < DB; ++m) vf[m] = keep_elements(vf[m], first, last);
             attend_tile<DB, KS, true>(acc, m_run, l_run, kf, vf, qf, jk, lo_col, p_col, scale_log2);
+        }
+    };
+
+    // Few tiles per wave (a decoded token behind a context of some hundred keys: up to AHEAD each, whose pages one
+    // register per lane holds): every tile's operands are asked for at once, so the wave's way through memory is
+    // one trip and not one per tile.  Every wave issues the same loads (a tile it does not have is the workgroup's
+    // last once more, which some other wave brings in anyway), so the compiler knows how many are in flight when
+    // it waits for the first.
+    constexpr int AHEAD = DB <= 4 ? 3 : DB <= 8 ? 2 : 1;  // (what the registers hold beside the sums)
+    const int t_first_here = split * per_split;
+    const bool at_once = t_end > t_first_here && t_end - t_first_here <= AHEAD * NW &&
+                         block_of(min(j_begin + 32 * t_end - 1, p_max)) - block_of(j_begin + 32 * t_first_here) < LLMS_WAVE;
+    if (at_once) {
+        load_pages(block_of(j_begin + 32 * t_first_here));
+        uint4 kfa[AHEAD][2][KS], vfa[AHEAD][DB];
+#pragma unroll
+        for (int i = 0; i < AHEAD; ++i) fetch_tile(j_begin + 32 * min(t_begin + i * NW, t_end - 1), kfa[i], vfa[i]);
+#pragma unroll
+        for (int i = 0; i < AHEAD; ++i)
+            if (t_begin + i * NW < t_end) attend(j_begin + 32 * (t_begin + i * NW), kfa[i], vfa[i]);
+    } else {
+        // the next tile's operands are requested before this tile's arithmetic starts
+        uint4 kf_next[2][KS], vf_next[DB];
+        if (t_begin < t_end) {
+            load_pages(block_of(j_begin + 32 * t_begin));
+            load_tile(j_begin + 32 * t_begin, kf_next, vf_next);
+        }
+        for (int t = t_begin; t < t_end; t += t_step) {
+            uint4 kf[2][KS], vf[DB];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int s = 0; s < KS; ++s) kf[u][s] = kf_next[u][s];
+#pragma unroll
+            for (int m = 0; m < DB; ++m) vf[m] = vf_next[m];
+            if (t + t_step < t_end) load_tile(j_begin + 32 * (t + t_step), kf_next, vf_next);
+            attend(j_begin + 32 * t, kf, vf);
         }
     }
 
