@@ -8,7 +8,10 @@ Layers with the same needs (same KV heads, head size and window) form a *group*:
 pool, one allocator, one block table per request.  Position p of a request lives in page
 `table[p // block_size]` at offset `p % block_size` (src/llmserve/kvcache/paged.py:196-197).
 Pages come back when the request ends, or, in a windowed group, as soon as every later
-query is out of their reach; a returned entry of the table becomes -1.
+query is out of their reach; a returned entry of the table becomes -1.  Every group has a pool
+of its own size: what a request costs is a number of pages *per group* (`pages_for`,
+`pages_owed`; none in a group of fixed-size state), and whoever plans steps compares it group by
+group with `free_pages`.
 
 `append` is atomic like the reference's `build_batch` (src/llmserve/kvcache/paged.py:174-200):
 it first sums what the whole step needs over all groups and raises `OutOfBlocks` before
@@ -59,16 +62,27 @@ class StepLayout:
     table_updates: dict[int, list[tuple[int, int, int]]] = field(default_factory=dict)
 
 
+def window_pages(window: int, step_tokens: int, block_size: int) -> int:
+    """Most pages a request holds in a group that keeps `window` keys, when a step brings up to `step_tokens` of
+    its tokens: the keys the portion's first query still sees, the portion itself, and one page more because
+    neither starts at a page's edge.  (Pages out of reach come back after the step that passed them.)"""
+    return -(-(window - 1 + step_tokens) // block_size) + 1
+
+
 class CacheManager:
-    def __init__(self, groups: list[CacheGroup], num_blocks: int, block_size: int, max_seqs: int):
+    def __init__(self, groups: list[CacheGroup], num_blocks: "int | dict[int, int]", block_size: int, max_seqs: int):
+        """`num_blocks`: pages of every paged group's pool, or a size per group id."""
         if block_size < 1 or max_seqs < 1:
             raise ValueError("block_size and max_seqs must be >= 1")
         self.groups = list(groups)
         self.paged_groups = [g for g in self.groups if g.paged]
-        self.num_blocks = num_blocks
+        sizes = num_blocks if isinstance(num_blocks, dict) else {g.group_id: num_blocks for g in self.paged_groups}
+        if set(sizes) != {g.group_id for g in self.paged_groups} or any(n < 1 for n in sizes.values()):
+            raise ValueError(f"pool sizes {sizes} do not name every paged group with at least one page")
+        self._single = num_blocks if isinstance(num_blocks, int) else 1  # (what a model without pages reports)
         self.block_size = block_size
         self.max_seqs = max_seqs
-        self.allocators = {g.group_id: BlockAllocator(num_blocks) for g in self.paged_groups}
+        self.allocators = {gid: BlockAllocator(n) for gid, n in sizes.items()}
         self.tables: dict[int, dict] = {g.group_id: {} for g in self.paged_groups}
         self.lengths: dict = {}
         self.slot_of: dict = {}
@@ -80,12 +94,52 @@ class CacheManager:
     def blocks_for(self, n_tokens: int) -> int:
         return -(-n_tokens // self.block_size)
 
+    def capacity(self) -> dict[int, int]:
+        """Pages of every paged group's pool."""
+        return {gid: a.num_blocks for gid, a in self.allocators.items()}
+
+    def free_pages(self) -> dict[int, int]:
+        return {gid: a.num_free for gid, a in self.allocators.items()}
+
+    def pages_for(self, n_tokens: int, step_tokens: int | None = None) -> dict[int, int]:
+        """Pages a request of `n_tokens` in all holds at most, per paged group: all its pages where every key is
+        kept; in a windowed group no more than the window and one step's portion need (`step_tokens`: the most
+        tokens of one request in a step; None: unknown, so all of them).  Groups of fixed-size state cost no
+        pages and are not named."""
+        full = self.blocks_for(n_tokens)
+        need = {}
+        for g in self.paged_groups:
+            if g.spec.window is None or step_tokens is None:
+                need[g.group_id] = full
+            else:
+                need[g.group_id] = min(full, window_pages(g.spec.window, step_tokens, self.block_size))
+        return need
+
+    def pages_owed(self, seq_id, new_tokens: int, step_tokens: int | None = None) -> dict[int, int]:
+        """Pages that `new_tokens` more tokens of a live request take, per paged group.  `step_tokens` None: the
+        tokens come in one step, so every page they touch is taken at once (what `append` checks).  Otherwise they
+        come in portions of up to `step_tokens`, and a windowed group is owed only what brings the request to the
+        most it ever holds there."""
+        want = self.blocks_for(self.lengths[seq_id] + new_tokens)
+        owed = {}
+        for g in self.paged_groups:
+            table = self.tables[g.group_id][seq_id]
+            owed[g.group_id] = max(0, want - len(table))
+            if g.spec.window is not None and step_tokens is not None:
+                held = sum(1 for page in table if page >= 0)
+                most = window_pages(g.spec.window, min(step_tokens, max(new_tokens, 1)), self.block_size)
+                owed[g.group_id] = min(owed[g.group_id], max(0, most - held))
+        return owed
+
+    @property
+    def num_blocks(self) -> int:
+        """Pages of the smallest pool (of the one pool, for a model whose layers all keep the same)."""
+        return min((a.num_blocks for a in self.allocators.values()), default=self._single)
+
     @property
     def num_free_blocks(self) -> int:
-        """Free pages of the tightest group (every group must fit a request)."""
-        if not self.allocators:
-            return self.num_blocks
-        return min(a.num_free for a in self.allocators.values())
+        """Free pages of the group that has the fewest."""
+        return min((a.num_free for a in self.allocators.values()), default=self._single)
 
     @property
     def num_free_slots(self) -> int:
@@ -93,9 +147,7 @@ class CacheManager:
 
     def utilization(self) -> float:
         """Fraction of pages in use (src/llmserve/kvcache/paged.py:145-147), fullest group."""
-        if not self.allocators:
-            return 0.0
-        return max(a.num_used for a in self.allocators.values()) / self.num_blocks
+        return max((a.num_used / a.num_blocks for a in self.allocators.values()), default=0.0)
 
     def internal_fragmentation(self) -> float:
         """Fraction of slots in held pages that hold no token (src/llmserve/kvcache/paged.py:149-153), over
@@ -140,16 +192,24 @@ class CacheManager:
         del self.lengths[seq_id]
 
     def extra_blocks_needed(self, seq_id, new_tokens: int) -> int:
-        """Pages that `new_tokens` more tokens cost in the group where they cost most (`num_free_blocks` is
-        the tightest group's count, so the two compare).  A table keeps its length when a windowed group gives
-        pages back, so today every group answers alike; nothing here relies on that."""
-        want = self.blocks_for(self.lengths[seq_id] + new_tokens)
-        return max((max(0, want - len(self.tables[g.group_id][seq_id])) for g in self.paged_groups), default=0)
+        """Pages that `new_tokens` more tokens cost in the group where they cost most."""
+        return max(self.pages_owed(seq_id, new_tokens).values(), default=0)
+
+    def _shortfall(self, seq_ids, counts) -> str | None:
+        """None if every group has the pages these appends take, else what is missing."""
+        need: dict[int, int] = {}
+        for s, n in zip(seq_ids, counts):
+            for gid, pages in self.pages_owed(s, n).items():
+                need[gid] = need.get(gid, 0) + pages
+        for gid, pages in need.items():
+            free = self.allocators[gid].num_free
+            if pages > free:
+                return f"step needs {pages} pages of cache group {gid}, {free} free"
+        return None
 
     def can_append(self, seq_ids, counts) -> bool:
         """Whether `append` with these arguments would find its pages."""
-        need = sum(self.extra_blocks_needed(s, n) for s, n in zip(seq_ids, counts))
-        return need <= self.num_free_blocks
+        return self._shortfall(seq_ids, counts) is None
 
     # ---- one step ---------------------------------------------------------------------------
     def append(self, seq_ids: list, counts: list[int]) -> StepLayout:
@@ -160,9 +220,9 @@ class CacheManager:
                 raise KeyError(f"unknown sequence {s!r}")
             if n < 1:
                 raise ValueError("every request of a step brings at least one token")
-        need = sum(self.extra_blocks_needed(s, n) for s, n in zip(seq_ids, counts))
-        if need > self.num_free_blocks:
-            raise OutOfBlocks(f"step needs {need} pages, {self.num_free_blocks} free")
+        short = self._shortfall(seq_ids, counts)
+        if short is not None:
+            raise OutOfBlocks(short)
 
         bs = self.block_size
         layout = StepLayout(seq_ids=list(seq_ids), counts=list(counts),

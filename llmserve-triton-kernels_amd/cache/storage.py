@@ -14,7 +14,7 @@ from dataclasses import dataclass
 
 import torch
 
-from .manager import CacheGroup
+from .manager import CacheGroup, window_pages
 
 
 @dataclass
@@ -34,26 +34,60 @@ class StateLayerCache:
     group_id: int
 
 
+def page_bytes_of(group: CacheGroup, block_size: int, elem_size: int) -> int:
+    """Bytes one page of a paged group costs over the group's layers (keys and values); L layers give the
+    reference's 2*L*kv_heads*block_size*head_dim*elem (src/llmserve/kvcache/paged.py:221-227)."""
+    return 2 * len(group.layers) * group.spec.num_kv_heads * block_size * group.spec.head_dim * elem_size
+
+
 def page_bytes(groups: list[CacheGroup], block_size: int, elem_size: int) -> int:
-    """Bytes one page id costs over all paged groups and their layers (keys and values);
-    one group of L layers gives the reference's 2*L*kv_heads*block_size*head_dim*elem
-    (src/llmserve/kvcache/paged.py:221-227)."""
+    """Bytes one page id costs over all paged groups together."""
+    return sum(page_bytes_of(g, block_size, elem_size) for g in groups if g.paged)
+
+
+def state_bytes(groups: list[CacheGroup], max_seqs: int) -> int:
+    """Bytes of the fixed-size state of all `max_seqs` slots, over all state groups and their layers."""
     total = 0
     for g in groups:
-        if g.paged:
-            total += 2 * len(g.layers) * g.spec.num_kv_heads * block_size * g.spec.head_dim * elem_size
+        if not g.paged:
+            elems = 1
+            for n in g.spec.shape:
+                elems *= n
+            total += len(g.layers) * max_seqs * elems * torch.empty(0, dtype=getattr(torch, g.spec.dtype)).element_size()
     return total
 
 
+def pool_sizes_for_budget(groups: list[CacheGroup], block_size: int, elem_size: int, budget_bytes: int, max_seqs: int,
+                          longest: int, step_tokens: int) -> dict[int, int]:
+    """Pages of every paged group's pool so that `budget_bytes` are shared out by need: the fixed-size state of all
+    slots comes off the budget first, then every group gets pages for the same number of longest requests (a
+    windowed group needs far fewer per request than one that keeps every key), at most what `max_seqs` such
+    requests could fill.  No paged group: an empty mapping."""
+    paged = [g for g in groups if g.paged]
+    fixed = state_bytes(groups, max_seqs)
+    if fixed > budget_bytes:
+        raise ValueError(f"the fixed-size state of {max_seqs} requests takes {fixed} bytes, the cache budget is {budget_bytes}")
+    if not paged:
+        return {}
+    full = -(-longest // block_size)
+    need = {g.group_id: full if g.spec.window is None else min(full, window_pages(g.spec.window, step_tokens, block_size))
+            for g in paged}
+    per_request = sum(need[g.group_id] * page_bytes_of(g, block_size, elem_size) for g in paged)
+    requests = min(float(max_seqs), (budget_bytes - fixed) / per_request)
+    return {gid: max(1, int(n * requests)) for gid, n in need.items()}
+
+
 def num_blocks_for_budget(groups: list[CacheGroup], block_size: int, elem_size: int, budget_bytes: int) -> int:
+    """Pages per pool when every paged group gets the same number (the reference's sizing for its one group)."""
     per_block = page_bytes(groups, block_size, elem_size)
     return max(1, budget_bytes // per_block) if per_block else 1
 
 
 class CacheStorage:
-    def __init__(self, groups: list[CacheGroup], num_blocks: int, block_size: int, max_seqs: int,
+    def __init__(self, groups: list[CacheGroup], num_blocks: "int | dict[int, int]", block_size: int, max_seqs: int,
                  dtype: torch.dtype, device: torch.device, table_width: int = 1):
-        """`table_width`: most pages a request can hold (longest request / block_size)."""
+        """`num_blocks`: pages of every paged group's pool, or a size per group id; `table_width`: most pages a
+        request can hold (longest request / block_size)."""
         self.groups = groups
         self.max_seqs = max_seqs
         self.table_width = table_width
@@ -71,9 +105,10 @@ class CacheStorage:
             n = len(g.layers)
             if g.paged:
                 s = g.spec
-                self.k[g.group_id] = torch.zeros((n, num_blocks, s.num_kv_heads, block_size, s.head_dim),
+                pages = num_blocks[g.group_id] if isinstance(num_blocks, dict) else num_blocks
+                self.k[g.group_id] = torch.zeros((n, pages, s.num_kv_heads, block_size, s.head_dim),
                                                  dtype=dtype, device=device)
-                self.v[g.group_id] = torch.zeros((n, num_blocks, s.num_kv_heads, s.head_dim, block_size),
+                self.v[g.group_id] = torch.zeros((n, pages, s.num_kv_heads, s.head_dim, block_size),
                                                  dtype=dtype, device=device)
                 self.tables[g.group_id] = torch.zeros((max_seqs, table_width), dtype=torch.int32, device=device)
             else:

@@ -17,7 +17,7 @@ from pathlib import Path
 import torch
 
 from ..cache.manager import CacheManager, group_layers
-from ..cache.storage import CacheStorage, num_blocks_for_budget
+from ..cache.storage import CacheStorage, pool_sizes_for_budget
 from ..config.engine_config import EngineConfig
 from ..config.registry import architecture_of, read_config
 from ..ops import library as ops
@@ -48,6 +48,10 @@ class ModelRunner:
         self.device = device
         self.dtype = model.ctx.dtype
         self.vocab_size = model.spec.vocab_size
+        if engine_config.max_model_len is not None and engine_config.max_model_len > model.spec.max_positions:
+            # (the reference refuses it too: src/llmserve/utils.py:8-13)
+            raise ValueError(f"max_model_len={engine_config.max_model_len} is more than the model's "
+                             f"{model.spec.max_positions} positions")
         self.max_model_len = engine_config.max_model_len or model.spec.max_positions
         self.block_size = engine_config.block_size
         groups = group_layers(model.cache_specs())
@@ -59,10 +63,11 @@ class ModelRunner:
             if budget is None:
                 free, _total = torch.cuda.mem_get_info(device)
                 budget = int(free * engine_config.gpu_memory_fraction)
-            num_blocks = num_blocks_for_budget(groups, self.block_size, elem, budget)
-            # more pages than every slot could ever fill are of no use
-            most = engine_config.max_num_seqs * -(-self.max_model_len // self.block_size)
-            num_blocks = min(num_blocks, most)
+            # the state of all slots comes off the budget; every paged group gets pages for the same number of longest
+            # requests, and no more than all slots could ever fill
+            step_tokens = min(engine_config.max_num_batched_tokens, engine_config.max_prefill_chunk or self.max_model_len)
+            num_blocks = pool_sizes_for_budget(groups, self.block_size, elem, budget, engine_config.max_num_seqs,
+                                               self.max_model_len, step_tokens)
         self.manager = CacheManager(groups, num_blocks, self.block_size, engine_config.max_num_seqs)
         self.storage = CacheStorage(groups, num_blocks, self.block_size, engine_config.max_num_seqs,
                                     self.dtype, device, table_width=-(-self.max_model_len // self.block_size))

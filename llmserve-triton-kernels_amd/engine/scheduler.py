@@ -46,6 +46,17 @@ from .request import EngineStats, Request, Status, TokenEvent
 from .runner import StepEntry
 
 
+def _add(total: dict[int, int], pages: dict[int, int]) -> None:
+    """total += pages, group by group."""
+    for gid, n in pages.items():
+        total[gid] = total.get(gid, 0) + n
+
+
+def _fits(need: dict[int, int], free: dict[int, int], spare: int = 0) -> bool:
+    """Whether every group has `need` pages free and `spare` more (a group that is not named needs none)."""
+    return all(free[gid] - n >= spare for gid, n in need.items())
+
+
 @dataclass
 class _Share:
     """One request's part of a planned step."""
@@ -68,6 +79,8 @@ class ContinuousBatchingEngine:
         self.max_num_seqs = max_num_seqs
         self.max_num_batched_tokens = max_num_batched_tokens
         self.max_prefill_chunk = max_prefill_chunk
+        # the most tokens of one request in a step: what a windowed cache group holds beside its window
+        self._portion = min(max_num_batched_tokens, max_prefill_chunk or max_num_batched_tokens)
         self.seed = seed
         self.waiting: deque[Request] = deque()  # arrival order; a preempted request re-enters at the left
         self.running: list[Request] = []  # admission order, oldest first
@@ -88,15 +101,18 @@ class ContinuousBatchingEngine:
         to generate, more positions than the model has, more pages than the pool has (the four checks
         of src/llmserve/scheduler/engine.py:111-125)."""
         positions = prompt_len + max_new_tokens
-        pages = self.manager.blocks_for(positions)
+        # what the request holds at most, group by group, against each group's whole pool (a model that keeps
+        # only fixed-size state has no pages to run out of)
+        need, pools = self.manager.pages_for(positions, self._portion), self.manager.capacity()
+        short = [(gid, n) for gid, n in need.items() if n > pools[gid]]
         problems = (
             (prompt_len < 1, "an empty prompt cannot be continued: give at least one token"),
             (max_new_tokens < 1, f"max_new_tokens is {max_new_tokens}; nothing would be generated"),
             (positions > self.runner.max_model_len,
              f"{prompt_len} prompt tokens and {max_new_tokens} new ones need {positions} positions; "
              f"the model stops at {self.runner.max_model_len}"),
-            (pages > self.manager.num_blocks,
-             f"{positions} tokens fill {pages} cache pages and the whole pool is {self.manager.num_blocks}"),
+            (bool(short), f"{positions} tokens fill {short[0][1] if short else 0} cache pages "
+                          f"and the whole pool is {pools[short[0][0]] if short else 0}"),
         )
         for failed, message in problems:
             if failed:
@@ -111,6 +127,8 @@ class ContinuousBatchingEngine:
         if strangers:
             raise ValueError(f"token ids {strangers[:5]} of the prompt are not in the vocabulary of {vocab} entries")
         rid = self._ids_issued if req_id is None else req_id
+        if any(r.req_id == rid for r in self.waiting) or any(r.req_id == rid for r in self.running):
+            raise ValueError(f"request id {rid} is already queued or running")
         self._ids_issued = max(self._ids_issued, rid + 1)
         when = perf_counter() if arrival_time is None else arrival_time
         self.waiting.append(Request(req_id=rid, prompt_ids=list(prompt_ids), params=params, arrival_time=when,
@@ -130,6 +148,8 @@ class ContinuousBatchingEngine:
         while self.running:
             self.manager.free_sequence(self.running.pop().req_id)
         self.waiting.clear()
+        with self._cancel_lock:
+            self._cancel.clear()  # (a stale cancellation must not hit a later request that reuses the id)
 
     # ================================================================== observation
     def has_unfinished(self) -> bool:
@@ -203,7 +223,7 @@ class ContinuousBatchingEngine:
             return False
         if self.waiting or self._cancel or not requests or len(requests) != len(self.running):
             return False
-        pages = 0
+        pages: dict[int, int] = {}
         for launched, live in zip(requests, self.running):
             if launched is not live or live.status is not Status.RUNNING:
                 return False  # another set of requests, or one has stopped meanwhile
@@ -211,8 +231,8 @@ class ContinuousBatchingEngine:
                 return False  # its known tokens are not all in the cache: it is not decoding
             if len(live.generated) + 2 > live.params.max_new_tokens:
                 return False  # the token on the device is its last: no step follows it
-            pages += self.manager.extra_blocks_needed(live.req_id, 1)
-        return pages <= self.manager.num_free_blocks
+            _add(pages, self.manager.pages_owed(live.req_id, 1, self._portion))
+        return _fits(pages, self.manager.free_pages())
 
     def _launch_continuation(self, events: list[TokenEvent]) -> None:
         requests, ids = self._in_flight
@@ -271,18 +291,23 @@ class ContinuousBatchingEngine:
             self._retire(request, reason, token, events)
 
     # ------------------------------------------------------------------ pages
-    def _pages_owed(self, request: Request) -> int:
-        """Pages the request has yet to take for tokens it already has."""
+    def _pages_owed(self, request: Request) -> dict[int, int]:
+        """Pages the request has yet to take for tokens it already has, per cache group."""
         missing = request.num_tokens - self.manager.lengths[request.req_id]
-        return self.manager.extra_blocks_needed(request.req_id, missing)
+        return self.manager.pages_owed(request.req_id, missing, self._portion)
+
+    def _all_owed(self) -> dict[int, int]:
+        owed: dict[int, int] = {}
+        for r in self.running:
+            _add(owed, self._pages_owed(r))
+        return owed
 
     def _evict_until_known_tokens_fit(self) -> bool:
         """Send the most recent admissions back to the queue until what remains can store its known
         tokens; the oldest request is never sent back.  True if anyone was."""
         evicted = False
         while len(self.running) > 1:
-            owed = sum(self._pages_owed(r) for r in self.running)
-            if owed <= self.manager.num_free_blocks:
+            if _fits(self._all_owed(), self.manager.free_pages()):
                 break
             victim = self.running.pop()
             self.manager.free_sequence(victim.req_id)
@@ -319,17 +344,19 @@ class ContinuousBatchingEngine:
             give(r, backlog[id(r)])
         if not admit:
             return shares
-        set_aside = sum(self._pages_owed(r) for r in self.running)
+        set_aside = self._all_owed()
         while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs:
             candidate = self.waiting[0]
-            pages = self.manager.blocks_for(candidate.num_tokens)
-            spare = len(self.running)  # one page per request already live stays free
-            if self.manager.num_free_blocks - set_aside - pages < spare or self.manager.num_free_slots < 1:
+            pages = self.manager.pages_for(candidate.num_tokens, self._portion)  # (what the cache manager says it costs)
+            wanted = dict(set_aside)
+            _add(wanted, pages)
+            spare = len(self.running)  # one page per request already live stays free, in every group
+            if not _fits(wanted, self.manager.free_pages(), spare) or self.manager.num_free_slots < 1:
                 break  # the head of the queue does not fit, and nobody overtakes it
             self.waiting.popleft()
             self.manager.add_sequence(candidate.req_id)
             candidate.status, candidate.num_computed_tokens = Status.RUNNING, 0
             self.running.append(candidate)
-            set_aside += pages
+            set_aside = wanted
             give(candidate, candidate.num_tokens)
         return shares

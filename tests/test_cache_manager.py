@@ -193,3 +193,75 @@ def test_sequence_lengths_give_table_lengths():
     for i in range(6):
         m.free_sequence(i)
     assert m.num_free_blocks == 64
+
+
+# ------------------------------------------------------------------ what a request costs, group by group
+def test_pages_are_counted_per_group_and_pools_have_sizes_of_their_own():
+    from llmserve.cache.manager import window_pages
+    from llmserve.parts.spec import StateCacheSpec
+
+    full, windowed, state = PagedCacheSpec(2, 16), PagedCacheSpec(2, 16, window=6), StateCacheSpec((5,), "float32")
+    groups = group_layers([full, windowed, state, full])
+    ids = {g.spec: g.group_id for g in groups}
+    m = CacheManager(groups, {ids[full]: 10, ids[windowed]: 4}, block_size=4, max_seqs=3)
+    assert m.capacity() == {ids[full]: 10, ids[windowed]: 4} and m.num_blocks == 4
+    # 30 tokens: 8 pages where every key stays; with a window of 6 and portions of up to 4 tokens no more than
+    # ceil((5 + 4) / 4) + 1 = 4; the state group costs no pages and is not named
+    assert window_pages(6, 4, 4) == 4
+    assert m.pages_for(30, step_tokens=4) == {ids[full]: 8, ids[windowed]: 4}
+    assert m.pages_for(30) == {ids[full]: 8, ids[windowed]: 8} and m.pages_for(3, step_tokens=4) == {ids[full]: 1, ids[windowed]: 1}
+    m.add_sequence("a")
+    for _ in range(7):  # 28 tokens in portions of 4: the windowed group never holds more than its 4 pages
+        m.append(["a"], [4])
+        m.release_passed(["a"])
+        assert m.allocators[ids[windowed]].num_used <= 4
+        m.check_invariants()
+    assert m.free_pages() == {ids[full]: 3, ids[windowed]: 2}
+    assert m.pages_owed("a", 9) == {ids[full]: 3, ids[windowed]: 3}
+    # many more tokens, in portions of 4: the windowed group is owed what brings the request to its most there
+    assert m.pages_owed("a", 90, step_tokens=4) == {ids[full]: 23, ids[windowed]: 4 - m.allocators[ids[windowed]].num_used}
+    assert not m.can_append(["a"], [9])  # the windowed group has 2
+    with pytest.raises(OutOfBlocks, match=f"group {ids[windowed]}"):
+        m.append(["a"], [9])
+    m.free_sequence("a")
+    assert m.free_pages() == m.capacity()
+    with pytest.raises(ValueError, match="every paged group"):
+        CacheManager(groups, {ids[full]: 10}, 4, 3)
+
+
+def test_a_model_of_fixed_size_state_alone_has_no_pages_to_run_out_of():
+    from llmserve.parts.spec import StateCacheSpec
+
+    m = CacheManager(group_layers([StateCacheSpec((8,), "float32")] * 3), 1, block_size=16, max_seqs=2)
+    assert m.capacity() == {} and m.pages_for(10_000, 64) == {} and m.free_pages() == {}
+    m.add_sequence(0)
+    assert m.pages_owed(0, 5000) == {} and m.can_append([0], [5000])
+    layout = m.append([0], [5000])
+    assert layout.slots == {} and m.lengths[0] == 5000 and m.utilization() == 0.0
+    m.add_sequence(1)
+    with pytest.raises(OutOfBlocks, match="state slots"):
+        m.add_sequence(2)
+
+
+def test_pools_are_sized_by_what_each_group_needs():
+    from llmserve.cache.storage import page_bytes_of, pool_sizes_for_budget, state_bytes
+    from llmserve.parts.spec import StateCacheSpec
+
+    full, windowed, state = PagedCacheSpec(4, 64), PagedCacheSpec(4, 64, window=128), StateCacheSpec((1000,), "float32")
+    groups = group_layers([full] * 30 + [windowed] * 2 + [state])
+    by_spec = {g.spec: g for g in groups}
+    fixed = state_bytes(groups, max_seqs=8)
+    assert fixed == 8 * 1000 * 4
+    budget = fixed + 50_000_000
+    sizes = pool_sizes_for_budget(groups, 16, 2, budget, max_seqs=8, longest=4096, step_tokens=512)
+    f, w = sizes[by_spec[full].group_id], sizes[by_spec[windowed].group_id]
+    # both groups hold the same number of longest requests: 256 pages each in the full group, 41 in the windowed
+    assert abs(f / 256 - w / 41) < 0.05 and w < f / 5
+    spent = f * page_bytes_of(by_spec[full], 16, 2) + w * page_bytes_of(by_spec[windowed], 16, 2)
+    assert 0.9 * 50_000_000 < spent <= 50_000_000
+    # never more than all slots could fill; the state alone may already be too much
+    roomy = pool_sizes_for_budget(groups, 16, 2, 10**12, max_seqs=8, longest=4096, step_tokens=512)
+    assert roomy == {by_spec[full].group_id: 8 * 256, by_spec[windowed].group_id: 8 * 41}
+    with pytest.raises(ValueError, match="fixed-size state"):
+        pool_sizes_for_budget(groups, 16, 2, fixed - 1, max_seqs=8, longest=4096, step_tokens=512)
+    assert pool_sizes_for_budget(group_layers([state]), 16, 2, budget, 8, 4096, 512) == {}

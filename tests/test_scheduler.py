@@ -306,3 +306,103 @@ def test_lagged_events_arrive_one_step_later_and_reset_forgets_them(weights):
     eng.reset()
     assert not eng.has_unfinished() and eng.manager.num_free_blocks == eng.manager.num_blocks
     assert eng.step() == []
+
+
+# ------------------------------------------------------------------ what a request costs is the cache manager's answer
+class CountingRunner:
+    """A step function for models that are not the reference's: the real cache manager over the given groups, and
+    logits that name (sum of the request's tokens so far) % vocab, kept per state slot as a model with fixed-size
+    state would keep it."""
+
+    def __init__(self, groups, num_blocks, block_size, max_seqs, vocab=50, max_model_len=4096):
+        from llmserve.cache import CacheManager
+
+        self.manager = CacheManager(groups, num_blocks, block_size, max_seqs)
+        self.vocab_size, self.max_model_len = vocab, max_model_len
+        self.sums = [0] * max_seqs
+        self.peak_used: dict[int, int] = {}
+
+    def step(self, entries):
+        layout = self.manager.append([e.seq_id for e in entries], [len(e.tokens) for e in entries])
+        for gid, a in self.manager.allocators.items():
+            self.peak_used[gid] = max(self.peak_used.get(gid, 0), a.num_used)
+        for slot in layout.fresh_slots:
+            self.sums[slot] = 0
+        rows = []
+        for e, slot in zip(entries, layout.state_slots):
+            for i, t in enumerate(e.tokens):
+                self.sums[slot] += t
+                if i in e.want:
+                    rows.append(torch.nn.functional.one_hot(torch.tensor(self.sums[slot] % self.vocab_size), self.vocab_size).float())
+        self.manager.release_passed(layout.seq_ids)
+        return torch.stack(rows) if rows else torch.empty(0, self.vocab_size)
+
+
+def counted(p, max_new, vocab=50):
+    ids = list(p)
+    for _ in range(max_new):
+        ids.append(sum(ids) % vocab)
+    return ids[len(p):]
+
+
+def test_a_model_that_keeps_only_fixed_size_state_is_served_with_default_sizing():
+    """No layer has pages: the pools are sized as the runner sizes them from a byte budget (none at all), and the
+    scheduler admits by slots alone; requests far longer than any page count would allow go through."""
+    from llmserve.cache import group_layers
+    from llmserve.cache.storage import pool_sizes_for_budget
+    from llmserve.parts.spec import StateCacheSpec
+
+    groups = group_layers([StateCacheSpec((6,), "float32")] * 2)
+    sizes = pool_sizes_for_budget(groups, 16, 2, 1 << 20, max_seqs=2, longest=4096, step_tokens=64)
+    assert sizes == {}
+    eng = ContinuousBatchingEngine(CountingRunner(groups, sizes, 16, 2), PlainSampler(), max_num_seqs=2,
+                                   max_num_batched_tokens=64)
+    prompts = [[(7 * i + j) % 50 for j in range(n)] for i, n in enumerate([48, 300, 5, 1000])]
+    ids = [eng.add_request(p, SamplingParams(max_new_tokens=6)) for p in prompts]
+    done = eng.run_until_complete()
+    for rid, p in zip(ids, prompts):
+        assert done[rid].generated == counted(p, 6)
+    assert eng.stats.preemptions == 0 and eng.manager.num_free_slots == 2
+    with pytest.raises(ValueError, match="positions"):
+        eng.add_request([1] * 4096, SamplingParams(max_new_tokens=1))
+
+
+def test_admission_charges_every_cache_group_what_it_costs_there():
+    """Two groups: one keeps every key (a large pool), one keeps a window of 8 keys (a small pool).  A prompt of 90
+    tokens costs 23 pages in the first and, in portions of up to 8 tokens, never more than 5 in the second, which
+    has 12: two such requests run side by side, where charging ceil(tokens / block_size) against the smaller
+    pool would refuse every one of them."""
+    from llmserve.cache import group_layers
+    from llmserve.parts.spec import PagedCacheSpec
+
+    full, windowed = PagedCacheSpec(1, 16), PagedCacheSpec(1, 16, window=8)
+    groups = group_layers([full, windowed])
+    gid = {g.spec: g.group_id for g in groups}
+    runner = CountingRunner(groups, {gid[full]: 60, gid[windowed]: 12}, 4, 3)
+    eng = ContinuousBatchingEngine(runner, PlainSampler(), max_num_seqs=3, max_num_batched_tokens=16, max_prefill_chunk=8)
+    prompts = [[(3 * i + j) % 50 for j in range(90)] for i in range(3)]
+    ids = [eng.add_request(p, SamplingParams(max_new_tokens=4)) for p in prompts]
+    eng.step()
+    assert len(eng.running) == 2 and len(eng.waiting) == 1  # the full group has room for two (2 x 24 + spare), not three
+    done = eng.run_until_complete()
+    for rid, p in zip(ids, prompts):
+        assert done[rid].generated == counted(p, 4)
+    assert runner.peak_used[gid[windowed]] <= 2 * 5 and runner.peak_used[gid[full]] >= 46
+    assert eng.manager.free_pages() == eng.manager.capacity() and eng.stats.preemptions == 0
+    with pytest.raises(ValueError, match="whole pool is 60"):  # the group that keeps every key is the one that refuses
+        eng.add_request([1] * 300, SamplingParams(max_new_tokens=4))
+
+
+def test_an_id_that_is_live_is_refused_and_reset_forgets_cancellations(weights):
+    eng = engine(weights, max_batch=2)
+    eng.add_request(prompt(5, 1), SamplingParams(max_new_tokens=3), req_id=7)
+    with pytest.raises(ValueError, match="already queued or running"):
+        eng.add_request(prompt(4, 2), SamplingParams(max_new_tokens=3), req_id=7)
+    eng.step()
+    with pytest.raises(ValueError, match="already queued or running"):
+        eng.add_request(prompt(4, 2), SamplingParams(max_new_tokens=3), req_id=7)
+    eng.abort(7)
+    eng.reset()  # the cancellation of the old request 7 must not hit a new one
+    eng.add_request(prompt(4, 2), SamplingParams(max_new_tokens=3), req_id=7)
+    done = eng.run_until_complete()
+    assert done[7].finish_reason == "length" and done[7].generated == reference(weights, prompt(4, 2), 3)
