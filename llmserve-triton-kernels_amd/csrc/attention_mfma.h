@@ -24,7 +24,10 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
 // llms_attention_mfma without the workspace: the partial results go through a fixed array in device memory
 // that the library owns, LLMS_ATTN_SCRATCH_BYTES per GPU for the life of the process.  The call allocates and
 // frees nothing (no hipMalloc, no hipFree, no allocating library routine); at its first call on a device it
-// asks the runtime once for the array's address there.
+// asks the runtime once for the array's address there (and the runtime, if nothing of this library has run on
+// that device yet, loads the library's code there, array included): make the first call outside a capture.
+//   cu_seqlens on the device must describe rows inside [token_begin, token_begin + n_tokens): the partial results
+//   are indexed by those rows, and a column whose row lies beyond is left out.
 //   Limit: (token_begin + n_tokens) * n_heads * num_splits * (head_dim + 2) * 4 bytes <= LLMS_ATTN_SCRATCH_BYTES,
 //   e.g. 64 rows x 32 heads x 8 splits at head_dim 128; a larger launch is refused (return code 1, message
 //   on stderr) and nothing runs.

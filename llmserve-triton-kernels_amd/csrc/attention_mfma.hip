@@ -76,6 +76,9 @@ struct AttnArgs {
     // zero between launches.  Non-null: the workgroups of a group count themselves here and the last to arrive adds
     // the shares up (no merge kernel).
     unsigned* arrive;
+    // token rows of the step that q, out and the workspace have: a column whose row lies beyond them (cu_seqlens on
+    // the device that disagree with what the caller sized its tensors by) is left out, not written past the end
+    int row_end;
     // prompts with twins: the first workgroup of every CU (the first `first_blocks` values of blockIdx.y) takes one
     // of the longest blocks of tokens, shortest of them first; the rest follow from the longest remaining one down
     int first_blocks;
@@ -306,7 +309,7 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
 
     // this lane's column
     const int c_tok = t_first + col / HG, c_head_in = hb * HG + col % HG;
-    const bool col_ok = col < HG * TPG && c_tok < n_new && c_head_in < G;
+    const bool col_ok = col < HG * TPG && c_tok < n_new && c_head_in < G && tok0 + c_tok < a.row_end;
     const int head = kvh * G + c_head_in;
     const int p_col = col_ok ? ctx - n_new + c_tok : -1;  // absolute position of the column's token
     const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
@@ -590,7 +593,7 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg) {
         c_tok[cg] = w_first + cg * TPG + col / HG;
-        col_ok[cg] = wave_on && col < HG * TPG && c_tok[cg] < n_new && c_head_in < G;
+        col_ok[cg] = wave_on && col < HG * TPG && c_tok[cg] < n_new && c_head_in < G && tok0 + c_tok[cg] < a.row_end;
         p_col[cg] = col_ok[cg] ? ctx - n_new + c_tok[cg] : -1;
         lo_col[cg] = (a.window > 0 && p_col[cg] - a.window + 1 > 0) ? p_col[cg] - a.window + 1 : 0;
     }
@@ -984,7 +987,7 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     const int groups = (max_new + TPG - 1) / TPG;
     AttnArgs a = {(bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pool, (const bf16*)v_pool,
                   block_tables, table_rows, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
-                  window, scale, num_splits, ws_o, ws_ml, nullptr, 0};
+                  window, scale, num_splits, ws_o, ws_ml, nullptr, token_begin + n_tokens, 0};
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
     LLMS_REQUIRE((unsigned long long)max_blocks * block_size * block_size <= 0xFFFFFFFFull,
                  "attention_mfma: block table too long for this page size (keys * block_size must stay below 2^32)");

@@ -71,6 +71,7 @@ class ModelRunner:
         self.manager = CacheManager(groups, num_blocks, self.block_size, engine_config.max_num_seqs)
         self.storage = CacheStorage(groups, num_blocks, self.block_size, engine_config.max_num_seqs,
                                     self.dtype, device, table_width=-(-self.max_model_len // self.block_size))
+        ops.reset_arrival_counters(device)  # (whatever an earlier runner's failed step may have left)
         self._uploader = BatchUploader(device)
         self._graphs: dict[tuple[int, int], "_DecodeGraph"] = {}
         self._use_graphs = engine_config.use_graphs and model.graph_safe()
@@ -191,22 +192,30 @@ class ModelRunner:
             row += len(e.tokens)
         logit_rows = [first_row[id(e)] + w for e in entries for w in e.want]
         self.storage.clear_state(layout.fresh_slots)
-        owned = True
-        if not self._use_graphs:  # launched kernel by kernel, on exactly the step's tokens
-            batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
-            logits = self.model.forward(batch, self.storage)
-        elif all(len(e.tokens) == 1 for e in ordered):
-            logits = self._replay_decode(layout, [e.tokens[0] for e in ordered], logit_rows, device_tokens)
-            owned = False
-        elif self._launch_bound(sum(layout.counts)):
-            logits, owned = self._run_bucketed_step(layout, [e.tokens for e in ordered], logit_rows)
-        else:  # the device is busy for longer than the host needs to launch the step: nothing to gain from a graph
-            batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
-            logits = self.model.forward(batch, self.storage)
-            self.rows_run += sum(layout.counts)
-            self.rows_asked += sum(layout.counts)
+        try:
+            logits, owned = self._run(layout, ordered, logit_rows, device_tokens)
+        except BaseException:
+            # a launch that failed half-way may have left workgroups counted where the next step counts again
+            ops.reset_arrival_counters(self.device)
+            raise
         self.manager.release_passed(layout.seq_ids)
         return logits if owned or borrow else logits.clone()
+
+    def _run(self, layout, ordered: list[StepEntry], logit_rows: list[int], device_tokens) -> tuple[torch.Tensor, bool]:
+        """The step's logits and whether the caller owns them (not a view of a graph's memory)."""
+        if not self._use_graphs:  # launched kernel by kernel, on exactly the step's tokens
+            batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
+            return self.model.forward(batch, self.storage), True
+        if all(len(e.tokens) == 1 for e in ordered):
+            return self._replay_decode(layout, [e.tokens[0] for e in ordered], logit_rows, device_tokens), False
+        if self._launch_bound(sum(layout.counts)):
+            return self._run_bucketed_step(layout, [e.tokens for e in ordered], logit_rows)
+        # the device is busy for longer than the host needs to launch the step: nothing to gain from a graph
+        batch = build_batch(layout, [e.tokens for e in ordered], logit_rows, self._uploader, self.storage)
+        logits = self.model.forward(batch, self.storage)
+        self.rows_run += sum(layout.counts)
+        self.rows_asked += sum(layout.counts)
+        return logits, True
 
     # ---- decode-only steps as HIP graphs --------------------------------------------------------
     @staticmethod

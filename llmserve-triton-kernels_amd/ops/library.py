@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import os
 import threading
 
 import torch
@@ -520,18 +521,39 @@ def gemm_slices(parts: torch.Tensor, x: torch.Tensor, w: torch.Tensor) -> torch.
 
 _ARRIVAL_COUNTERS: dict = {}
 ARRIVAL_COUNTERS = 1 << 16
+# LLMSERVE_ATTN_MERGE=kernel: the shares of a split decode attention are always added up by the second kernel
+MERGE_BY_KERNEL = os.environ.get("LLMSERVE_ATTN_MERGE", "") == "kernel"
 
 
 def _arrival_counters(dev) -> torch.Tensor | None:
-    """The device's counters for workgroups that add each other's shares up inside a kernel: all zero, and every
-    kernel that uses them leaves them so.  Made at the first call that is not being captured into a graph (a fill
-    inside a graph would run at every replay); until then there are none and the caller takes its other way."""
+    """The device's counters for workgroups that add each other's shares up inside a kernel: all zero between
+    launches, and every kernel that uses them leaves them so.  Launches that use them must not overlap in time:
+    the engine keeps all of a device's steps on one stream (a graph replays where its launches were ordered at
+    capture), and whoever runs decode attention with splits on two streams at once passes `merge_kernel=True`
+    (or sets LLMSERVE_ATTN_MERGE=kernel).  Made at the first call that is not being captured into a graph (a fill
+    inside a graph would run at every replay); until then there are none and the caller takes its other way.  A
+    launch that dies half-way may leave a count behind: whoever catches such an error calls
+    `reset_arrival_counters` before the next step (the runner does)."""
     key = (dev.type, dev.index)
     if key not in _ARRIVAL_COUNTERS:
         if torch.cuda.is_current_stream_capturing():
             return None
         _ARRIVAL_COUNTERS[key] = torch.zeros(ARRIVAL_COUNTERS, dtype=torch.int32, device=dev)
     return _ARRIVAL_COUNTERS[key]
+
+
+def reset_arrival_counters(dev=None) -> None:
+    """Zero the counters (of one device, or of all): after an error in the middle of a step, and when a runner is
+    built.  A small fill kernel, on the current stream."""
+    for (kind, index), counters in _ARRIVAL_COUNTERS.items():
+        if dev is None or (kind, index) == (dev.type, dev.index):
+            counters.zero_()
+
+
+def arrival_counters_are_zero(dev=None) -> bool:
+    """Whether every launch so far has left its counters as it found them (tests ask after their workloads)."""
+    return all(int(c.abs().max()) == 0 for (kind, index), c in _ARRIVAL_COUNTERS.items()
+               if dev is None or (kind, index) == (dev.type, dev.index))
 
 
 def _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size):
@@ -636,7 +658,7 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
     if n_seqs == 0 or n_tokens == 0:
         return out
     ws_o = ws_ml = arrive = None
-    if num_splits > 1 and split_waves and not merge_kernel:
+    if num_splits > 1 and split_waves and not (merge_kernel or MERGE_BY_KERNEL):
         arrive = _arrival_counters(dev)
     if num_splits > 1:
         ws_o = torch.empty((q.shape[0] * n_heads * num_splits * head_dim,), dtype=torch.float32, device=dev)

@@ -121,3 +121,19 @@ def test_engine_config_validation():
     for bad in (dict(dtype="float16"), dict(block_size=0), dict(num_blocks=0), dict(max_num_seqs=0)):
         with pytest.raises(ValueError):
             EngineConfig(**bad).validate()
+
+
+def test_a_length_limit_beyond_the_models_positions_is_refused():
+    """src/llmserve/utils.py:8-13 of the reference refuses it; so does the runner, before it takes any memory."""
+    import torch
+
+    from llmserve.engine.runner import ModelRunner
+    from llmserve.parts.model import Model
+    from llmserve.parts.registry import BuildContext
+
+    arch = architecture_of(TINY_B)
+    cfg = LlamaConfig.from_dict(TINY_B)
+    model = Model(arch.build_spec(cfg), BuildContext(torch.float32, torch.device("cpu")))
+    limit = TINY_B["max_position_embeddings"]
+    with pytest.raises(ValueError, match=f"more than the model's {limit} positions"):
+        ModelRunner(model, cfg, EngineConfig(dtype="float32", max_model_len=limit + 1, num_blocks=4), torch.device("cpu"))

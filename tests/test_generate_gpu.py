@@ -194,6 +194,55 @@ def test_temperature_sampling_is_seeded_and_matches_plain_sampler(model_dirs):
             assert lo - 1e-5 <= u < float(cdf[tok]) + 1e-5, (i, tok, u, lo, float(cdf[tok]))
 
 
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_requests_with_their_own_sampling_options_share_a_batch(model_dirs, dtype_name):
+    """Greedy requests beside requests with temperature, top-k, top-p and seeds of their own, in one batch through
+    the scheduler and the device sampler (ids read a step late; the reference's engine test runs top_k=20:
+    tests/test_scheduler.py:122-131 there).  Every token is what the plain sampler picks from the plain logits
+    with the same uniform number: exactly in 32-bit; in bfloat16 within what the logits' rounding moves the
+    distribution, and never a token that the filters of the plain logits exclude by more than that rounding."""
+    from llmserve import SamplingParams
+    from llmserve.sampling import uniform
+
+    name = "b"
+    vocab = TINY[name][0]["vocab_size"]
+    dtype = getattr(torch, dtype_name)
+    prompts = [traces.random_ids(vocab, n, 800 + i) for i, n in enumerate([3, 30, 11, 64, 7, 19])]
+    params = [SamplingParams(max_new_tokens=14),
+              SamplingParams(temperature=0.9, top_k=20, seed=11, max_new_tokens=14),
+              SamplingParams(temperature=1.3, top_p=0.9, seed=12, max_new_tokens=14),
+              SamplingParams(max_new_tokens=9),
+              SamplingParams(temperature=0.7, top_k=5, top_p=0.8, seed=13, max_new_tokens=14),
+              SamplingParams(temperature=1.0, seed=14, max_new_tokens=14)]
+    llm = _llm(model_dirs[name], name, dtype_name, max_num_batched_tokens=48)
+    results = [r.tokens for r in llm.generate(prompts, params)]
+    assert llm.engine.stats.steps > 14 and [len(t) for t in results] == [p.max_new_tokens for p in params]
+    if dtype_name == "float32":  # another way of cutting the same work: the same tokens
+        again = _llm(model_dirs[name], name, dtype_name, max_num_batched_tokens=2048, use_graphs=False)
+        assert [r.tokens for r in again.generate(prompts, params)] == results
+    cfg, w = plain_llama.read_model_dir(model_dirs[name], dtype)
+    for p, sp, toks in zip(prompts, params, results):
+        logits = plain_llama.forward(cfg, w, p + toks, dtype).float()
+        max_tol, _ = traces.tolerance(dtype, logits)
+        for i, tok in enumerate(toks):
+            row = logits[len(p) - 1 + i]
+            if sp.temperature == 0:
+                slack = 0.0 if dtype_name == "float32" else 2 * max_tol
+                assert row.max() - row[tok] <= slack, (i, tok)
+                continue
+            probs = plain_llama.filtered_probs(row, sp.temperature, sp.top_k, sp.top_p)
+            cdf = probs.cumsum(-1)
+            u = uniform(sp.seed, i)
+            lo = float(cdf[tok - 1]) if tok > 0 else 0.0
+            # the logits' rounding moves every probability by about that much relative to itself, so a cumulated sum
+            # by no more than that in all
+            slack = 1e-5 if dtype_name == "float32" else 4 * max_tol / sp.temperature
+            assert lo - slack <= u < float(cdf[tok]) + slack, (i, tok, u, lo, float(cdf[tok]))
+            if sp.top_k:  # inside the plain top-k, or tied with its last member within the rounding
+                kth = row.topk(sp.top_k).values[-1]
+                assert row[tok] >= kth - (0.0 if dtype_name == "float32" else 2 * max_tol), (i, tok)
+
+
 def test_warm_up_captures_the_decode_graphs_ahead(model_dirs):
     """After `warm_up` no decode step has to capture anything, and the tokens are the same as without it."""
     from llmserve import SamplingParams

@@ -603,7 +603,9 @@ def test_sampler_reference_vector():
 @pytest.mark.parametrize("vocab,temperature,top_k,top_p", [(333, 0.8, 0, 1.0), (32000, 1.0, 50, 1.0),
                                                            (32000, 0.7, 0, 0.9), (5000, 1.3, 40, 0.5),
                                                            (50257, 1.0, 0, 1.0), (50257, 0.9, 30, 0.8),
-                                                           (32768, 0.9, 64, 0.95), (32769, 1.1, 0, 0.7)])
+                                                           (32768, 0.9, 64, 0.95), (32769, 1.1, 0, 0.7),
+                                                           # (more survivors of top-k than the kernel gathers before top-p)
+                                                           (32000, 0.9, 2000, 0.9), (50257, 1.2, 1500, 0.6)])
 def test_sample_rows_inverts_the_plain_cdf(vocab, temperature, top_k, top_p):
     rows = 24
     logits = rnd(rows, vocab, seed=41, scale=3.0)

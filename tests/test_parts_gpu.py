@@ -237,8 +237,9 @@ class ToyConfig:
 
 def register_toy():
     from llmserve.config import register_architecture
-    from llmserve.parts import (FeedForward, LayerSpec, Mixer, ModelSpec, ParamInfo, PartSpec, PositionEncoding,
-                                StateCacheSpec, register_feed_forward, register_mixer, register_position_encoding)
+    from llmserve.parts import (Block, FeedForward, LayerSpec, Mixer, ModelSpec, ParamInfo, PartSpec, PositionEncoding,
+                                StateCacheSpec, register_block, register_feed_forward, register_mixer,
+                                register_position_encoding)
     from llmserve.parts.linear import linear
 
     @register_position_encoding("interleaved")
@@ -322,6 +323,21 @@ def register_toy():
                 row += n
             return linear(means.to(x.dtype), self.weight)
 
+    @register_block("sandwich")
+    class SandwichBlock(Block):
+        """x = x + post_norm(mixer(norm1(x))); x = x + feed_forward(norm2(x)): an arrangement with a third norm, a
+        role the reference's layer does not have.  The model builds, loads and names the tensors of whatever
+        roles an arrangement declares."""
+
+        ROLES = dict(Block.ROLES, post_mixer_norm="norm")
+
+        def forward(self, x, delta, batch, cache):
+            h = self.mixer_norm.add_norm(x, delta)  # (x += delta in place)
+            a = self.mixer.forward(h, batch, cache)
+            a = self.post_mixer_norm.forward(a if isinstance(a, torch.Tensor) else a.total())
+            h2 = self.feed_forward_norm.add_norm(x, a)
+            return x, self.feed_forward.forward(h2)
+
     def toy_spec(cfg: ToyConfig) -> ModelSpec:
         h = cfg.hidden_size
         norm = PartSpec("rmsnorm", {"hidden": h, "eps": cfg.eps})
@@ -339,11 +355,12 @@ def register_toy():
             p = f"toy.{i}."
             ffn = (PartSpec("soft_experts", {"hidden": h, "intermediate": inter, "experts": 3}) if i == 2
                    else PartSpec("swiglu", {"hidden": h, "intermediate": inter}))
-            layers.append(LayerSpec(
-                parts={"mixer": mixer, "feed_forward": ffn, "mixer_norm": norm, "feed_forward_norm": norm},
-                cache_from=0 if i == 3 else None,
-                weights={"mixer": p + "mix.", "feed_forward": p + "ffn.", "mixer_norm": p + "n1.",
-                         "feed_forward_norm": p + "n2."}))
+            parts = {"mixer": mixer, "feed_forward": ffn, "mixer_norm": norm, "feed_forward_norm": norm}
+            weights = {"mixer": p + "mix.", "feed_forward": p + "ffn.", "mixer_norm": p + "n1.", "feed_forward_norm": p + "n2."}
+            if i == 1:  # the layer that runs twice has a third norm
+                parts["post_mixer_norm"], weights["post_mixer_norm"] = norm, p + "n3."
+            layers.append(LayerSpec(parts=parts, weights=weights, block="sandwich" if i == 1 else "prenorm",
+                                    cache_from=0 if i == 3 else None))
         return ModelSpec(hidden_size=h, vocab_size=cfg.vocab_size, max_positions=128,
                          embedding=PartSpec("embedding", {"vocab": cfg.vocab_size, "hidden": h}),
                          layers=tuple(layers), schedule=(0, 1, 2, 3, 1), final_norm=norm,
@@ -397,6 +414,8 @@ def plain_toy_forward(w, ids, dtype):
             a = pl.linear(means.to(dtype), w[p + "mix.proj.weight"])
         else:
             a = attention(3, hn, 2, 2, 16, 777.0, None, borrow=0)
+        if i == 1:
+            a = pl.rms_norm(a, w[p + "n3.weight"], eps)
         x = x + a
         hn2 = pl.rms_norm(x, w[p + "n2.weight"], eps)
         if i == 2:  # the routed feed-forward

@@ -24,13 +24,13 @@ def sequences(name: str) -> dict[str, list[int]]:
     return {f"{name}{i}": traces.random_ids(vocab, n, 1000 + 17 * i) for i, n in enumerate(LENGTHS[name])}
 
 
-def replay_in_process(model_dir, dtype_name, steps, block_size, num_blocks, use_graphs=True):
+def replay_in_process(model_dir, dtype_name, steps, block_size, num_blocks, use_graphs=True, max_seqs=4):
     from llmserve.config import EngineConfig
     from llmserve.engine.replay import Replayer
     from llmserve.engine.runner import ModelRunner
 
     runner = ModelRunner.from_folder(model_dir, EngineConfig(dtype=dtype_name, block_size=block_size,
-                                                              num_blocks=num_blocks, max_num_seqs=4,
+                                                              num_blocks=num_blocks, max_num_seqs=max_seqs,
                                                               use_graphs=use_graphs))
     runner.storage.poison()  # a slot that was never written must never be read
     rep = Replayer(runner)
@@ -41,7 +41,9 @@ def replay_in_process(model_dir, dtype_name, steps, block_size, num_blocks, use_
         if logits.shape[0]:
             outputs[rec["step"]] = logits.float().cpu()
     assert runner.manager.num_free_blocks == num_blocks, "pages were not all returned"
-    assert runner.manager.num_free_slots == 4, "state slots were not all returned"
+    assert runner.manager.num_free_slots == max_seqs, "state slots were not all returned"
+    from llmserve.ops import library as ops
+    assert ops.arrival_counters_are_zero(), "a decode attention left workgroups counted"
     return outputs
 
 
@@ -212,6 +214,55 @@ def test_replay_at_full_layer_sizes(wide_model_dir, dtype_name, mode, monkeypatc
     check_against_plain(model_dir, dtype_name, seqs, steps, outputs)
     if dtype_name == "bfloat16" and mode == "portions":
         assert any(not waves and splits > 1 for waves, splits in shared_out), "no portion shared its keys out"
+
+
+@pytest.mark.parametrize("use_graphs", [True, False], ids=["graphs", "launches"])
+@pytest.mark.parametrize("live", [20, 48])
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_many_live_requests_at_full_layer_sizes(wide_model_dir, dtype_name, live, use_graphs):
+    """17 to 64 rows at the widths of real models: the products for that many rows (a slice of all rows in LDS for
+    o_proj and down_proj, the library's product and the activation kernel for gate and up, the rotary epilogue over
+    several blocks of rows, the library's head), decode graphs for 32 and 64 requests.  Prompts come in portions
+    beside decoded tokens of others; then all requests decode side by side."""
+    model_dir, cfg = wide_model_dir
+    if cfg["hidden_size"] > 4096:
+        pytest.skip("the 1.1B and 7B widths cover the arrangement; the 70B width is replayed with four requests above")
+    import random
+
+    rng = random.Random(live)
+    seqs = {f"m{i}": traces.random_ids(cfg["vocab_size"], rng.randint(12, 70), 3000 + i) for i in range(live)}
+    # portions of some prompts beside decoded tokens of requests whose prompt is in, until every request has at
+    # most 5 tokens to go; then all of them decode side by side
+    pos = {rid: 0 for rid in seqs}
+    steps = []
+
+    def step_of(entries):
+        ended = [e["id"] for e in entries if pos[e["id"]] == len(seqs[e["id"]])]
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+
+    def bring(rid, n):
+        ids = seqs[rid]
+        entry = {"id": rid, "tokens": ids[pos[rid]:pos[rid] + n], "want": list(range(n))}
+        pos[rid] += n
+        return entry
+
+    while any(len(ids) - pos[rid] > 5 for rid, ids in seqs.items()):
+        entries = []
+        for rid, ids in seqs.items():
+            to_go = len(ids) - pos[rid]
+            if to_go > 5 and rng.random() < 0.5:
+                entries.append(bring(rid, min(rng.choice([2, 3, 5, 8, 13, 24]), to_go - 5)))
+            elif 2 < to_go <= 5 and rng.random() < 0.2:
+                entries.append(bring(rid, 1))
+        if entries:
+            step_of(entries)
+    while any(pos[rid] < len(ids) for rid, ids in seqs.items()):
+        step_of([bring(rid, 1) for rid, ids in seqs.items() if pos[rid] < len(ids)])
+    assert any(len(rec["entries"]) == live and all(len(e["tokens"]) == 1 for e in rec["entries"]) for rec in steps)
+    assert any(len(rec["entries"]) > 16 and any(len(e["tokens"]) > 1 for e in rec["entries"]) for rec in steps) or live <= 20
+    num_blocks = traces.tokens_needed(steps, round_to=16) // 16
+    outputs = replay_in_process(model_dir, dtype_name, steps, 16, num_blocks, use_graphs=use_graphs, max_seqs=live)
+    check_against_plain(model_dir, dtype_name, seqs, steps, outputs)
 
 
 @pytest.mark.parametrize("seed", [1, 2, 3, 4])

@@ -67,14 +67,20 @@ def test_decode_attention_without_allocation_matches_the_workspace_entry_point()
     big, big_ref = decode_case(32, 4, 64, 16, [600, 31, 257, 1, 90, 333], seed=5)
     small, small_ref = decode_case(8, 2, 128, 8, [150, 40], seed=9)
     out_big, out_small = new_out(big), new_out(small)
-    # neither call takes memory from the device: torch's pool and its counters stay as they are (the fixed
-    # array was placed when the library was loaded)
+    # A first call outside the measurement: it loads the library's code object onto the device (which places the
+    # fixed array) and asks for the array's address; callers under graph capture make it before they capture.
+    warm, _ = decode_case(4, 2, 32, 8, [9], seed=2)
+    assert call_noalloc(lib, warm, 2, 4, new_out(warm))[0] == 0
+    # Neither of the two calls takes memory from the device: the free memory of the whole device (which a hipMalloc
+    # behind torch's back would lower as well) and torch's own counters stay as they are.
     torch.cuda.synchronize()
+    free_before, _total = torch.cuda.mem_get_info()
     reserved_before, allocated_before = torch.cuda.memory_reserved(), torch.cuda.memory_allocated()
     status_big, got_big = call_noalloc(lib, big, 5, 8, out_big)
     status_small, got_small = call_noalloc(lib, small, 3, 4, out_small)  # right behind it, over what the first call left
     torch.cuda.synchronize()
     assert status_big == 0 and status_small == 0
+    assert torch.cuda.mem_get_info()[0] == free_before
     assert torch.cuda.memory_reserved() == reserved_before and torch.cuda.memory_allocated() == allocated_before
     for case, got, ref, splits, waves in ((big, got_big, big_ref, 5, 8), (small, got_small, small_ref, 3, 4)):
         want = call_with_workspace(ops, case, splits, waves)
