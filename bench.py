@@ -8,9 +8,13 @@ scheduler steps (step function + sampling + the read-back of the token ids) afte
 ones, with synchronisation on both sides.  `prefill` is one request of 2,048 tokens in one
 step (`chunked`: the same prompt in portions of 512 tokens, the scheduler cutting it);
 `roofline` prices the decode step against HBM bandwidth (every weight it uses read once, plus
-the keys and values of the live requests); `points` holds decode at batch 1 and 64;
-`measured_peaks` is what this box delivers to a plain device copy and to a large library
-matrix product, the practical ceilings beside the published ones.
+the keys and values of the live requests); `points` holds decode at further batch sizes
+(1, 16, 24, 32, 64: the step grows with the blocks of 16 rows) and, at the default batch, behind
+contexts of 2,048 and 4,096 tokens; `serve` is a short continuous-batching run on the same model
+(requests with random prompt lengths arriving at once: tokens a second, time to first token,
+inter-token latency); `peak_mib` is the most device memory the process held; `measured_peaks` is
+what this box delivers to a plain device copy and to a large library matrix product, the
+practical ceilings beside the published ones.
 
     python bench.py --workload serve [--model llama2-7b] [--requests 64] [--new-tokens 256]
                     [--prompt-min 128] [--prompt-max 2048] [--pages-fraction 1.0]
@@ -38,6 +42,7 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}  # dense matrix-core peaks, MI355X
 PREFILL_TOKENS = 2048
 PREFILL_CHUNK = 512  # the portion size of the chunked prefill measurement
+MODEL_NAMES = {"tinyllama-1.1b": "TinyLlama 1.1B", "llama2-7b": "Llama-2-7B", "llama2-70b": "Llama-2-70B"}
 
 
 def measured_peaks(torch) -> dict:
@@ -66,6 +71,40 @@ def percentile(values, q):
     if not values:
         return 0.0
     return values[min(len(values) - 1, int(q * len(values)))]
+
+
+def serve_summary(torch, runner, sampler, vocab: int, budget: int, max_seqs: int, requests: int = 32,
+                  new_tokens: int = 64) -> dict:
+    """A short continuous-batching run on a runner that is already there: `requests` requests with seeded random
+    prompt lengths of 64 to 1,024 tokens that all arrive at once, `new_tokens` each (the figures of the reference's
+    benchmarks/run_benchmark.py:85-91: tokens a second, time to first token, inter-token latency, peak memory)."""
+    from llmserve import SamplingParams
+    from llmserve.engine.scheduler import ContinuousBatchingEngine
+
+    gen = torch.Generator().manual_seed(7)
+    requests = min(requests, max_seqs)
+    lengths = torch.randint(64, 1025, (requests,), generator=gen).tolist()
+    lo = min(100, vocab // 4)
+    texts = [torch.randint(lo, vocab, (n,), generator=gen).tolist() for n in lengths]
+    need = sum(-(-(n + new_tokens + 1) // runner.block_size) + 1 for n in lengths)
+    if need > runner.manager.num_blocks:
+        return {}
+    runner.warm_up(requests, max(lengths) + new_tokens + 1)  # a server captures its decode graphs after loading
+    eng = ContinuousBatchingEngine(runner, sampler, max_num_seqs=requests, max_num_batched_tokens=budget)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ids = [eng.add_request(p, SamplingParams(max_new_tokens=new_tokens), arrival_time=t0) for p in texts]
+    while eng.has_unfinished():
+        eng.step()
+    torch.cuda.synchronize()
+    total_s = time.perf_counter() - t0
+    reqs = [eng.finished[i] for i in ids]
+    ttft = [r.token_times[0] - r.arrival_time for r in reqs]
+    itl = [b - a for r in reqs for a, b in zip(r.token_times, r.token_times[1:])]
+    return {"requests": requests, "prompt_tokens": sum(lengths), "new_tokens": new_tokens,
+            "value": round(sum(len(r.generated) for r in reqs) / total_s, 1),
+            "ttft_p50_ms": round(percentile(ttft, 0.5) * 1e3, 2), "itl_p50_ms": round(percentile(itl, 0.5) * 1e3, 3),
+            "itl_p99_ms": round(percentile(itl, 0.99) * 1e3, 3), "preemptions": eng.stats.preemptions}
 
 
 def serve(args) -> int:
@@ -132,6 +171,7 @@ def serve(args) -> int:
         "itl_ms": {"p50": round(percentile(itl, 0.5) * 1e3, 3), "p90": round(percentile(itl, 0.9) * 1e3, 3),
                    "p99": round(percentile(itl, 0.99) * 1e3, 3), "max": round(max(itl) * 1e3, 3)},
         "preemptions": eng.stats.preemptions,
+        "peak_mib": round(torch.cuda.max_memory_allocated() / 2 ** 20, 1),
         # rows the steps held, rows that ran with the padding of buckets and graphs, and the padded fraction
         "rows": {"asked": runner.rows_asked, "run": runner.rows_run,
                  "padding": round(runner.rows_run / max(runner.rows_asked, 1) - 1, 4)},
@@ -205,89 +245,6 @@ def gemv(args) -> int:
     return 0
 
 
-def sync_costs(args) -> int:
-    """What the two ways of ordering dependent work on the GPU cost (csrc/probe.hip): a kernel boundary in a
-    captured chain of launches, and a barrier over all workgroups inside one kernel, without and with the fences
-    that make stores visible across XCDs.  The decode step is a chain of kernels because of these figures."""
-    import ctypes
-
-    import torch
-
-    from llmserve.ops import library as ops
-
-    lib = ops.load("probe")
-    scratch = torch.zeros(1024 * 256 + 16, dtype=torch.float32, device="cuda:0")
-    results = (ctypes.c_float * 12)()
-    torch.cuda.synchronize()
-    status = lib.llms_probe_sync(results, ctypes.c_void_p(scratch.data_ptr()))
-    if status != 0:
-        print(f"the probe failed with status {status}")
-        return 1
-    r = [round(float(v), 2) for v in results]
-    hand = (ctypes.c_float * 16)()
-    space = torch.zeros(1024 * 768 + 2048, dtype=torch.float32, device="cuda:0")
-    torch.cuda.synchronize()
-    status = lib.llms_probe_handover(hand, ctypes.c_void_p(space.data_ptr()))
-    if status != 0:
-        print(f"the probe failed with status {status}")
-        return 1
-    h = [round(float(v), 2) for v in hand]
-    cases = ["64_workgroups_in_pairs", "64_workgroups_in_eights", "256_workgroups_in_fours", "1024_workgroups_in_fours"]
-    handover = {name: {"stores_only": h[3 * i], "atomic_accesses_no_fence": h[3 * i + 1], "fences": h[3 * i + 2]}
-                for i, name in enumerate(cases)}
-    line = {"metric": "microseconds per kernel boundary in a captured chain of launches", "value": r[1], "unit": "us",
-            "n_gpus": 1, "steps": 0, "warmup": 0, "ms_per_step": 0.0, "higher_is_better": False, "scaling": "weak",
-            "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"parallelism": "single-gpu"},
-            "kernel_boundary_us": {"8_workgroups": r[0], "256_workgroups": r[1], "1024_workgroups": r[2]},
-            "grid_barrier_us": {"64": r[3], "256": r[4], "512": r[5], "1024": r[6]},
-            "grid_barrier_with_fences_us": {"64": r[7], "256": r[8], "512": r[9]},
-            "spin_limits_hit": r[10], "stale_reads": r[11],
-            # a launch in which the last workgroup of every group reads what the others of the group wrote
-            "handover_us_per_launch": handover, "handover_stale_reads": h[12]}
-    print(json.dumps(line))
-    return 0
-
-
-def stream_rates(args) -> int:
-    """What memory gives a kernel that only reads (csrc/probe.hip): a gigabyte in one launch, by three ways of
-    sharing the addresses out to a wave's lanes, and pieces as large as the weight matrices of a decode step, each
-    in a launch of its own within a captured chain: the least that a product which must read such a matrix costs."""
-    import ctypes
-
-    import torch
-
-    from llmserve.config import preset
-    from llmserve.ops import library as ops
-
-    cfg = preset(args.model)
-    h, inter, nh, nkv = cfg["hidden_size"], cfg["intermediate_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
-    d = h // nh
-    pieces = {"qkv": (nh + 2 * nkv) * d * h * 2, "o_proj": h * nh * d * 2, "gate_up": 2 * inter * h * 2, "down_proj": h * inter * 2}
-    lib = ops.load("probe")
-    total = max(1 << 30, 16 * max(pieces.values()))
-    buf = torch.empty(total, dtype=torch.uint8, device="cuda:0")
-    sink = torch.zeros(4, dtype=torch.int32, device="cuda:0")
-    results = (ctypes.c_float * 16)()
-    sizes = (ctypes.c_size_t * len(pieces))(*pieces.values())
-    torch.cuda.synchronize()
-    lib.llms_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
-    status = lib.llms_probe_stream(results, ctypes.c_void_p(buf.data_ptr()), total, sizes, len(pieces), ctypes.c_void_p(sink.data_ptr()))
-    if status != 0:
-        print(f"the probe failed with status {status}")
-        return 1
-    r = [float(v) for v in results]
-    per_piece = {name: {"MB": round(nbytes / 1e6, 1), "us": round(r[3 + i], 2), "GBps": round(nbytes / r[3 + i] / 1e3, 1)}
-                 for i, (name, nbytes) in enumerate(pieces.items())}
-    line = {"metric": "GB/s of a kernel that reads 1 GiB once, 1 KB of a row per instruction", "value": round(r[0], 1),
-            "unit": "GB/s", "n_gpus": 1, "steps": 0, "warmup": 0, "ms_per_step": 0.0, "higher_is_better": True,
-            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-            "config": {"model": args.model, "parallelism": "single-gpu", "bytes": total},
-            "stream_GBps": {"1KB_of_a_row": round(r[0], 1), "64B_of_16_rows": round(r[1], 1), "256B_of_4_rows": round(r[2], 1)},
-            "one_launch_per_matrix": per_piece}
-    print(json.dumps(line))
-    return 0
-
-
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -299,11 +256,12 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--model", default="tinyllama-1.1b")
     ap.add_argument("--no-points", action="store_true", help="skip the further batch sizes")
-    ap.add_argument("--points", default="1,64", help="further batch sizes to measure decoding at")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill", "gemv", "sync", "stream"], default="all",
+    ap.add_argument("--points", default="1,16,24,32,64", help="further batch sizes to measure decoding at")
+    ap.add_argument("--context-points", default="2048,4096", help="further context lengths to measure decoding at (default batch)")
+    ap.add_argument("--no-serve", action="store_true", help="skip the short continuous-batching run")
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "gemv"], default="all",
                     help="run one phase only (for profiles; the line then holds zeros for the other); gemv: the "
-                         "decode products alone, each over copies of its weight that do not fit the caches; sync: what a kernel "
-                         "boundary and a barrier inside a kernel cost; stream: what memory gives a kernel that only reads")
+                         "decode products alone, each over copies of its weight that do not fit the caches")
     ap.add_argument("--workload", choices=["steps", "serve"], default="steps")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
@@ -319,10 +277,6 @@ def main() -> int:
         return serve(args)
     if args.phase == "gemv":
         return gemv(args)
-    if args.phase == "sync":
-        return sync_costs(args)
-    if args.phase == "stream":
-        return stream_rates(args)
 
     import torch
 
@@ -342,16 +296,22 @@ def main() -> int:
     d = h // nh
     elem = 2 if args.dtype == "bfloat16" else 4
     block_size = 16
-    point_batches = [int(b) for b in args.points.split(",") if b] if not args.no_points and args.phase == "all" else []
+    extra = not args.no_points and args.phase == "all"
+    point_batches = [int(b) for b in args.points.split(",") if b] if extra else []
+    point_contexts = [int(c) for c in args.context_points.split(",") if c] if extra else []
     max_batch = max([args.batch] + point_batches)
     budget = max(PREFILL_TOKENS, max_batch)
-    # requests whose prompt went in first decode while the others' prompts still go in (and take a growing share
-    # of every step's budget from them)
-    slack = 2 * -(-max_batch * args.context // budget) + 8
-    new_tokens = args.warmup + args.steps + slack
-    decode_len = args.context + new_tokens + 1
-    cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], PREFILL_TOKENS + 8, decode_len)
-    pages = max(max_batch * -(-decode_len // block_size), -(-(PREFILL_TOKENS + 8) // block_size)) + 16
+
+    def new_tokens_for(batch, context):
+        # requests whose prompt went in first decode while the others' prompts still go in (and take a growing share
+        # of every step's budget from them)
+        return args.warmup + args.steps + 2 * -(-batch * context // budget) + 8
+
+    runs = [(args.batch, args.context)] + [(b, args.context) for b in point_batches] + [(args.batch, c) for c in point_contexts]
+    longest = max(c + new_tokens_for(b, c) + 1 for b, c in runs)
+    cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], PREFILL_TOKENS + 8, longest)
+    pages = max([b * -(-(c + new_tokens_for(b, c) + 1) // block_size) for b, c in runs]
+                + [-(-(PREFILL_TOKENS + 8) // block_size)]) + 16
     engine_cfg = EngineConfig(dtype=args.dtype, block_size=block_size, num_blocks=pages, max_num_seqs=max_batch,
                               max_num_batched_tokens=budget, seed=0)
     runner = ModelRunner.from_random(cfg, seed=0, engine_config=engine_cfg)
@@ -362,11 +322,11 @@ def main() -> int:
         lo = min(100, vocab // 4)
         return [torch.randint(lo, vocab, (length,), generator=gen).tolist() for _ in range(n)]
 
-    def decode_rate(batch):
+    def decode_rate(batch, context=args.context):
         eng = ContinuousBatchingEngine(runner, sampler, max_num_seqs=batch,
                                        max_num_batched_tokens=engine_cfg.max_num_batched_tokens)
-        for p in prompts(batch, args.context):
-            eng.add_request(p, SamplingParams(max_new_tokens=new_tokens))
+        for p in prompts(batch, context):
+            eng.add_request(p, SamplingParams(max_new_tokens=new_tokens_for(batch, context)))
         while eng.waiting or any(r.num_tokens - r.num_computed_tokens > 1 for r in eng.running):
             eng.step()  # prompts in
         for _ in range(args.warmup):
@@ -398,6 +358,9 @@ def main() -> int:
     points = {}
     for b in point_batches:
         points[f"decode_b{b}"] = round(decode_rate(b)[0], 1)
+    for c in point_contexts:
+        points[f"decode_b{args.batch}_ctx{c}"] = round(decode_rate(args.batch, c)[0], 1)
+    served = serve_summary(torch, runner, sampler, vocab, budget, max_batch) if extra and not args.no_serve else {}
     pre_s = prefill_time() if args.phase != "decode" else float("inf")
     chunked_s = prefill_time(PREFILL_CHUNK) if args.phase == "all" else float("inf")
     peaks = measured_peaks(torch) if args.phase == "all" else {}
@@ -418,7 +381,7 @@ def main() -> int:
         return round(seconds * 1e3, 4) if seconds != float("inf") else 0.0
 
     line = {
-        "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (TinyLlama 1.1B)",
+        "metric": f"decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens ({MODEL_NAMES.get(args.model, args.model)})",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms(step_s), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
@@ -432,6 +395,8 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
+        "serve": served,
+        "peak_mib": round(torch.cuda.max_memory_allocated() / 2 ** 20, 1),
         "measured_peaks": peaks,
     }
     print(json.dumps(line))

@@ -226,7 +226,7 @@ __device__ __forceinline__ void attend_tile(f32x4 (&acc)[DB], float& m_run, floa
 // workgroup leaves for another inside a kernel goes this way, with a relaxed atomic access at agent scope, which
 // the compiler turns into a store that is written through and a load that does not hit a stale line.  No fence:
 // a release at agent scope writes a whole L2 back and costs more than the kernel (9 to 130 microseconds a
-// launch where this costs 1.5 to 3: llms_probe_handover in csrc/probe.hip measures both).
+// launch where this costs 1.5 to 3).
 __device__ __forceinline__ void store_across(float* p, float a, float b) {
     const unsigned long long v = ((unsigned long long)__float_as_uint(b) << 32) | __float_as_uint(a);
     __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
