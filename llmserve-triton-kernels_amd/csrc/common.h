@@ -74,6 +74,20 @@ __device__ __forceinline__ bf16 from_f32<bf16>(float v) {
 template <typename T>
 __device__ __forceinline__ float round_to(float v) { return to_f32(from_f32<T>(v)); }
 
+// Sine and cosine of position * frequency, and (a, b) turned by that angle.  Never inlined, and every product and
+// sum rounded on its own: inlined, the compiler schedules and contracts this arithmetic differently from kernel to
+// kernel, and a result that falls next to a rounding boundary of bfloat16 then differs between kernels that must
+// agree to the bit (the rotation kernel, and the products that rotate in their epilogue).
+// (Results come back by value: an address of a caller's variable would put it in private memory.)
+__device__ __noinline__ float2 rotary_angle(float position, float frequency) {  // (sine, cosine)
+    float sine, cosine;
+    sincosf(__fmul_rn(position, frequency), &sine, &cosine);
+    return make_float2(sine, cosine);
+}
+__device__ __noinline__ float2 rotate_pair(float a, float b, float cs, float sn) {
+    return make_float2(__fsub_rn(__fmul_rn(a, cs), __fmul_rn(b, sn)), __fadd_rn(__fmul_rn(b, cs), __fmul_rn(a, sn)));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = LLMS_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, LLMS_WAVE);

@@ -198,10 +198,10 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const float* __restrict__
         float a = to_f32(x[i]), b = to_f32(x[i + half]);
         float ra = a, rb = b;
         if (inv_freq) {
-            float sn, cs;
-            sincosf(pos * inv_freq[i], &sn, &cs);
-            ra = a * cs - b * sn;
-            rb = b * cs + a * sn;
+            const float2 angle = rotary_angle(pos, inv_freq[i]);
+            const float2 r = rotate_pair(a, b, angle.y, angle.x);
+            ra = r.x;
+            rb = r.y;
         }
         if (h < n_heads || k_pool == nullptr) {
             x[i] = from_f32<T>(ra);
@@ -279,7 +279,11 @@ __global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restri
     }
     if (inv_freq) {
         const float pos = (float)positions[n];
-        for (int i = tid; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &angles[i], &angles[half + i]);
+        for (int i = tid; i < half; i += blockDim.x) {
+            const float2 angle = rotary_angle(pos, inv_freq[i]);
+            angles[i] = angle.x;
+            angles[half + i] = angle.y;
+        }
     }
     __syncthreads();
     const bool in_run = run_found != 0;
@@ -321,8 +325,9 @@ __global__ __launch_bounds__(256) void rope_store_bf16_vec_kernel(bf16* __restri
                         for (int u = 0; u < 2; ++u) {
                             const float a = bf16_bits_to_f32((uint16_t)(u ? av[j] >> 16 : av[j] & 0xffffu));
                             const float b = bf16_bits_to_f32((uint16_t)(u ? bv[j] >> 16 : bv[j] & 0xffffu));
-                            lo_a[u] = a * cs[2 * j + u] - b * sn[2 * j + u];
-                            lo_b[u] = b * cs[2 * j + u] + a * sn[2 * j + u];
+                            const float2 r = rotate_pair(a, b, cs[2 * j + u], sn[2 * j + u]);
+                            lo_a[u] = r.x;
+                            lo_b[u] = r.y;
                         }
                         ra[j] = pack_bf16x2(lo_a[0], lo_a[1]);
                         rb[j] = pack_bf16x2(lo_b[0], lo_b[1]);

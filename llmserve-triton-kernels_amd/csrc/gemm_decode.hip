@@ -122,6 +122,96 @@ __device__ __forceinline__ int gd_weight_row(const DecodeGemmArgs& a, int u0, in
     return (a.n_heads + a.n_kv_heads) * D + (u - rot_units) + (hi ? a.n_kv_heads * half : 0);
 }
 
+// What a thread needs from memory to finish one place (a unit or row of the weight, a row of X): asked for early,
+// whether the place exists or not (from nowhere if it does not), used after the waves' sums have met.
+struct GdFinish {
+    int pos, slot;
+    float freq;
+    unsigned res;
+};
+
+struct GdFinishBuffers {
+    __amdgpu_buffer_rsrc_t pos, slot, freq, res;
+};
+
+__device__ __forceinline__ GdFinishBuffers gd_finish_buffers(const DecodeGemmArgs& a) {
+    GdFinishBuffers b;
+    b.pos = gd_buffer(a.positions, a.positions ? (unsigned)a.M * 4 : 0u);
+    b.slot = gd_buffer(a.slots, a.slots ? (unsigned)a.M * 4 : 0u);
+    b.freq = gd_buffer(a.inv_freq, a.inv_freq ? (unsigned)a.head_dim * 2 : 0u);
+    b.res = gd_buffer(a.residual, a.residual ? (unsigned)(((size_t)(a.M - 1) * a.ldr + a.N) * 2) : 0u);
+    return b;
+}
+
+// `u`: the unit (pairs) or weight row (plain, residual) of the place, `m` its row of X; `live`: the place exists.
+template <int EPI>
+__device__ __forceinline__ void gd_ask(const DecodeGemmArgs& a, const GdFinishBuffers& b, bool live, int m, int u, GdFinish& f) {
+    if (EPI == GD_ROPE_QKV) {
+        const int half = a.head_dim / 2;
+        f.slot = (int)__builtin_amdgcn_raw_buffer_load_b32(b.slot, live ? (unsigned)m * 4 : GD_NOWHERE, 0, 0);
+        if (!a.slots) f.slot = -1;
+        const bool rot = live && u < (a.n_heads + a.n_kv_heads) * half;
+        f.pos = (int)__builtin_amdgcn_raw_buffer_load_b32(b.pos, rot ? (unsigned)m * 4 : GD_NOWHERE, 0, 0);
+        f.freq = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(b.freq, rot ? (unsigned)(u % half) * 4 : GD_NOWHERE, 0, 0));
+    }
+    if (EPI == GD_RESIDUAL)
+        f.res = __builtin_amdgcn_raw_buffer_load_b16(b.res, live ? (unsigned)(m * a.ldr + u) * 2 : GD_NOWHERE, 0, 0);
+}
+
+// PLAIN, RESIDUAL: the sum `s` of weight row n and row m of X.
+template <typename TOut, int EPI>
+__device__ __forceinline__ void gd_finish_row(const DecodeGemmArgs& a, int m, int n, float s, const GdFinish& f) {
+    if (a.bias) s += bf16_bits_to_f32(a.bias[n].bits);
+    if (EPI == GD_PLAIN)
+        gd_store<TOut>(reinterpret_cast<TOut*>(a.C) + (size_t)m * a.ldc + n, s);
+    else
+        a.residual[(size_t)m * a.ldr + n].bits = f32_to_bf16_bits(bf16_bits_to_f32((uint16_t)f.res) + gd_bfr(s));
+}
+
+// SWIGLU, ROPE_QKV: the sums `lo` and `hi` of unit u's two weight rows and row m of X.
+template <typename TOut, int EPI>
+__device__ __forceinline__ void gd_finish_pair(const DecodeGemmArgs& a, int m, int u, float lo, float hi, const GdFinish& f) {
+    if (EPI == GD_SWIGLU) {
+        const float gate = gd_bfr(lo), up = gd_bfr(hi);
+        gd_store<TOut>(reinterpret_cast<TOut*>(a.C) + (size_t)m * a.ldc + u, gd_bfr(gate / (1.f + expf(-gate))) * up);
+        return;
+    }
+    const int nh = a.n_heads, nkv = a.n_kv_heads, D = a.head_dim, half = D / 2, bs = a.block_size;
+    const int rot_units = (nh + nkv) * half;
+    if (a.bias) {
+        lo += bf16_bits_to_f32(a.bias[gd_weight_row<EPI>(a, u, u + 1, 8, 0)].bits);
+        hi += bf16_bits_to_f32(a.bias[gd_weight_row<EPI>(a, u, u + 1, 8, 8)].bits);
+    }
+    lo = gd_bfr(lo);  // the projection's result is bfloat16 before it is rotated
+    hi = gd_bfr(hi);
+    const int slot = f.slot;
+    if (u < rot_units) {
+        const int h = u / half, d = u - h * half;
+        float ra = lo, rb = hi;
+        if (a.inv_freq) {
+            const float2 angle = rotary_angle((float)f.pos, f.freq);
+            const float2 r = rotate_pair(lo, hi, angle.y, angle.x);
+            ra = r.x;
+            rb = r.y;
+        }
+        if (h < nh) {
+            TOut* q = reinterpret_cast<TOut*>(a.C) + (size_t)m * a.ldc + h * D + d;
+            gd_store<TOut>(q, ra);
+            gd_store<TOut>(q + half, rb);
+        } else if (slot >= 0) {
+            const int page = slot / bs, off = slot % bs;
+            bf16* dst = a.k_pool + (((size_t)page * nkv + (h - nh)) * bs + off) * D;
+            dst[d].bits = f32_to_bf16_bits(ra);
+            dst[d + half].bits = f32_to_bf16_bits(rb);
+        }
+    } else if (slot >= 0) {
+        const int page = slot / bs, off = slot % bs;
+        const int f_lo = u - rot_units, f_hi = f_lo + nkv * half;  // features among the value heads
+        a.v_pool[(((size_t)page * nkv + f_lo / D) * D + f_lo % D) * bs + off].bits = f32_to_bf16_bits(lo);
+        a.v_pool[(((size_t)page * nkv + f_hi / D) * D + f_hi % D) * bs + off].bits = f32_to_bf16_bits(hi);
+    }
+}
+
 // XC: chunks of K a wave holds (ceil(K / 128 / 16)); LPI: load instructions per item, each 4 rows of 256 bytes (a
 // tile is 4 LPI rows); NT: tiles of a group, whose partial sums meet in LDS together (the items of a group,
 // NT * XC, are unrolled).
@@ -173,47 +263,24 @@ __global__ __launch_bounds__(GD_NW* LLMS_WAVE) void gemm_decode_kernel(const Dec
         __builtin_amdgcn_s_barrier();
     }
 
-    // ---- what a thread needs from memory to finish its places of a group of tiles (asked for whether the place
-    // exists or not, from nowhere if it does not)
-    struct Finish {
-        int pos, slot;
-        float freq;
-        unsigned res;
-    };
-    const __amdgpu_buffer_rsrc_t pos_buf = gd_buffer(a.positions, a.positions ? (unsigned)M * 4 : 0u);
-    const __amdgpu_buffer_rsrc_t slot_buf = gd_buffer(a.slots, a.slots ? (unsigned)M * 4 : 0u);
-    const __amdgpu_buffer_rsrc_t freq_buf = gd_buffer(a.inv_freq, a.inv_freq ? (unsigned)a.head_dim * 2 : 0u);
-    const __amdgpu_buffer_rsrc_t res_buf =
-        gd_buffer(a.residual, a.residual ? (unsigned)(((size_t)(M - 1) * a.ldr + a.N) * 2) : 0u);
+    // ---- what a thread needs from memory to finish its places of a group of tiles
+    const GdFinishBuffers fin_bufs = gd_finish_buffers(a);
     auto place_of = [&](int e, int& te, int& idx) {  // round e of this thread: tile of the group, place in the tile
         const int p = e * THREADS + tid;
         te = p / PLACES;
         idx = p % PLACES;
     };
-    auto ask_finish = [&](int tile0, Finish(&f)[EPI_ROUNDS]) {
+    auto ask_finish = [&](int tile0, GdFinish(&f)[EPI_ROUNDS]) {
 #pragma unroll
         for (int e = 0; e < EPI_ROUNDS; ++e) {
             int te, idx;
             place_of(e, te, idx);
-            const int eu0 = u_begin + (tile0 + te) * UPT;
-            if (EPI == GD_ROPE_QKV) {
-                const int m = idx / 8, u = eu0 + idx % 8, half = a.head_dim / 2;
-                const bool live = te < NT && m < M && u < u_last;
-                f[e].slot = (int)__builtin_amdgcn_raw_buffer_load_b32(slot_buf, live ? (unsigned)m * 4 : GD_NOWHERE, 0, 0);
-                if (!a.slots) f[e].slot = -1;
-                const bool rot = live && u < (a.n_heads + a.n_kv_heads) * half;
-                f[e].pos = (int)__builtin_amdgcn_raw_buffer_load_b32(pos_buf, rot ? (unsigned)m * 4 : GD_NOWHERE, 0, 0);
-                f[e].freq = __uint_as_float(
-                    __builtin_amdgcn_raw_buffer_load_b32(freq_buf, rot ? (unsigned)(u % half) * 4 : GD_NOWHERE, 0, 0));
-            }
-            if (EPI == GD_RESIDUAL) {
-                const int m = idx / UPT, n = eu0 + idx % UPT;
-                const bool live = te < NT && m < M && n < u_last;
-                f[e].res = __builtin_amdgcn_raw_buffer_load_b16(res_buf, live ? (unsigned)(m * a.ldr + n) * 2 : GD_NOWHERE, 0, 0);
-            }
+            const int per = PAIRS ? 8 : UPT;
+            const int m = idx / per, u = u_begin + (tile0 + te) * UPT + idx % per;
+            gd_ask<EPI>(a, fin_bufs, te < NT && m < M && u < u_last, m, u, f[e]);
         }
     };
-    Finish fin[EPI_ROUNDS];
+    GdFinish fin[EPI_ROUNDS];
     ask_finish(0, fin);
 
     // ---- then the stream of weights
@@ -349,60 +416,10 @@ __global__ __launch_bounds__(GD_NW* LLMS_WAVE) void gemm_decode_kernel(const Dec
             };
             if (!PAIRS) {
                 const int i = idx % UPT, m = idx / UPT, n = eu0 + i;
-                if (m < M && n < u_last) {
-                    float s = total_of(i, m);
-                    if (a.bias) s += bf16_bits_to_f32(a.bias[n].bits);
-                    if (EPI == GD_PLAIN)
-                        gd_store<TOut>(reinterpret_cast<TOut*>(a.C) + (size_t)m * a.ldc + n, s);
-                    else
-                        a.residual[(size_t)m * a.ldr + n].bits =
-                            f32_to_bf16_bits(bf16_bits_to_f32((uint16_t)fin[e].res) + gd_bfr(s));
-                }
+                if (m < M && n < u_last) gd_finish_row<TOut, EPI>(a, m, n, total_of(i, m), fin[e]);
             } else {
                 const int j = idx % 8, m = idx / 8, u = eu0 + j;
-                if (m < M && u < u_last) {
-                    float lo = total_of(j, m), hi = total_of(j + 8, m);
-                    if (EPI == GD_SWIGLU) {
-                        const float gate = gd_bfr(lo), up = gd_bfr(hi);
-                        gd_store<TOut>(reinterpret_cast<TOut*>(a.C) + (size_t)m * a.ldc + u,
-                                       gd_bfr(gate / (1.f + expf(-gate))) * up);
-                    } else {
-                        const int nh = a.n_heads, nkv = a.n_kv_heads, D = a.head_dim, half = D / 2, bs = a.block_size;
-                        const int rot_units = (nh + nkv) * half;
-                        if (a.bias) {
-                            lo += bf16_bits_to_f32(a.bias[gd_weight_row<EPI>(a, eu0, u_last, UPT, j)].bits);
-                            hi += bf16_bits_to_f32(a.bias[gd_weight_row<EPI>(a, eu0, u_last, UPT, j + 8)].bits);
-                        }
-                        lo = gd_bfr(lo);  // the projection's result is bfloat16 before it is rotated
-                        hi = gd_bfr(hi);
-                        const int slot = fin[e].slot;
-                        if (u < rot_units) {
-                            const int h = u / half, d = u - h * half;
-                            float ra = lo, rb = hi;
-                            if (a.inv_freq) {
-                                float sn, cs;
-                                sincosf((float)fin[e].pos * fin[e].freq, &sn, &cs);
-                                ra = lo * cs - hi * sn;
-                                rb = hi * cs + lo * sn;
-                            }
-                            if (h < nh) {
-                                TOut* q = reinterpret_cast<TOut*>(a.C) + (size_t)m * a.ldc + h * D + d;
-                                gd_store<TOut>(q, ra);
-                                gd_store<TOut>(q + half, rb);
-                            } else if (slot >= 0) {
-                                const int page = slot / bs, off = slot % bs;
-                                bf16* dst = a.k_pool + (((size_t)page * nkv + (h - nh)) * bs + off) * D;
-                                dst[d].bits = f32_to_bf16_bits(ra);
-                                dst[d + half].bits = f32_to_bf16_bits(rb);
-                            }
-                        } else if (slot >= 0) {
-                            const int page = slot / bs, off = slot % bs;
-                            const int f_lo = u - rot_units, f_hi = f_lo + nkv * half;  // features among the value heads
-                            a.v_pool[(((size_t)page * nkv + f_lo / D) * D + f_lo % D) * bs + off].bits = f32_to_bf16_bits(lo);
-                            a.v_pool[(((size_t)page * nkv + f_hi / D) * D + f_hi % D) * bs + off].bits = f32_to_bf16_bits(hi);
-                        }
-                    }
-                }
+                if (m < M && u < u_last) gd_finish_pair<TOut, EPI>(a, m, u, total_of(j, m), total_of(j + 8, m), fin[e]);
             }
         }
     };
@@ -417,6 +434,255 @@ __global__ __launch_bounds__(GD_NW* LLMS_WAVE) void gemm_decode_kernel(const Dec
     }
     run_group(tile0, false);
     finish_group(tile0);
+}
+
+// 17 to 64 rows of X (RB blocks of 16): the same sharing out of weight rows and of K, with 8 waves that have
+// twice the registers.  A wave keeps its chunks of all rows of X in registers, loaded straight in the operand
+// layout (64 rows are full load instructions there), and every chunk of weights it stages meets RB blocks of rows:
+// RB matrix instructions per fragment read from LDS.  X enters a compute unit once, as much as the unit's share of
+// a large weight; with one workgroup per block of 16 rows it would enter four times as many workgroups.
+#define GR_NW 8
+
+template <typename TOut, int EPI, int XC, int RB, int NT, bool NORM>
+__global__ __launch_bounds__(GR_NW* LLMS_WAVE) void gemm_decode_rows_kernel(const DecodeGemmArgs a) {
+    static_assert(!NORM || RB <= 2, "the norm's registers fit beside up to 32 rows of X");
+    constexpr int NW = GR_NW, LPI = 4;
+    constexpr bool PAIRS = EPI == GD_SWIGLU || EPI == GD_ROPE_QKV;
+    constexpr int UPT = PAIRS ? 8 : 16;  // units per tile
+    constexpr int ITEMS = NT * XC;
+    constexpr int RING = ITEMS % 2 == 0 ? 2 : (ITEMS < 3 ? ITEMS : 3);  // (1, 2, 3, 4, 6 items: 1, 2, 3, 2, 2)
+    static_assert(ITEMS % RING == 0, "the ring must go round a whole number of times per group");
+    constexpr int THREADS = NW * LLMS_WAVE;
+    constexpr int PLACES = UPT * RB * 16;  // (unit or row, row of X) pairs of a tile: one thread each
+    constexpr int EPI_ROUNDS = (NT * PLACES + THREADS - 1) / THREADS;
+    __shared__ u32x4 lds[NW * 16 * (GD_KC / 8)];         // per wave 16 rows x 16 pieces of 16 bytes
+    __shared__ __attribute__((aligned(16))) float red[NT * NW * RB * LLMS_WAVE * 4];  // [tile of the group][wave][block of rows][lane][4]
+    float* sq_lds = red;  // the norm's sums of squares, [row][wave], before the first sums of the product
+    const int tid = threadIdx.x, wave = tid / LLMS_WAVE, lane = tid % LLMS_WAVE;
+    const int r16 = lane % 16, g = lane / 16;
+    const int M = a.M, K = a.K, n_chunks = (K + GD_KC - 1) / GD_KC;
+    const int wg = blockIdx.x;
+    const int u_begin = wg * a.units_each + min(wg, a.units_more);
+    const int u_last = u_begin + a.units_each + (wg < a.units_more ? 1 : 0);
+
+    // ---- this wave's chunks of all rows of X, asked for as whole 256-byte pieces of 4 rows per instruction (every
+    // compute unit reads the same rows from L2 at this moment: half as many requests as 64-byte pieces would be);
+    // they reach the operand layout (lane (r16, g): X[16 rb + r16][c*128 + 32 s + 8 g ..+7]) through the wave's
+    // LDS tile further down
+    u32x4 xr[XC][RB][4];
+    const __amdgpu_buffer_rsrc_t x_buf = gd_buffer(a.X, (unsigned)(((size_t)(M - 1) * a.ldx + K) * 2));
+#pragma unroll
+    for (int j = 0; j < XC; ++j)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = 16 * rb + 4 * i + lane / 16, k = (wave + NW * j) * GD_KC + 8 * (lane % 16);
+                xr[j][rb][i] = gd_load(x_buf, row < M && k < K ? (unsigned)(row * a.ldx + k) * 2 : GD_NOWHERE);
+            }
+    u32x4 nwf[NORM ? XC : 1];
+    if (NORM) {
+        const __amdgpu_buffer_rsrc_t nw_buf = gd_buffer(a.norm_weight, (unsigned)K * 2);
+#pragma unroll
+        for (int j = 0; j < XC; ++j) nwf[j] = gd_load(nw_buf, (unsigned)((wave + NW * j) * GD_KC + 8 * (lane % 16)) * 2);
+        __builtin_amdgcn_s_barrier();  // (no wave asks for weights before every wave has asked for its rows)
+    }
+
+    const GdFinishBuffers fin_bufs = gd_finish_buffers(a);
+    auto place_of = [&](int e, int& te, int& idx) {
+        const int p = e * THREADS + tid;
+        te = p / PLACES;
+        idx = p % PLACES;
+    };
+    auto ask_finish = [&](int tile0, GdFinish(&f)[EPI_ROUNDS]) {
+#pragma unroll
+        for (int e = 0; e < EPI_ROUNDS; ++e) {
+            int te, idx;
+            place_of(e, te, idx);
+            const int m = idx / UPT, u = u_begin + (tile0 + te) * UPT + idx % UPT;
+            gd_ask<EPI>(a, fin_bufs, te < NT && m < M && u < u_last, m, u, f[e]);
+        }
+    };
+    GdFinish fin[EPI_ROUNDS];
+    ask_finish(0, fin);
+
+    u32x4 ring[RING][LPI];
+    const __amdgpu_buffer_rsrc_t w_buf = gd_buffer(a.W, (unsigned)((size_t)a.N * K * 2));
+    auto issue = [&](u32x4(&w)[LPI], int tile0, int q) {
+        const int c = wave + NW * (q % XC), kl = c * GD_KC + 8 * (lane % 16);
+        const int u0 = u_begin + (tile0 + q / XC) * UPT;
+#pragma unroll
+        for (int i = 0; i < LPI; ++i) {
+            const int n = gd_weight_row<EPI>(a, u0, u_last, UPT, i * 4 + lane / 16);
+            w[i] = gd_load_streaming(w_buf, n >= 0 && kl < K ? (unsigned)(n * K + kl) * 2 : GD_NOWHERE);
+        }
+    };
+#pragma unroll
+    for (int q = 0; q < RING; ++q) issue(ring[q], 0, q);
+
+    // ---- the norm of the rows, if asked: as in the kernel above (there the rows go to LDS afterwards, here they
+    // stay in registers), under the cover of the weights in flight
+    if (NORM) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float ss = 0.f;
+#pragma unroll
+                for (int j = 0; j < XC; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ss = gd_dot2(xr[j][rb][i][e], xr[j][rb][i][e], ss);
+                ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x111, 0xf, 0xf, true));
+                ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x112, 0xf, 0xf, true));
+                ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x114, 0xf, 0xf, true));
+                ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x118, 0xf, 0xf, true));
+                if (r16 == 15) sq_lds[(16 * rb + 4 * i + g) * NW + wave] = ss;
+            }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // (LDS writes done; the weights stay in flight across the barrier)
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float total = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; w += 4) {
+                    const f32x4 part = *reinterpret_cast<const f32x4*>(sq_lds + (16 * rb + 4 * i + g) * NW + w);
+                    total += part[0];
+                    total += part[1];
+                    total += part[2];
+                    total += part[3];
+                }
+                const float inv = rsqrtf(total / (float)K + a.eps);
+#pragma unroll
+                for (int j = 0; j < XC; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t xv = xr[j][rb][i][e], wv = nwf[j][e];
+                        const uint32_t y = pack_bf16x2(__uint_as_float(xv << 16) * inv, __uint_as_float(xv & 0xffff0000u) * inv);
+                        xr[j][rb][i][e] = pack_bf16x2(gd_dot2(y, wv & 0xffffu, 0.f), gd_dot2(y, wv & 0xffff0000u, 0.f));
+                    }
+            }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();  // (every wave has read the sums of squares before the product's sums go there)
+    }
+
+    u32x4* tile = lds + wave * 16 * (GD_KC / 8);
+#pragma unroll
+    for (int j = 0; j < XC; ++j)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = i * 4 + lane / 16;
+                tile[row * 16 + ((lane % 16) ^ row)] = xr[j][rb][i];
+            }
+#pragma unroll
+            for (int s_ = 0; s_ < 4; ++s_) xr[j][rb][s_] = tile[r16 * 16 + ((4 * s_ + g) ^ r16)];
+        }
+    auto run_group = [&](int tile0, const bool more) {
+        f32x4 acc[RB];  // (of the tile under way: its sums go to LDS when its last chunk is in)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) acc[rb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < ITEMS; ++q) {
+            const bool live = wave + NW * (q % XC) < n_chunks;  // (a chunk beyond K: its loads brought zeros)
+            if (live) {
+#pragma unroll
+                for (int i = 0; i < LPI; ++i) {
+                    const int row = i * 4 + lane / 16;
+                    tile[row * 16 + ((lane % 16) ^ row)] = ring[q % RING][i];
+                }
+            }
+            if (q + RING < ITEMS) issue(ring[q % RING], tile0, q + RING);  // the registers are free again
+            else if (more) issue(ring[q % RING], tile0 + NT, q + RING - ITEMS);
+            if (live) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const u32x4 av = tile[r16 * 16 + ((4 * s + g) ^ r16)];
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb)
+                        acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gd_as_bf16x8(av), gd_as_bf16x8(xr[q % XC][rb][s]), acc[rb], 0, 0, 0);
+                }
+            }
+            if (q % XC == XC - 1) {
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    *reinterpret_cast<f32x4*>(red + ((((q / XC) * NW + wave) * RB + rb) * LLMS_WAVE + lane) * 4) = acc[rb];
+                    acc[rb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                }
+            }
+        }
+    };
+    auto finish_group = [&](int tile0) {
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < EPI_ROUNDS; ++e) {
+            int te, idx;
+            place_of(e, te, idx);
+            if (te >= NT) continue;
+            const int i = idx % UPT, m = idx / UPT, u = u_begin + (tile0 + te) * UPT + i;
+            // sum of the waves for row i (0..15) of the tile and row m of X, wave 0 first
+            auto total_of = [&](int row) -> float {
+                const int src_lane = (row / 4) * 16 + m % 16, r = row % 4;
+                float sum = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) sum += red[(((te * NW + w) * RB + m / 16) * LLMS_WAVE + src_lane) * 4 + r];
+                return sum;
+            };
+            if (m >= M || u >= u_last) continue;
+            if (!PAIRS) gd_finish_row<TOut, EPI>(a, m, u, total_of(i), fin[e]);
+            else gd_finish_pair<TOut, EPI>(a, m, u, total_of(i), total_of(i + 8), fin[e]);
+        }
+    };
+    int tile0 = 0;
+    for (int gr = 0; gr + 1 < a.groups; ++gr, tile0 += NT) {
+        run_group(tile0, true);
+        finish_group(tile0);
+        ask_finish(tile0 + NT, fin);
+        __syncthreads();  // the sums are read before the next tiles overwrite them
+    }
+    run_group(tile0, false);
+    finish_group(tile0);
+}
+
+// 17 to 64 rows: K up to 2,048 (a wave's two chunks of 64 rows are 128 registers).
+#define GR_GO(XC, RB, NT)                                                                                  \
+    do {                                                                                                   \
+        a.groups = (tiles + NT - 1) / NT;                                                                  \
+        gemm_decode_rows_kernel<TOut, EPI, XC, RB, NT, NORM><<<grid, GR_NW * LLMS_WAVE, 0, stream>>>(a);   \
+    } while (0)
+
+template <typename TOut, int EPI, int RB, bool NORM>
+static void gd_launch_rows_one_chunk(int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
+    const int groups = (tiles + 3) / 4, nt = (tiles + groups - 1) / groups;
+    if (nt == 1) GR_GO(1, RB, 1);
+    else if (nt == 2) GR_GO(1, RB, 2);
+    else if (nt == 3) GR_GO(1, RB, 3);
+    else GR_GO(1, RB, 4);
+}
+
+template <typename TOut, int EPI, int RB, bool NORM>
+static void gd_launch_rows_two_chunks(int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
+    if (tiles == 1) GR_GO(2, RB, 1);
+    else if (tiles % 3 == 0 || tiles > 4) GR_GO(2, RB, 3);
+    else GR_GO(2, RB, 2);
+}
+#undef GR_GO
+
+template <typename TOut, int EPI>
+static int gd_launch_rows(int chunks, int rows, int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
+    if (a.norm_weight) {  // (up to 32 rows: checked by the caller)
+        if (chunks <= GR_NW) gd_launch_rows_one_chunk<TOut, EPI, 2, true>(tiles, grid, a, stream);
+        else gd_launch_rows_two_chunks<TOut, EPI, 2, true>(tiles, grid, a, stream);
+    } else if (chunks <= GR_NW) {
+        if (rows <= 32) gd_launch_rows_one_chunk<TOut, EPI, 2, false>(tiles, grid, a, stream);
+        else gd_launch_rows_one_chunk<TOut, EPI, 4, false>(tiles, grid, a, stream);
+    } else {
+        if (rows <= 32) gd_launch_rows_two_chunks<TOut, EPI, 2, false>(tiles, grid, a, stream);
+        else gd_launch_rows_two_chunks<TOut, EPI, 4, false>(tiles, grid, a, stream);
+    }
+    return LLMS_OK;
 }
 
 // `tiles`: tiles of the workgroup with the most units; `lds_bytes`: what the kernel needs of LDS.
@@ -452,9 +718,11 @@ static int gd_launch(int chunks, int tiles, unsigned grid, unsigned lds_bytes, D
 
 extern "C" {
 
-// Whether M rows of K elements fit: the rows of X (8 of them up to 8 rows, else 16) stay in LDS beside the tiles.
+// Whether M rows of K elements fit: up to 16 rows stay in LDS beside the tiles (8 of them up to 8 rows, else 16);
+// 17 to 64 rows in the registers of 8 waves, two chunks of 128 each.
 int llms_gemm_decode_fits(int M, int K) {
-    if (M <= 0 || M > 16 || K <= 0 || K > GD_MAX_K) return 0;
+    if (M <= 0 || M > 64 || K <= 0 || K > GD_MAX_K) return 0;
+    if (M > 16) return K <= 2 * GR_NW * GD_KC;
     return (M <= 8 ? 8 : 16) * ((K + GD_KC - 1) / GD_KC * (GD_KC * 2) + 16) <= GD_LDS_X_MAX;
 }
 
@@ -468,12 +736,12 @@ int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* 
                      int n_heads, int n_kv_heads, int head_dim, int block_size, const float* inv_freq,
                      const int* positions, const int* slots, void* k_pool, void* v_pool, void* residual, int ldr,
                      int workgroups, hipStream_t stream) {
-    LLMS_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_decode: needs 1 <= M <= 16 and positive sizes");
+    LLMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_decode: needs 1 <= M <= 64 and positive sizes");
     LLMS_REQUIRE((long long)N * K < (1ll << 30) && (long long)M * ldx < (1ll << 30), "gemm_decode: operands of 2 GB or more");
     const int x_rows = M <= 8 ? 8 : 16, x_pitch = (K + GD_KC - 1) / GD_KC * (GD_KC * 2) + 16;
-    LLMS_REQUIRE(K <= GD_MAX_K && x_rows * x_pitch <= GD_LDS_X_MAX,
-                 "gemm_decode: the rows of X do not fit a compute unit's LDS (see llms_gemm_decode_fits)");
+    LLMS_REQUIRE(llms_gemm_decode_fits(M, K), "gemm_decode: the rows of X do not fit a compute unit (see llms_gemm_decode_fits)");
     LLMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "gemm_decode: K and the row stride of X must be multiples of 8");
+    LLMS_REQUIRE(M <= 32 || norm_weight == nullptr, "gemm_decode: more than 32 rows are taken as they are (no norm on the way in)");
     LLMS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)norm_weight % 16) == 0,
                  "gemm_decode: X, W and the norm's weight must be 16-byte aligned");
     LLMS_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm_decode: epilogue must be 0..3");
@@ -508,7 +776,14 @@ int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* 
     const int chunks = (K + GD_KC - 1) / GD_KC;
     const unsigned lds = GD_LDS_TILES + GD_LDS_SQ + (unsigned)(x_rows * x_pitch);
     int rc;
-    if (epilogue == GD_SWIGLU) rc = gd_launch<bf16, GD_SWIGLU, 4>(chunks, (most + 7) / 8, grid, lds, a, stream);
+    if (M > 16) {  // tiles of 16 rows (8 units with partners), 8 waves
+        const int tiles = epilogue == GD_SWIGLU || epilogue == GD_ROPE_QKV ? (most + 7) / 8 : (most + 15) / 16;
+        if (epilogue == GD_SWIGLU) rc = gd_launch_rows<bf16, GD_SWIGLU>(chunks, M, tiles, grid, a, stream);
+        else if (epilogue == GD_ROPE_QKV) rc = gd_launch_rows<bf16, GD_ROPE_QKV>(chunks, M, tiles, grid, a, stream);
+        else if (epilogue == GD_RESIDUAL) rc = gd_launch_rows<bf16, GD_RESIDUAL>(chunks, M, tiles, grid, a, stream);
+        else if (out_dtype == 0) rc = gd_launch_rows<float, GD_PLAIN>(chunks, M, tiles, grid, a, stream);
+        else rc = gd_launch_rows<bf16, GD_PLAIN>(chunks, M, tiles, grid, a, stream);
+    } else if (epilogue == GD_SWIGLU) rc = gd_launch<bf16, GD_SWIGLU, 4>(chunks, (most + 7) / 8, grid, lds, a, stream);
     else if (epilogue == GD_ROPE_QKV) rc = gd_launch<bf16, GD_ROPE_QKV, 4>(chunks, (most + 7) / 8, grid, lds, a, stream);
     else {
         // tiles of 8 rows where the last tile of 16 would be half empty (a share of up to 8 rows, of 17 to 24, ...):

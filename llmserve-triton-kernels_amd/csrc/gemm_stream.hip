@@ -233,10 +233,10 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void gemm_stream_kernel(const Stream
                 hi = bfr(hi);
                 float ra = lo, rb = hi;
                 if (a.inv_freq) {
-                    float sn, cs;
-                    sincosf((float)epi_pos * epi_freq, &sn, &cs);
-                    ra = lo * cs - hi * sn;
-                    rb = hi * cs + lo * sn;
+                    const float2 angle = rotary_angle((float)epi_pos, epi_freq);
+                    const float2 r = rotate_pair(lo, hi, angle.y, angle.x);
+                    ra = r.x;
+                    rb = r.y;
                 }
                 if (h < nh) {
                     store_out<TOut>(C + (size_t)m * a.ldc + h * D + d, ra);

@@ -388,15 +388,19 @@ def compute_units(dev: torch.device) -> int:
     return _cu_count[index]
 
 
-GEMM_DECODE_MAX_ROWS = 16
+GEMM_DECODE_MAX_ROWS = 64
+GEMM_DECODE_NORM_ROWS = 32  # up to here the kernel can norm its rows on the way in (beyond, their registers are full)
 GEMM_DECODE_MAX_K = 16 * 3 * 128  # 16 waves with up to three chunks of 128 each
 _GEMM_DECODE_LDS_FOR_ROWS = 160 * 1024 - 16 * 4096 - 1024  # what the waves' tiles leave of a compute unit's LDS
 
 
 def gemm_decode_fits(m: int, k: int) -> bool:
-    """Whether m rows of k elements fit ops.gemm_decode: the rows (8 of them up to 8 rows, else 16) stay in LDS."""
+    """Whether m rows of k elements fit ops.gemm_decode: up to 16 rows stay in LDS (8 of them up to 8 rows, else
+    16); 17 to 64 rows in the registers of 8 waves, two chunks of 128 each (k up to 2,048)."""
     if not (0 < m <= GEMM_DECODE_MAX_ROWS and 0 < k <= GEMM_DECODE_MAX_K):
         return False
+    if m > 16:
+        return k <= 2 * 8 * 128
     return (8 if m <= 8 else 16) * (-(-k // 128) * 256 + 16) <= _GEMM_DECODE_LDS_FOR_ROWS
 
 
@@ -408,9 +412,9 @@ def gemm_decode_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
 def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, *,
                 norm: tuple[torch.Tensor, float] | None = None, swiglu: bool = False, rope: dict | None = None,
                 residual: torch.Tensor | None = None) -> torch.Tensor:
-    """The product for up to 16 bfloat16 rows with one workgroup per compute unit, and what surrounds it fused in.
+    """The product for up to 64 bfloat16 rows with one workgroup per compute unit, and what surrounds it fused in.
 
-    norm = (weight [K], eps): the rows of x are replaced by RMSNorm(x) * weight on the way in.
+    norm = (weight [K], eps): the rows of x are replaced by RMSNorm(x) * weight on the way in (up to 32 rows).
     plain:     out[M, N] = x w^T (+ bias), bfloat16 or float32.
     swiglu:    w = [gate; up] ([2I, K]); out[M, I] = silu(gate) * up.
     rope = dict(n_heads, n_kv_heads, head_dim, inv_freq | None, positions, slots | None, k_pool, v_pool,
@@ -427,8 +431,8 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
     if not 0 < m <= GEMM_DECODE_MAX_ROWS:
         raise ValueError(f"gemm_decode takes 1..{GEMM_DECODE_MAX_ROWS} rows")
     if not gemm_decode_fits(m, k):
-        raise ValueError(f"gemm_decode keeps the rows of x in LDS: {m} rows of K = {k} do not fit (K up to "
-                         f"{GEMM_DECODE_MAX_K}, and up to 2,944 with more than 8 rows)")
+        raise ValueError(f"gemm_decode keeps the rows of x in a compute unit: {m} rows of K = {k} do not fit (K up to "
+                         f"{GEMM_DECODE_MAX_K} with up to 8 rows, 2,944 with up to 16, 2,048 beyond)")
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ValueError("gemm_decode takes bfloat16 operands")
     if not gemm_bf16_supported(x, w):
@@ -441,6 +445,8 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
     norm_weight, eps = None, 0.0
     if norm is not None:
         norm_weight, eps = norm
+        if m > GEMM_DECODE_NORM_ROWS:
+            raise ValueError(f"gemm_decode norms up to {GEMM_DECODE_NORM_ROWS} rows on the way in; {m} rows are taken as they are")
         if norm_weight.dtype != torch.bfloat16 or norm_weight.numel() != k or not norm_weight.is_contiguous() \
                 or norm_weight.data_ptr() % 16:
             raise ValueError("the norm's weight must be a contiguous, 16-byte aligned bfloat16 vector of K elements")

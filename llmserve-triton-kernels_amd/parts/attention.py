@@ -16,7 +16,7 @@ import math
 import torch
 
 from ..ops import library as ops
-from .linear import decode_product, few_rows, linear, linear_partial_sums
+from .linear import adds_residual_in_epilogue, decode_product, few_rows, linear, linear_partial_sums
 from .registry import ADDED_IN_PLACE, POSITION_ENCODINGS, DeferredNorm, Mixer, register_mixer
 from .spec import PagedCacheSpec, ParamInfo
 
@@ -86,7 +86,7 @@ class Attention(Mixer):
                                    cache.block_size)
         out = torch.empty((q.shape[0], nh * d), dtype=q.dtype, device=q.device)
         self.attend(out, q, cache, view, batch)
-        if deferred is not None and deferred.may_add_in_place and decode_product(out, self.o_weight):
+        if deferred is not None and deferred.may_add_in_place and adds_residual_in_epilogue(out, self.o_weight):
             ops.gemm_decode(None, out, self.o_weight, residual=deferred.residual)  # the residual sum in the epilogue
             return ADDED_IN_PLACE
         return (linear_partial_sums(out, self.o_weight) if deferred is not None else None) or linear(out, self.o_weight)
@@ -109,7 +109,7 @@ class Attention(Mixer):
         if frequencies is None and not getattr(self.position, "identity", False):
             return None  # a position encoding this kernel does not know
         decode = decode_product(rows, self.qkv_weight)
-        norm = x.fused() if deferred and decode else None
+        norm = x.fused() if deferred and decode and m <= ops.GEMM_DECODE_NORM_ROWS else None
         if norm is not None:
             x.resolve(None)  # nothing is left to add: the kernel norms the residual rows as they are
         elif deferred:

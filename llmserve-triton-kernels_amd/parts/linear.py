@@ -1,9 +1,10 @@
 """y = x W^T (+ b) for the parts: picks the matrix product by dtype and shape.
 
 float32: the 32-bit multiply-add kernel, always (no reduced-precision matrix mode).
-bfloat16, up to 16 rows whose K fits a compute unit's LDS: ops.gemm_decode, one workgroup per compute
-  unit, which also norms its rows on the way in and adds its result to the residual rows where the
-  parts ask for that (decode_product).
+bfloat16, up to 16 rows whose K fits a compute unit's LDS, or 17 to 64 rows of up to 2,048 columns:
+  ops.gemm_decode, one workgroup per compute unit, with the activation or the rotation and cache store in
+  its epilogue; up to 32 rows it also norms its rows on the way in and adds its result to the residual
+  rows where the parts ask for that (decode_product, adds_residual_in_epilogue).
 bfloat16, few rows otherwise: the hand-written kernel that streams the weight once
   (ops.gemm_stream); it takes up to 64 rows, one workgroup per 16 rows and 16 weight rows, so
   beyond 16 rows the weights are re-read from L2 and it only pays for the smaller matrices.
@@ -39,12 +40,27 @@ STREAM_MAX_ROWS = 64
 STREAM_REREAD_BYTES = 64e6
 
 
+# A plain product of up to 8 rows against a weight this large (the vocabulary's) stays with the streaming kernel:
+# its two thousand small workgroups even out better than 256 large ones with a barrier per group of tiles
+# (measured on 32000 x 2048: 25.8 and 27.0 microseconds at 1 and 8 rows against 27.9 and 28.3).
+STREAM_LARGE_ROWS = 8
+STREAM_LARGE_BYTES = 100e6
+
 DECODE_KERNEL = os.environ.get("LLMSERVE_DECODE_GEMM", "1") != "0"
 
 
 def decode_product(x: torch.Tensor, weight: torch.Tensor) -> bool:
     """Whether x [M, K] against weight goes to ops.gemm_decode (one workgroup per compute unit)."""
     return DECODE_KERNEL and ops.gemm_decode_supported(x, weight)
+
+
+def adds_residual_in_epilogue(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether a product whose result is added to the residual rows does that sum itself (ops.gemm_decode's
+    residual epilogue).  It pays while the norm that follows is the next product's prologue (up to
+    GEMM_DECODE_NORM_ROWS rows): with more rows that norm is a kernel of its own, which adds up partial sums
+    as it reads them, and a short, wide weight is faster shared out over K (measured at 32 and 64 rows on
+    2048 x 2048: 4.9 and 6.3 microseconds against 5.3 and 7.8; the norm kernel costs 5)."""
+    return x.shape[0] <= ops.GEMM_DECODE_NORM_ROWS and decode_product(x, weight)
 
 
 def few_rows(m: int, weight: torch.Tensor) -> bool:
@@ -113,7 +129,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     if m == 0:
         return out
     if x.dtype == torch.bfloat16 and ops.gemm_bf16_supported(x, weight):
-        if decode_product(x, weight):
+        if decode_product(x, weight) and not (m <= STREAM_LARGE_ROWS and weight.numel() * 2 >= STREAM_LARGE_BYTES):
             return ops.gemm_decode(out, x, weight, bias)
         if few_rows(m, weight):
             return ops.gemm_stream(out, x, weight, bias)

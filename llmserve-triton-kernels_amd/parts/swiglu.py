@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .linear import decode_product, few_rows, linear, linear_partial_sums
+from .linear import adds_residual_in_epilogue, decode_product, few_rows, linear, linear_partial_sums
 from .registry import ADDED_IN_PLACE, DeferredNorm, FeedForward, register_feed_forward
 from .spec import ParamInfo
 
@@ -42,7 +42,7 @@ class SwiGLU(FeedForward):
         dtype, device = self.gate_up.dtype, self.gate_up.device
         act = torch.empty((m, self.intermediate), dtype=dtype, device=device)
         if decode_product(rows, self.gate_up):
-            norm = x.fused() if deferred else None
+            norm = x.fused() if deferred and m <= ops.GEMM_DECODE_NORM_ROWS else None
             if norm is not None:
                 x.resolve(None)  # nothing is left to add: the kernel norms the residual rows as they are
             elif deferred:
@@ -56,7 +56,7 @@ class SwiGLU(FeedForward):
                 ops.gemm_stream(act, rows, self.gate_up, swiglu=True)  # activation in the product's epilogue
             else:
                 ops.silu_mul(act, linear(rows, self.gate_up))
-        if deferred and x.may_add_in_place and decode_product(act, self.down):
+        if deferred and x.may_add_in_place and adds_residual_in_epilogue(act, self.down):
             ops.gemm_decode(None, act, self.down, residual=x.residual)  # the residual sum in the product's epilogue
             return ADDED_IN_PLACE
         return (linear_partial_sums(act, self.down) if deferred else None) or linear(act, self.down)

@@ -53,13 +53,14 @@ def test_library_names_follow_the_headers_a_source_includes(tmp_path, monkeypatc
 @pytest.mark.parametrize("name,kernels,most_bytes", [
     ("gemm_stream", ("gemm_stream_kernel", "gemm_slices_kernel"), 0),
     ("attention_mfma", ("attn_prompt_kernel", "attn_mfma_kernel"), 64),
+    ("gemm_decode", ("gemm_decode_kernel", "gemm_decode_rows_kernel"), 128),
 ])
 def test_streaming_kernels_hold_what_they_fetch_in_registers(tmp_path, name, kernels, most_bytes):
     """What a lane has fetched and not yet used must stay in registers.  The compiler may lower an array of a
     struct (uint4) that one place fills and another empties to copies through the lane's private memory, which puts
     a wait behind every load: twice the time, and no numerics test sees it.  The kernels' private segment (in the
     code object's metadata) is empty, or holds the few registers spilt by the kernels that are compiled for two
-    workgroups per CU."""
+    workgroups per CU or that keep 64 rows of X in registers."""
     import re
     import subprocess
 
