@@ -74,18 +74,23 @@ __device__ __forceinline__ bf16 from_f32<bf16>(float v) {
 template <typename T>
 __device__ __forceinline__ float round_to(float v) { return to_f32(from_f32<T>(v)); }
 
-// Sine and cosine of position * frequency, and (a, b) turned by that angle.  Never inlined, and every product and
-// sum rounded on its own: inlined, the compiler schedules and contracts this arithmetic differently from kernel to
-// kernel, and a result that falls next to a rounding boundary of bfloat16 then differs between kernels that must
-// agree to the bit (the rotation kernel, and the products that rotate in their epilogue).
-// (Results come back by value: an address of a caller's variable would put it in private memory.)
+// Sine and cosine of position * frequency, and (a, b) turned by that angle, with the same bits in every kernel
+// that rotates (the rotation kernel, and the products that rotate in their epilogue): a result that falls next to a
+// rounding boundary of bfloat16 would otherwise differ between kernels that must agree.  The sine and cosine are
+// never inlined (inlined, the compiler specialises and schedules them differently from kernel to kernel; the result
+// comes back by value, since an address of a caller's variable would put it in private memory); the rotation is
+// inlined, which keeps a call's register saves out of the epilogues, with every product and sum rounded on its own
+// (no contraction to multiply-adds, which the compiler would otherwise choose by context).
 __device__ __noinline__ float2 rotary_angle(float position, float frequency) {  // (sine, cosine)
+#pragma clang fp contract(off)
     float sine, cosine;
-    sincosf(__fmul_rn(position, frequency), &sine, &cosine);
+    sincosf(position * frequency, &sine, &cosine);
     return make_float2(sine, cosine);
 }
-__device__ __noinline__ float2 rotate_pair(float a, float b, float cs, float sn) {
-    return make_float2(__fsub_rn(__fmul_rn(a, cs), __fmul_rn(b, sn)), __fadd_rn(__fmul_rn(b, cs), __fmul_rn(a, sn)));
+__device__ __forceinline__ float2 rotate_pair(float a, float b, float cs, float sn) {
+#pragma clang fp contract(off)
+    const float ac = a * cs, bs = b * sn, bc = b * cs, as = a * sn;
+    return make_float2(ac - bs, bc + as);
 }
 
 __device__ __forceinline__ float wave_sum(float v) {

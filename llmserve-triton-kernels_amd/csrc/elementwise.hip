@@ -448,6 +448,11 @@ __global__ void scatter_i32_kernel(int* __restrict__ dst, const int* __restrict_
         LLMS_REQUIRE(false, "dtype must be 0 (float32) or 1 (bfloat16)"); \
     }
 
+__global__ void rotary_angles_kernel(float2* out, const int* positions, const float* inv_freq, int total, int half) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) out[i] = rotary_angle((float)positions[i / half], inv_freq[i % half]);
+}
+
 extern "C" {
 
 int llms_embed_gather(int dtype, void* out, const void* table, const int* ids, int n_tokens, int hidden,
@@ -511,6 +516,16 @@ int llms_rope_store(int dtype, void* qkv, const float* inv_freq, const int* posi
     DISPATCH_DTYPE(dtype, rope_store_kernel<T><<<n_tokens, 256, 0, stream>>>(
                               (T*)qkv, inv_freq, positions, slots, (T*)k_pool, (T*)v_pool, n_heads,
                               n_kv_heads, head_dim, block_size);)
+    LLMS_LAUNCH_CHECK();
+}
+
+// out[m][i] = (sine, cosine) of positions[m] * inv_freq[i]: the angles of a step's tokens, once for all layers.
+int llms_rotary_angles(float* out, const int* positions, const float* inv_freq, int n_tokens, int half,
+                       hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && half > 0 && (long long)n_tokens * half < (1ll << 30), "rotary_angles: sizes out of range");
+    const int total = n_tokens * half;
+    rotary_angles_kernel<<<(total + 255) / 256, 256, 0, stream>>>(reinterpret_cast<float2*>(out), positions, inv_freq,
+                                                                  total, half);
     LLMS_LAUNCH_CHECK();
 }
 

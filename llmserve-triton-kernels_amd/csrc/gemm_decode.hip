@@ -67,7 +67,12 @@ struct DecodeGemmArgs {
     int x_pitch;    // bytes from row to row there: all chunks of K and 16 more (rows then start in different banks)
     int inter;  // SWIGLU
     int n_heads, n_kv_heads, head_dim, block_size;  // ROPE_QKV
+    // ceil(2^32 / (head_dim / 2)): a unit's head by one multiply (exact while unit * head_dim < 2^32, which the
+    // entry point checks); log2 of the page size, or -1 if it is no power of 2
+    unsigned half_inv;
+    int bs_shift;
     const float* inv_freq;
+    const float* angles;  // [M][head_dim / 2] (sine, cosine): given, it stands for positions and inv_freq
     const int* positions;
     const int* slots;
     bf16* k_pool;
@@ -116,7 +121,7 @@ __device__ __forceinline__ int gd_weight_row(const DecodeGemmArgs& a, int u0, in
     if (EPI == GD_SWIGLU) return hi ? a.inter + u : u;
     const int D = a.head_dim, half = D / 2, rot_units = (a.n_heads + a.n_kv_heads) * half;
     if (u < rot_units) {
-        const int h = u / half, j = u - h * half;
+        const int h = (int)__umulhi((unsigned)u, a.half_inv), j = u - h * half;
         return h * D + j + (hi ? half : 0);
     }
     return (a.n_heads + a.n_kv_heads) * D + (u - rot_units) + (hi ? a.n_kv_heads * half : 0);
@@ -127,11 +132,12 @@ __device__ __forceinline__ int gd_weight_row(const DecodeGemmArgs& a, int u0, in
 struct GdFinish {
     int pos, slot;
     float freq;
+    float sn, cs;
     unsigned res;
 };
 
 struct GdFinishBuffers {
-    __amdgpu_buffer_rsrc_t pos, slot, freq, res;
+    __amdgpu_buffer_rsrc_t pos, slot, freq, angles, res;
 };
 
 __device__ __forceinline__ GdFinishBuffers gd_finish_buffers(const DecodeGemmArgs& a) {
@@ -139,6 +145,7 @@ __device__ __forceinline__ GdFinishBuffers gd_finish_buffers(const DecodeGemmArg
     b.pos = gd_buffer(a.positions, a.positions ? (unsigned)a.M * 4 : 0u);
     b.slot = gd_buffer(a.slots, a.slots ? (unsigned)a.M * 4 : 0u);
     b.freq = gd_buffer(a.inv_freq, a.inv_freq ? (unsigned)a.head_dim * 2 : 0u);
+    b.angles = gd_buffer(a.angles, a.angles ? (unsigned)a.M * a.head_dim * 4 : 0u);
     b.res = gd_buffer(a.residual, a.residual ? (unsigned)(((size_t)(a.M - 1) * a.ldr + a.N) * 2) : 0u);
     return b;
 }
@@ -151,8 +158,16 @@ __device__ __forceinline__ void gd_ask(const DecodeGemmArgs& a, const GdFinishBu
         f.slot = (int)__builtin_amdgcn_raw_buffer_load_b32(b.slot, live ? (unsigned)m * 4 : GD_NOWHERE, 0, 0);
         if (!a.slots) f.slot = -1;
         const bool rot = live && u < (a.n_heads + a.n_kv_heads) * half;
-        f.pos = (int)__builtin_amdgcn_raw_buffer_load_b32(b.pos, rot ? (unsigned)m * 4 : GD_NOWHERE, 0, 0);
-        f.freq = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(b.freq, rot ? (unsigned)(u % half) * 4 : GD_NOWHERE, 0, 0));
+        // the angle's sine and cosine from the step's table, or position and frequency to work them out here
+        // (every load is issued either way, from nowhere where it is not wanted, so that their number is known)
+        const bool table = a.angles != nullptr;
+        const int i_rot = u - (int)__umulhi((unsigned)u, a.half_inv) * half;  // u % half
+        f.pos = (int)__builtin_amdgcn_raw_buffer_load_b32(b.pos, rot && !table ? (unsigned)m * 4 : GD_NOWHERE, 0, 0);
+        f.freq = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(b.freq, rot && !table ? (unsigned)i_rot * 4 : GD_NOWHERE, 0, 0));
+        typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+        const u32x2 sc = __builtin_amdgcn_raw_buffer_load_b64(b.angles, rot && table ? (unsigned)(m * half + i_rot) * 8 : GD_NOWHERE, 0, 0);
+        f.sn = __uint_as_float(sc[0]);
+        f.cs = __uint_as_float(sc[1]);
     }
     if (EPI == GD_RESIDUAL)
         f.res = __builtin_amdgcn_raw_buffer_load_b16(b.res, live ? (unsigned)(m * a.ldr + u) * 2 : GD_NOWHERE, 0, 0);
@@ -185,11 +200,12 @@ __device__ __forceinline__ void gd_finish_pair(const DecodeGemmArgs& a, int m, i
     lo = gd_bfr(lo);  // the projection's result is bfloat16 before it is rotated
     hi = gd_bfr(hi);
     const int slot = f.slot;
+    const int page = a.bs_shift >= 0 ? slot >> a.bs_shift : slot / bs, off = slot - page * bs;  // (used where slot >= 0)
     if (u < rot_units) {
-        const int h = u / half, d = u - h * half;
+        const int h = (int)__umulhi((unsigned)u, a.half_inv), d = u - h * half;
         float ra = lo, rb = hi;
-        if (a.inv_freq) {
-            const float2 angle = rotary_angle((float)f.pos, f.freq);
+        if (a.inv_freq || a.angles) {
+            const float2 angle = a.angles ? make_float2(f.sn, f.cs) : rotary_angle((float)f.pos, f.freq);
             const float2 r = rotate_pair(lo, hi, angle.y, angle.x);
             ra = r.x;
             rb = r.y;
@@ -199,16 +215,16 @@ __device__ __forceinline__ void gd_finish_pair(const DecodeGemmArgs& a, int m, i
             gd_store<TOut>(q, ra);
             gd_store<TOut>(q + half, rb);
         } else if (slot >= 0) {
-            const int page = slot / bs, off = slot % bs;
             bf16* dst = a.k_pool + (((size_t)page * nkv + (h - nh)) * bs + off) * D;
             dst[d].bits = f32_to_bf16_bits(ra);
             dst[d + half].bits = f32_to_bf16_bits(rb);
         }
     } else if (slot >= 0) {
-        const int page = slot / bs, off = slot % bs;
-        const int f_lo = u - rot_units, f_hi = f_lo + nkv * half;  // features among the value heads
-        a.v_pool[(((size_t)page * nkv + f_lo / D) * D + f_lo % D) * bs + off].bits = f32_to_bf16_bits(lo);
-        a.v_pool[(((size_t)page * nkv + f_hi / D) * D + f_hi % D) * bs + off].bits = f32_to_bf16_bits(hi);
+        // features f_lo and f_hi among the value heads: a page holds [kv head][dimension][token], and kv head times
+        // D plus dimension is the feature itself
+        const int f_lo = u - rot_units, f_hi = f_lo + nkv * half;
+        a.v_pool[((size_t)page * nkv * D + f_lo) * bs + off].bits = f32_to_bf16_bits(lo);
+        a.v_pool[((size_t)page * nkv * D + f_hi) * bs + off].bits = f32_to_bf16_bits(hi);
     }
 }
 
@@ -665,6 +681,7 @@ static void gd_launch_rows_one_chunk(int tiles, unsigned grid, DecodeGemmArgs& a
 template <typename TOut, int EPI, int RB, bool NORM>
 static void gd_launch_rows_two_chunks(int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
     if (tiles == 1) GR_GO(2, RB, 1);
+    else if constexpr (RB == 4) GR_GO(2, RB, 2);  // (three tiles of 64 rows of two chunks would not fit the registers)
     else if (tiles % 3 == 0 || tiles > 4) GR_GO(2, RB, 3);
     else GR_GO(2, RB, 2);
 }
@@ -728,14 +745,15 @@ int llms_gemm_decode_fits(int M, int K) {
 
 // epilogue: 0 plain (C [M,N] + bias; out_dtype 0 float32, 1 bfloat16), 1 gated (W = [gate; up] of `inter` rows each,
 // C [M, inter] bfloat16), 2 rotary q/k/v (W = [q; k; v], C = q [M, n_heads*head_dim] bfloat16, k and v stored at
-// `slots` when given), 3 residual (residual[M, N] += X W^T in place, bfloat16; C unused).
+// `slots` when given; the angles as position times inv_freq, or their sines and cosines as `angles` [M][head_dim / 2][2],
+// or neither: no rotation), 3 residual (residual[M, N] += X W^T in place, bfloat16; C unused).
 // norm_weight (bfloat16 [K]) given: the rows of X are replaced by RMSNorm(X) * norm_weight with `eps` on the way in.
 // workgroups: how many share the work out (the caller passes the number of compute units).
 int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* X, int ldx, const void* W,
                      const void* bias, const void* norm_weight, float eps, int M, int N, int K, int inter,
                      int n_heads, int n_kv_heads, int head_dim, int block_size, const float* inv_freq,
-                     const int* positions, const int* slots, void* k_pool, void* v_pool, void* residual, int ldr,
-                     int workgroups, hipStream_t stream) {
+                     const float* angles, const int* positions, const int* slots, void* k_pool, void* v_pool,
+                     void* residual, int ldr, int workgroups, hipStream_t stream) {
     LLMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_decode: needs 1 <= M <= 64 and positive sizes");
     LLMS_REQUIRE((long long)N * K < (1ll << 30) && (long long)M * ldx < (1ll << 30), "gemm_decode: operands of 2 GB or more");
     const int x_rows = M <= 8 ? 8 : 16, x_pitch = (K + GD_KC - 1) / GD_KC * (GD_KC * 2) + 16;
@@ -748,7 +766,7 @@ int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* 
     LLMS_REQUIRE(out_dtype == 1 || (out_dtype == 0 && epilogue == GD_PLAIN), "gemm_decode: 32-bit output goes with the plain epilogue");
     LLMS_REQUIRE(workgroups > 0 && workgroups <= 4096, "gemm_decode: bad number of workgroups");
     DecodeGemmArgs a = {(const bf16*)W, (const bf16*)X, (const bf16*)bias, (const bf16*)norm_weight, eps, C, ldc, ldx,
-                        M, N, K, 0, 0, 0, 0, x_rows, x_pitch, inter, n_heads, n_kv_heads, head_dim, block_size, inv_freq, positions, slots,
+                        M, N, K, 0, 0, 0, 0, x_rows, x_pitch, inter, n_heads, n_kv_heads, head_dim, block_size, 0u, -1, inv_freq, angles, positions, slots,
                         (bf16*)k_pool, (bf16*)v_pool, (bf16*)residual, ldr};
     if (epilogue == GD_PLAIN) {
         LLMS_REQUIRE(C != nullptr && ldc >= N, "gemm_decode: bad output");
@@ -761,13 +779,17 @@ int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* 
                      "gemm_decode: the gated epilogue needs N = 2*inter and no bias");
         a.units = inter;
     } else {
-        LLMS_REQUIRE(C != nullptr && n_heads > 0 && n_kv_heads > 0 && head_dim >= 2 && head_dim % 2 == 0 &&
+        LLMS_REQUIRE(C != nullptr && n_heads > 0 && n_kv_heads > 0 && head_dim >= 4 && head_dim % 2 == 0 &&
                          (n_kv_heads * head_dim) % 2 == 0 && N == (n_heads + 2 * n_kv_heads) * head_dim &&
                          ldc >= n_heads * head_dim,
-                     "gemm_decode: the rotary epilogue needs an even head_dim and N = (heads + 2 kv heads) * head_dim");
+                     "gemm_decode: the rotary epilogue needs an even head_dim of 4 or more and N = (heads + 2 kv heads) * head_dim");
         LLMS_REQUIRE(positions != nullptr || inv_freq == nullptr, "gemm_decode: rotation needs positions");
+        LLMS_REQUIRE(angles == nullptr || ((uintptr_t)angles % 8) == 0, "gemm_decode: the table of angles must be 8-byte aligned");
         LLMS_REQUIRE(slots == nullptr || (k_pool && v_pool && block_size > 0), "gemm_decode: slots given without pools");
         a.units = (n_heads + n_kv_heads) * (head_dim / 2) + n_kv_heads * head_dim / 2;
+        LLMS_REQUIRE((long long)a.units * head_dim < (1ll << 32), "gemm_decode: too many heads for the rotary epilogue");
+        a.half_inv = (unsigned)(((1ull << 32) + head_dim / 2 - 1) / (head_dim / 2));
+        a.bs_shift = block_size > 0 && (block_size & (block_size - 1)) == 0 ? __builtin_ctz((unsigned)block_size) : -1;
     }
     const unsigned grid = (unsigned)(workgroups < a.units ? workgroups : a.units);
     a.units_each = a.units / (int)grid;

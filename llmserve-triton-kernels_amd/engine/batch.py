@@ -44,6 +44,9 @@ class StepBatch:
     max_count: int = 0
     max_context: int = 0
     max_decode_context: int = 0  # longest context among the leading single-token requests
+    # what a part has worked out for this step and the same kind of part in later layers can use again (the sines
+    # and cosines of the tokens' angles); emptied by the model when a step starts
+    shared: dict = field(default_factory=dict)
 
 
 class BatchUploader:

@@ -214,6 +214,20 @@ def rope_store(qkv: torch.Tensor, inv_freq: torch.Tensor | None, positions: torc
         "rope_store")
 
 
+def rotary_angles(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """float32 [N, half, 2]: (sine, cosine) of positions[n] * inv_freq[i], by the arithmetic of the kernels that
+    rotate: a step's angles worked out once, for every layer's product with the rotary epilogue to read."""
+    dev = _dev(positions, inv_freq)
+    _i32(positions, "positions")
+    _f32(inv_freq, "inv_freq")
+    n, half = positions.numel(), inv_freq.numel()
+    out = torch.empty((n, half, 2), dtype=torch.float32, device=dev)
+    if n and half:
+        _check(load("elementwise").llms_rotary_angles(_ptr(out), _ptr(positions), _ptr(inv_freq), c_int(n), c_int(half),
+                                                      _stream(dev)), "rotary_angles")
+    return out
+
+
 def scatter_i32(dst: torch.Tensor, index: torch.Tensor, value: torch.Tensor) -> None:
     """dst.flatten()[index[i]] = value[i] wherever index[i] >= 0.  The caller has checked the indices."""
     dev = _dev(dst, index, value)
@@ -346,7 +360,7 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
         raise ValueError("one epilogue at a time")
     epilogue, inter, cols = 0, 0, n
     r = dict(n_heads=0, n_kv_heads=0, head_dim=0, block_size=0, inv_freq=None, positions=None, slots=None,
-             k_pool=None, v_pool=None)
+             k_pool=None, v_pool=None, angles=None)
     if swiglu:
         if n % 16 or bias is not None:
             raise ValueError("the gated epilogue needs 2I % 16 == 0 and no bias")
@@ -359,6 +373,8 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
         _i32(r["positions"], "positions", m)
         if r["inv_freq"] is not None:
             _f32(r["inv_freq"], "inv_freq", d // 2)
+        if r["angles"] is not None:
+            _f32(r["angles"], "angles", m * d)
         if r["slots"] is not None:
             _i32(r["slots"], "slots", m)
             bs, kp, vp = r["block_size"], r["k_pool"], r["v_pool"]
@@ -366,7 +382,7 @@ def gemm_stream(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch
             if (tuple(kp.shape) != (pages, nkv, bs, d) or tuple(vp.shape) != (pages, nkv, d, bs)
                     or not kp.is_contiguous() or not vp.is_contiguous() or kp.dtype != x.dtype or vp.dtype != x.dtype):
                 raise ValueError("pools do not have the cache layout [pages, kv, block, D] / [pages, kv, D, block]")
-        _dev(x, r["inv_freq"], r["positions"], r["slots"], r["k_pool"], r["v_pool"])
+        _dev(x, r["inv_freq"], r["angles"], r["positions"], r["slots"], r["k_pool"], r["v_pool"])
         epilogue, cols = 2, nh * d
     if tuple(out.shape) != (m, cols):
         raise ValueError(f"out shape {tuple(out.shape)} is not {(m, cols)}")
@@ -418,8 +434,9 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
     plain:     out[M, N] = x w^T (+ bias), bfloat16 or float32.
     swiglu:    w = [gate; up] ([2I, K]); out[M, I] = silu(gate) * up.
     rope = dict(n_heads, n_kv_heads, head_dim, inv_freq | None, positions, slots | None, k_pool, v_pool,
-               block_size): w = [q; k; v]; out[M, n_heads * head_dim] = rotated q; rotated k and v are stored at
-               the tokens' cache slots.
+               block_size, angles | None): w = [q; k; v]; out[M, n_heads * head_dim] = rotated q; rotated k and v
+               are stored at the tokens' cache slots.  `angles` (rotary_angles(positions, inv_freq), float32
+               [M, head_dim / 2, 2]) saves the kernel the sines and cosines; the result is the same to the bit.
     residual:  residual[M, N] += x w^T (+ bias) in place (32-bit sum of the rounded product and the row, rounded
                once); `out` is not used and `residual` is returned."""
     dev = _dev(out, x, w, bias, residual, norm[0] if norm else None)
@@ -452,7 +469,7 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
             raise ValueError("the norm's weight must be a contiguous, 16-byte aligned bfloat16 vector of K elements")
     epilogue, inter, cols = 0, 0, n
     r = dict(n_heads=0, n_kv_heads=0, head_dim=0, block_size=0, inv_freq=None, positions=None, slots=None,
-             k_pool=None, v_pool=None)
+             k_pool=None, v_pool=None, angles=None)
     if swiglu:
         if n % 2 or bias is not None:
             raise ValueError("the gated epilogue needs an even number of weight rows and no bias")
@@ -465,6 +482,8 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
         _i32(r["positions"], "positions", m)
         if r["inv_freq"] is not None:
             _f32(r["inv_freq"], "inv_freq", d // 2)
+        if r["angles"] is not None:
+            _f32(r["angles"], "angles", m * d)
         if r["slots"] is not None:
             _i32(r["slots"], "slots", m)
             bs, kp, vp = r["block_size"], r["k_pool"], r["v_pool"]
@@ -472,7 +491,7 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
             if (tuple(kp.shape) != (pages, nkv, bs, d) or tuple(vp.shape) != (pages, nkv, d, bs)
                     or not kp.is_contiguous() or not vp.is_contiguous() or kp.dtype != x.dtype or vp.dtype != x.dtype):
                 raise ValueError("pools do not have the cache layout [pages, kv, block, D] / [pages, kv, D, block]")
-        _dev(x, r["inv_freq"], r["positions"], r["slots"], r["k_pool"], r["v_pool"])
+        _dev(x, r["inv_freq"], r["angles"], r["positions"], r["slots"], r["k_pool"], r["v_pool"])
         epilogue, cols = 2, nh * d
     elif residual is not None:
         if (residual.dim() != 2 or residual.stride(1) != 1 or tuple(residual.shape) != (m, n)
@@ -488,7 +507,7 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
         c_int(1 if epilogue == 3 else _code(out)), c_int(epilogue), _ptr(None if epilogue == 3 else out),
         c_int(0 if epilogue == 3 else out.stride(0)), _ptr(x), c_int(x.stride(0)), _ptr(w), _ptr(bias),
         _ptr(norm_weight), c_float(eps), c_int(m), c_int(n), c_int(k), c_int(inter), c_int(r["n_heads"]),
-        c_int(r["n_kv_heads"]), c_int(r["head_dim"]), c_int(r["block_size"]), _ptr(r["inv_freq"]), _ptr(r["positions"]),
+        c_int(r["n_kv_heads"]), c_int(r["head_dim"]), c_int(r["block_size"]), _ptr(r["inv_freq"]), _ptr(r["angles"]), _ptr(r["positions"]),
         _ptr(r["slots"]), _ptr(r["k_pool"]), _ptr(r["v_pool"]), _ptr(residual),
         c_int(residual.stride(0) if residual is not None else 0), c_int(compute_units(dev)), _stream(dev)), "gemm_decode")
     return residual if epilogue == 3 else out

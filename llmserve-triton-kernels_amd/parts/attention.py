@@ -119,6 +119,9 @@ class Attention(Mixer):
                     slots=slots, k_pool=cache.k_pool, v_pool=cache.v_pool, block_size=cache.block_size)
         q = torch.empty((m, self.num_heads * self.head_dim), dtype=rows.dtype, device=rows.device)
         if decode:
+            angles = getattr(self.position, "rotary_angles", None)
+            if angles is not None and getattr(batch, "shared", None) is not None:
+                rope["angles"] = angles(batch)  # worked out once per step, not once per layer and workgroup
             ops.gemm_decode(q, rows, self.qkv_weight, self.qkv_bias, rope=rope, norm=norm)
         else:
             ops.gemm_stream(q, rows, self.qkv_weight, self.qkv_bias, rope=rope)
@@ -135,16 +138,16 @@ class Attention(Mixer):
         common = (out, qkv, cache.k_pool, cache.v_pool, view.block_tables, batch.cu_seqlens, batch.context_lens)
         n_dec = batch.num_decode
         if n_dec:  # requests that bring one token: their keys are spread over waves and workgroups
-            splits, waves = self.decode_arrangement(n_dec, batch.max_decode_context)
+            splits, waves = self.decode_arrangement(n_dec, batch.max_decode_context, ops.compute_units(qkv.device))
             ops.attention_mfma(*common, 0, n_dec, 1, 0, n_dec, nh, nkv, d, bs, window, self.scale,
                                split_waves=True, num_splits=splits, waves=waves, table_rows=batch.state_slots)
         if n_dec < batch.num_seqs:  # portions of prompts: one wave per group of tokens and heads
-            splits = self.prompt_splits(batch.num_seqs - n_dec, batch.max_count, batch.max_context)
+            splits = self.prompt_splits(batch.num_seqs - n_dec, batch.max_count, batch.max_context, ops.compute_units(qkv.device))
             ops.attention_mfma(*common, n_dec, batch.num_seqs - n_dec, batch.max_count, n_dec,
                                batch.num_tokens - n_dec, nh, nkv, d, bs, window, self.scale, num_splits=splits,
                                table_rows=batch.state_slots)
 
-    def prompt_splits(self, n_requests: int, max_new: int, max_context: int) -> int:
+    def prompt_splits(self, n_requests: int, max_new: int, max_context: int, cus: int = 256) -> int:
         """Workgroups that share the keys of one block of prompt tokens (a second kernel merges their shares).
         Blocks enough for a workgroup of 8 waves on every CU need no sharing: there each wave has a twin that
         takes every other tile of keys for the same tokens, and with two such workgroups per CU the long blocks
@@ -153,7 +156,7 @@ class Attention(Mixer):
         are shared out, 8 tiles of keys a workgroup at least (16 where the blocks alone are half a chip), up to
         about two workgroups of 4 waves per CU, and not in more than 4 once the blocks alone are a quarter of a
         chip (measured on portions of 16 to 256 tokens behind 256 to 4,032 keys, at head sizes 64 and 128: the
-        merge kernel's work grows with blocks times shares)."""
+        merge kernel's work grows with blocks times shares).  `cus`: the device's compute units."""
         if self.window:
             return 1
         g = self.num_heads // self.num_kv_heads
@@ -161,28 +164,28 @@ class Attention(Mixer):
         blocks = -(-max_new // (4 * (16 // hg)))  # of 4 waves with one column group each
         workgroups = blocks * self.num_kv_heads * -(-g // hg) * n_requests
         tiles = -(-max_context // 32)
-        if workgroups >= 512:
+        if workgroups >= 2 * cus:
             return 1
-        if workgroups >= 256:
+        if workgroups >= cus:
             return 4 if tiles >= 96 else 1
-        per_share = 16 if workgroups >= 128 else 8
-        most = 4 if workgroups >= 64 else 8
-        return max(1, min(512 // max(workgroups, 1), tiles // per_share, most))
+        per_share = 16 if workgroups >= cus // 2 else 8
+        most = 4 if workgroups >= cus // 4 else 8
+        return max(1, min(2 * cus // max(workgroups, 1), tiles // per_share, most))
 
-    def decode_arrangement(self, n_requests: int, max_context: int) -> tuple[int, int]:
+    def decode_arrangement(self, n_requests: int, max_context: int, cus: int = 256) -> tuple[int, int]:
         """(workgroups per request and KV head, waves per workgroup) for decoding.  The waves of a
         workgroup take 32 keys at a time each and merge in LDS; workgroups that share a request hand
         their shares to the one that finishes last, through memory, which costs more (2 to 3
         microseconds) than a few extra tiles per wave.  So a small batch first gets 8 waves, and is
         split over workgroups only when a wave would still walk more than 4 tiles (measured: at a
         context of 512 no split pays at any batch size, at 4,096 four to eight do up to batch 8); once
-        the batch alone fills the chip (256 workgroups) nothing is split."""
+        the batch alone fills the chip (a workgroup for each of its `cus` compute units) nothing is split."""
         g = self.num_heads // self.num_kv_heads
         groups = n_requests * self.num_kv_heads * -(-g // 16)
         reach = min(max_context, self.window) if self.window else max_context
         waves = 8 if self.head_dim <= 160 else 4  # (8 waves of wider heads would not fit the registers)
-        if groups >= 256:
+        if groups >= cus:
             return 1, waves
         tiles = -(-reach // 32)
-        splits = max(1, min(256 // groups, -(-tiles // (4 * waves))))
+        splits = max(1, min(cus // groups, -(-tiles // (4 * waves))))
         return splits, waves

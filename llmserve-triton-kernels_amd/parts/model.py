@@ -92,6 +92,9 @@ class Model:
     # ---- one step ----------------------------------------------------------------------------
     def forward(self, batch, storage) -> torch.Tensor:
         """Logits [R, vocab] in 32-bit at `batch.logit_rows` (empty tensor when R = 0)."""
+        shared = getattr(batch, "shared", None)
+        if shared is not None:
+            shared.clear()  # (a batch object may serve several steps)
         x = self.embedding.forward(batch.token_ids)
         delta = None
         if self._sources is None:

@@ -39,6 +39,15 @@ class RotaryEncoding(PositionEncoding):
         position * frequency, which lets a mixer fold the rotation into a kernel of its own."""
         return self.inv_freq
 
+    def rotary_angles(self, batch):
+        """float32 [N, head_dim / 2, 2]: sine and cosine of every new token's angles.  The first layer of a step
+        that asks works them out (one small kernel); the others find them in what the step's parts share."""
+        key = ("rotary_angles", self.head_dim, self.theta)
+        table = batch.shared.get(key)
+        if table is None:
+            table = batch.shared[key] = ops.rotary_angles(batch.positions, self.inv_freq)
+        return table
+
     def rotate(self, qkv, positions, n_heads, n_kv_heads, head_dim):
         ops.rope_store(qkv, self.inv_freq, positions, None, None, None, n_heads, n_kv_heads, head_dim, 1)
 

@@ -452,6 +452,14 @@ def test_gemm_decode_rotary_epilogue(nh, nkv, d, bs, theta, bias, m):
     k3, v3 = pools()  # without slots only q is produced
     q3 = ops().gemm_decode(torch.empty(m, nh * d, dtype=torch.bfloat16, device=DEV), x, w, b, rope=dict(rope, slots=None, k_pool=k3, v_pool=v3))
     assert torch.equal(q3, q) and (k3 == 7).all() and (v3 == 7).all()
+    if theta:  # the sines and cosines from a table made ahead: the same bits
+        angles = ops().rotary_angles(positions, inv_freq)
+        exact = positions.double().cpu()[:, None] * inv_freq.double().cpu()[None, :]
+        assert (angles.cpu().double() - torch.stack([exact.sin(), exact.cos()], dim=-1)).abs().max() < 1e-3  # (32-bit angles of up to 4,096)
+        k4, v4 = pools()
+        q4 = ops().gemm_decode(torch.empty(m, nh * d, dtype=torch.bfloat16, device=DEV), x, w, b,
+                               rope=dict(rope, k_pool=k4, v_pool=v4, angles=angles))
+        assert torch.equal(q4, q) and torch.equal(k4, k2) and torch.equal(v4, v2)
 
 
 @pytest.mark.parametrize("m,n,k,bias", [(1, 64, 64, False), (8, 2048, 2048, False), (8, 2048, 5632, True), (16, 333, 176, True),
