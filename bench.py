@@ -181,11 +181,11 @@ def serve(args) -> int:
 
 
 def gemv(args) -> int:
-    """The decode step's matrix products one by one, as the step launches them (`ops.gemm_stream` with the
-    epilogue and the split of K the parts choose), at 1, 8 and 64 rows.  Every launch of a chain takes the next
-    of several copies of its weight, a gigabyte in all, so that nothing is left in the 256 MB memory-side cache
-    from the launch before (the convention of the reference's benchmarks/bench_decode_matmul.py:28,78-81); the
-    chain is captured as a graph, so the figure is device time per launch, start and drain included."""
+    """The decode step's matrix products one by one, as the step's parts launch them (the kernel, the epilogue and
+    the prologue they choose for the row count), at 1, 8, 32 and 64 rows.  Every launch of a chain takes the next of
+    several copies of its weight, a gigabyte in all, so that nothing is left in the 256 MB memory-side cache from the
+    launch before (the convention of the reference's benchmarks/bench_decode_matmul.py:28,78-81); the chain is
+    captured as a graph, so the figure is device time per launch, start and drain included."""
     import torch
 
     from llmserve.config import preset
@@ -196,28 +196,64 @@ def gemv(args) -> int:
     h, inter, vocab = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     nh, nkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
     d = h // nh
+    block_size = 16
     ops.ensure_built("bfloat16")
     dev = torch.device("cuda:0")
     shapes = {"qkv": ((nh + 2 * nkv) * d, h), "o_proj": (h, nh * d), "gate_up": (2 * inter, h), "down_proj": (h, inter),
               "lm_head": (vocab, h)}
+    inv_freq = (1.0 / (cfg.get("rope_theta", 10000.0) ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(dev)
     results = {}
     for name, (n, k) in shapes.items():
         copies = max(2, -(-(1 << 30) // (n * k * 2)))
         weights = [torch.randn(n, k, device=dev, dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
-        for m in (1, 8, 64):
+        norm_weight = torch.ones(k, device=dev, dtype=torch.bfloat16)
+        for m in (1, 8, 32, 64):
             x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+            decode = lin.decode_product(x, weights[0])
+            norm = (norm_weight, 1e-5) if decode and m <= ops.GEMM_DECODE_NORM_ROWS else None
+            how = "gemm_decode" if decode else "gemm_stream" if lin.few_rows(m, weights[0]) else "library"
             if name == "gate_up":
                 out = torch.empty(m, inter, device=dev, dtype=torch.bfloat16)
-                if lin.few_rows(m, weights[0]):
+                if decode:
+                    run = lambda w: ops.gemm_decode(out, x, w, swiglu=True, norm=norm)  # noqa: E731
+                elif lin.few_rows(m, weights[0]):
                     run = lambda w: ops.gemm_stream(out, x, w, swiglu=True)  # noqa: E731
                 else:
                     wide = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
                     run = lambda w: ops.silu_mul(out, torch.mm(x, w.t(), out=wide))  # noqa: E731
+                    how = "library + silu_mul"
+            elif name == "qkv":
+                positions = torch.randint(500, 600, (m,), dtype=torch.int32, device=dev)
+                slots = torch.randperm(64 * block_size, device=dev)[:m].to(torch.int32)
+                k_pool = torch.zeros(64, nkv, block_size, d, dtype=torch.bfloat16, device=dev)
+                v_pool = torch.zeros(64, nkv, d, block_size, dtype=torch.bfloat16, device=dev)
+                rope = dict(n_heads=nh, n_kv_heads=nkv, head_dim=d, inv_freq=inv_freq, positions=positions, slots=slots,
+                            k_pool=k_pool, v_pool=v_pool, block_size=block_size)
+                q = torch.empty(m, nh * d, dtype=torch.bfloat16, device=dev)
+                if decode:
+                    rope["angles"] = ops.rotary_angles(positions, inv_freq)
+                    run = lambda w: ops.gemm_decode(q, x, w, rope=rope, norm=norm)  # noqa: E731
+                elif lin.few_rows(m, weights[0]):
+                    run = lambda w: ops.gemm_stream(q, x, w, rope=rope)  # noqa: E731
+                else:
+                    wide = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+                    run = lambda w: ops.rope_store(torch.mm(x, w.t(), out=wide), inv_freq, positions, slots, k_pool,  # noqa: E731
+                                                   v_pool, nh, nkv, d, block_size)
+                    how = "library + rope_store"
             elif name in ("o_proj", "down_proj"):
-                run = lambda w: lin.linear_partial_sums(x, w) or lin.linear(x, w)  # noqa: E731
+                residual = torch.zeros(m, n, device=dev, dtype=torch.bfloat16)
+                if lin.adds_residual_in_epilogue(x, weights[0]):
+                    run = lambda w: ops.gemm_decode(None, x, w, residual=residual)  # noqa: E731
+                    how = "gemm_decode + residual"
+                else:
+                    run = lambda w: lin.linear_partial_sums(x, w) or lin.linear(x, w)  # noqa: E731
+                    how = "partial sums" if lin.linear_partial_sums(x, weights[0]) is not None else how
             else:
-                out_dtype = torch.float32 if name == "lm_head" else torch.bfloat16
-                run = lambda w: lin.linear(x, w, out_dtype=out_dtype)  # noqa: E731
+                run = lambda w: lin.linear(x, w, out_dtype=torch.float32)  # noqa: E731
+                if m <= lin.STREAM_LARGE_ROWS and n * k * 2 >= lin.STREAM_LARGE_BYTES:
+                    how = "gemm_stream"
+            if norm is not None and name in ("qkv", "gate_up"):
+                how += " + norm"
             for w in weights[:2]:
                 run(w)
             torch.cuda.synchronize()
@@ -233,7 +269,7 @@ def gemv(args) -> int:
                 graph.replay()
             torch.cuda.synchronize()
             us = (time.perf_counter() - t0) / (reps * copies) * 1e6
-            results[f"{name}_m{m}"] = {"us": round(us, 2), "GBps": round(n * k * 2 / us / 1e3, 1)}
+            results[f"{name}_m{m}"] = {"us": round(us, 2), "GBps": round(n * k * 2 / us / 1e3, 1), "kernel": how}
         del weights
     line = {"metric": "decode matrix products alone: microseconds per launch, weights streamed from HBM",
             "value": results["gate_up_m8"]["us"], "unit": "us", "n_gpus": 1, "steps": 0, "warmup": 0, "ms_per_step": 0.0,
@@ -296,7 +332,7 @@ def main() -> int:
     d = h // nh
     elem = 2 if args.dtype == "bfloat16" else 4
     block_size = 16
-    extra = not args.no_points and args.phase == "all"
+    extra = not args.no_points and args.phase in ("all", "decode")
     point_batches = [int(b) for b in args.points.split(",") if b] if extra else []
     point_contexts = [int(c) for c in args.context_points.split(",") if c] if extra else []
     max_batch = max([args.batch] + point_batches)

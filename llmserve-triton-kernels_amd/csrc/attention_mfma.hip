@@ -82,6 +82,9 @@ struct AttnArgs {
     // prompts with twins: the first workgroup of every CU (the first `first_blocks` values of blockIdx.y) takes one
     // of the longest blocks of tokens, shortest of them first; the rest follow from the longest remaining one down
     int first_blocks;
+    // decoding, every request of the launch with exactly one new token: the row of request seq_begin + i is
+    // one_token_from + i, which saves a workgroup the wait for cu_seqlens before it can ask for its queries (-1: not so)
+    int one_token_from;
 };
 
 // 2^x by the hardware's own instruction.  Scores are kept in units of log2(e) (scale_log2 = scale * log2 e), so
@@ -298,19 +301,38 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
     const int HB = (G + HG - 1) / HG;     // column groups needed to cover a KV head's query heads
     const int kvh = blockIdx.y / HB, hb = blockIdx.y % HB;
     const int b = a.seq_begin + blockIdx.z;
-    const int tok0 = a.cu_seqlens[b], n_new = a.cu_seqlens[b + 1] - tok0;
+    const bool one_each = a.one_token_from >= 0;
+    const int tok0 = one_each ? a.one_token_from + (int)blockIdx.z : a.cu_seqlens[b];
+    const int n_new = one_each ? 1 : a.cu_seqlens[b + 1] - tok0;
     const int ctx = a.context_lens[b];
     // (asked for together with the lengths: one trip to memory earlier than where the block table is first needed)
     const int table_row = a.table_rows ? a.table_rows[b] : b;
+    // The request's first 64 page ids are asked for before its length is known (whatever the length, they are the
+    // ones most launches need; entries beyond the request's own blocks are never used): with a table that has a row
+    // per request and one token each, a workgroup's lengths, page ids and queries are one trip to memory.
+    const int* table = a.block_tables + (size_t)table_row * a.max_blocks;
+    int blk_base = 0, pages_reg = table[min(lane, a.max_blocks - 1)];
 
     const int tile = blockIdx.x / a.num_splits, split = blockIdx.x % a.num_splits;
     const int t_first = tile * TPG;  // first token (within the request's new tokens) of this group
-    if (t_first >= n_new || ctx <= 0) return;  // (uniform over the workgroup)
 
     // this lane's column
     const int c_tok = t_first + col / HG, c_head_in = hb * HG + col % HG;
     const bool col_ok = col < HG * TPG && c_tok < n_new && c_head_in < G && tok0 + c_tok < a.row_end;
     const int head = kvh * G + c_head_in;
+    // queries of this lane's column: Q[col][32s + 8g .. +7]; asked for before the request's length is here where
+    // the rows are known without it
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    uint4 qf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int d = 32 * s + 8 * g;
+        qf[s] = (col_ok && d < D)
+                    ? *reinterpret_cast<const uint4*>(a.q + (size_t)(tok0 + c_tok) * a.q_stride + (size_t)head * D + d)
+                    : zero;
+    }
+    if (t_first >= n_new || ctx <= 0) return;  // (uniform over the workgroup)
+
     const int p_col = col_ok ? ctx - n_new + c_tok : -1;  // absolute position of the column's token
     const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
     // key range of the whole group
@@ -321,23 +343,11 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
     const int j_begin = lo_min & ~31;
     const int n_tiles = (p_max - j_begin) / 32 + 1;
 
-    // queries of this lane's column: Q[col][32s + 8g .. +7]
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-    uint4 qf[KS];
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        const int d = 32 * s + 8 * g;
-        qf[s] = (col_ok && d < D)
-                    ? *reinterpret_cast<const uint4*>(a.q + (size_t)(tok0 + c_tok) * a.q_stride + (size_t)head * D + d)
-                    : zero;
-    }
-
     f32x4 acc[DB];
 #pragma unroll
     for (int m = 0; m < DB; ++m) acc[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    const int* table = a.block_tables + (size_t)table_row * a.max_blocks;
     const uint32_t page_stride = (uint32_t)a.n_kv_heads * a.block_size * D;
     const bf16* k_base = a.k_pool + (size_t)kvh * a.block_size * D;
     const bf16* v_base = a.v_pool + (size_t)kvh * a.block_size * D;
@@ -355,8 +365,8 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
     const int bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
     auto block_of = [&](int key) { return bs_shift >= 0 ? key >> bs_shift : key / a.block_size; };
     const int last_blk = block_of(p_max);
-    int blk_base = 0, pages_reg = 0;
     auto load_pages = [&](int base) {
+        if (base == blk_base) return;  // (uniform over the wave; the first 64 are there from the start)
         blk_base = base;
         pages_reg = table[min(base + lane, last_blk)];
     };
@@ -987,7 +997,9 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     const int groups = (max_new + TPG - 1) / TPG;
     AttnArgs a = {(bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pool, (const bf16*)v_pool,
                   block_tables, table_rows, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
-                  window, scale, num_splits, ws_o, ws_ml, nullptr, token_begin + n_tokens, 0};
+                  window, scale, num_splits, ws_o, ws_ml, nullptr, token_begin + n_tokens, 0, -1};
+    // (at most one token each and as many tokens as requests: every request has exactly one, in the order of the requests)
+    if (split_waves > 0 && max_new == 1 && n_tokens == n_seqs) a.one_token_from = token_begin;
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
     LLMS_REQUIRE((unsigned long long)max_blocks * block_size * block_size <= 0xFFFFFFFFull,
                  "attention_mfma: block table too long for this page size (keys * block_size must stay below 2^32)");
