@@ -358,11 +358,11 @@ def main() -> int:
         lo = min(100, vocab // 4)
         return [torch.randint(lo, vocab, (length,), generator=gen).tolist() for _ in range(n)]
 
-    def decode_rate(batch, context=args.context):
+    def decode_rate(batch, context=args.context, **sampling):
         eng = ContinuousBatchingEngine(runner, sampler, max_num_seqs=batch,
                                        max_num_batched_tokens=engine_cfg.max_num_batched_tokens)
         for p in prompts(batch, context):
-            eng.add_request(p, SamplingParams(max_new_tokens=new_tokens_for(batch, context)))
+            eng.add_request(p, SamplingParams(max_new_tokens=new_tokens_for(batch, context), **sampling))
         while eng.waiting or any(r.num_tokens - r.num_computed_tokens > 1 for r in eng.running):
             eng.step()  # prompts in
         for _ in range(args.warmup):
@@ -396,6 +396,8 @@ def main() -> int:
         points[f"decode_b{b}"] = round(decode_rate(b)[0], 1)
     for c in point_contexts:
         points[f"decode_b{args.batch}_ctx{c}"] = round(decode_rate(args.batch, c)[0], 1)
+    if extra:  # every request with temperature, top-k and top-p (the device sampler's longest path) instead of greedy
+        points[f"decode_b{args.batch}_sampled"] = round(decode_rate(args.batch, temperature=0.8, top_k=40, top_p=0.95)[0], 1)
     served = serve_summary(torch, runner, sampler, vocab, budget, max_batch) if extra and not args.no_serve else {}
     pre_s = prefill_time() if args.phase != "decode" else float("inf")
     chunked_s = prefill_time(PREFILL_CHUNK) if args.phase == "all" else float("inf")

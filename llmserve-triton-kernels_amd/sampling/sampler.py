@@ -61,9 +61,38 @@ class PendingTokens:
         return self._host.tolist()  # the step's one read-back
 
 
+class _Staging:
+    """A small ring of pinned host buffers for a step's sampling options, each guarded by an event: the options go
+    to the device with one copy that the host does not wait for (a copy from pageable memory would make it wait)."""
+
+    def __init__(self, ring: int = 4):
+        self._buffers: list[torch.Tensor | None] = [None] * ring
+        self._events: list[torch.cuda.Event | None] = [None] * ring
+        self._next = 0
+
+    def send(self, values: torch.Tensor, device: torch.device) -> torch.Tensor:
+        """values: int32 [n] on the host (pageable).  Returns the same numbers on the device."""
+        i = self._next
+        self._next = (i + 1) % len(self._buffers)
+        n = values.numel()
+        if self._events[i] is not None:
+            self._events[i].synchronize()  # the copy that last used this buffer is done
+        if self._buffers[i] is None or self._buffers[i].numel() < n:
+            self._buffers[i] = torch.empty(max(256, 2 * n), dtype=torch.int32, pin_memory=True)
+        host = self._buffers[i][:n]
+        host.copy_(values)
+        out = torch.empty(n, dtype=torch.int32, device=device)
+        out.copy_(host, non_blocking=True)
+        if self._events[i] is None:
+            self._events[i] = torch.cuda.Event()
+        self._events[i].record(torch.cuda.current_stream(device))
+        return out
+
+
 class Sampler:
     def __init__(self, device: torch.device):
         self.device = device
+        self._staging = _Staging()
 
     def sample(self, logits: torch.Tensor, items: list[tuple[SamplingParams, int, int]]) -> list[int]:
         """logits float32 [R, V]; items[r] = (params, seed, index of the token being generated)."""
@@ -81,9 +110,12 @@ class Sampler:
         if all(p.temperature <= 0 for p, _, _ in items):
             ops.sample_rows(out, logits)
         else:
-            host = torch.tensor(
-                [[max(p.temperature, 0.0), float(p.top_p), uniform(seed, index)] for p, seed, index in items],
-                dtype=torch.float32).t().contiguous().to(logits.device)
-            top_k = torch.tensor([p.top_k for p, _, _ in items], dtype=torch.int32).to(logits.device)
-            ops.sample_rows(out, logits, temperature=host[0], top_k=top_k, top_p=host[1], uniform=host[2])
+            # temperature, top-p and the uniform numbers as 32-bit floats, top-k as integers: one buffer, one copy
+            floats = torch.tensor([[max(p.temperature, 0.0) for p, _, _ in items], [float(p.top_p) for p, _, _ in items],
+                                   [uniform(seed, index) for _, seed, index in items]], dtype=torch.float32)
+            top_k = torch.tensor([p.top_k for p, _, _ in items], dtype=torch.int32)
+            sent = self._staging.send(torch.cat([floats.view(torch.int32).reshape(-1), top_k]), logits.device)
+            options = sent[: 3 * r].view(torch.float32)
+            ops.sample_rows(out, logits, temperature=options[:r], top_k=sent[3 * r:], top_p=options[r: 2 * r],
+                            uniform=options[2 * r:])
         return PendingTokens(out)
