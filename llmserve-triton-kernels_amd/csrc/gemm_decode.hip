@@ -543,6 +543,7 @@ __global__ __launch_bounds__(GR_NW* LLMS_WAVE) void gemm_decode_rows_kernel(cons
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
+                if (16 * rb + 4 * i >= M) continue;  // (rows that do not exist are zeros and stay zeros)
                 float ss = 0.f;
 #pragma unroll
                 for (int j = 0; j < XC; ++j)
@@ -560,6 +561,7 @@ __global__ __launch_bounds__(GR_NW* LLMS_WAVE) void gemm_decode_rows_kernel(cons
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
+                if (16 * rb + 4 * i >= M) continue;
                 float total = 0.f;
 #pragma unroll
                 for (int w = 0; w < NW; w += 4) {
