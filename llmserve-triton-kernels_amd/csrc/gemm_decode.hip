@@ -79,6 +79,11 @@ struct DecodeGemmArgs {
     bf16* v_pool;
     bf16* residual;  // RESIDUAL
     int ldr;
+    // 17 to 64 rows, plain 32-bit output: K shared out to k_parts sets of wgs_per_part workgroups, part p taking the
+    // columns from p * k_each on (k_each a multiple of 128) and leaving its sums at C + p * part_stride; a norm adds the
+    // parts up.  ldw is the row stride of W (K of the whole weight).
+    int ldw, k_parts, k_each, wgs_per_part;
+    long long part_stride;
 };
 
 __device__ __forceinline__ bf16x8 gd_as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
@@ -175,10 +180,11 @@ __device__ __forceinline__ void gd_ask(const DecodeGemmArgs& a, const GdFinishBu
 
 // PLAIN, RESIDUAL: the sum `s` of weight row n and row m of X.
 template <typename TOut, int EPI>
-__device__ __forceinline__ void gd_finish_row(const DecodeGemmArgs& a, int m, int n, float s, const GdFinish& f) {
+__device__ __forceinline__ void gd_finish_row(const DecodeGemmArgs& a, int m, int n, float s, const GdFinish& f,
+                                              size_t part_offset = 0) {
     if (a.bias) s += bf16_bits_to_f32(a.bias[n].bits);
     if (EPI == GD_PLAIN)
-        gd_store<TOut>(reinterpret_cast<TOut*>(a.C) + (size_t)m * a.ldc + n, s);
+        gd_store<TOut>(reinterpret_cast<TOut*>(a.C) + part_offset + (size_t)m * a.ldc + n, s);
     else
         a.residual[(size_t)m * a.ldr + n].bits = f32_to_bf16_bits(bf16_bits_to_f32((uint16_t)f.res) + gd_bfr(s));
 }
@@ -476,8 +482,9 @@ __global__ __launch_bounds__(GR_NW* LLMS_WAVE) void gemm_decode_rows_kernel(cons
     float* sq_lds = red;  // the norm's sums of squares, [row][wave], before the first sums of the product
     const int tid = threadIdx.x, wave = tid / LLMS_WAVE, lane = tid % LLMS_WAVE;
     const int r16 = lane % 16, g = lane / 16;
-    const int M = a.M, K = a.K, n_chunks = (K + GD_KC - 1) / GD_KC;
-    const int wg = blockIdx.x;
+    const int part = (int)blockIdx.x / a.wgs_per_part, wg = (int)blockIdx.x - part * a.wgs_per_part;
+    const int k_from = part * a.k_each;
+    const int M = a.M, K = min(a.K - k_from, a.k_each), n_chunks = (K + GD_KC - 1) / GD_KC;  // (this part's columns)
     const int u_begin = wg * a.units_each + min(wg, a.units_more);
     const int u_last = u_begin + a.units_each + (wg < a.units_more ? 1 : 0);
 
@@ -486,7 +493,7 @@ __global__ __launch_bounds__(GR_NW* LLMS_WAVE) void gemm_decode_rows_kernel(cons
     // they reach the operand layout (lane (r16, g): X[16 rb + r16][c*128 + 32 s + 8 g ..+7]) through the wave's
     // LDS tile further down
     u32x4 xr[XC][RB][4];
-    const __amdgpu_buffer_rsrc_t x_buf = gd_buffer(a.X, (unsigned)(((size_t)(M - 1) * a.ldx + K) * 2));
+    const __amdgpu_buffer_rsrc_t x_buf = gd_buffer(a.X + k_from, (unsigned)(((size_t)(M - 1) * a.ldx + K) * 2));
 #pragma unroll
     for (int j = 0; j < XC; ++j)
 #pragma unroll
@@ -523,14 +530,14 @@ __global__ __launch_bounds__(GR_NW* LLMS_WAVE) void gemm_decode_rows_kernel(cons
     ask_finish(0, fin);
 
     u32x4 ring[RING][LPI];
-    const __amdgpu_buffer_rsrc_t w_buf = gd_buffer(a.W, (unsigned)((size_t)a.N * K * 2));
+    const __amdgpu_buffer_rsrc_t w_buf = gd_buffer(a.W + k_from, (unsigned)(((size_t)(a.N - 1) * a.ldw + K) * 2));
     auto issue = [&](u32x4(&w)[LPI], int tile0, int q) {
         const int c = wave + NW * (q % XC), kl = c * GD_KC + 8 * (lane % 16);
         const int u0 = u_begin + (tile0 + q / XC) * UPT;
 #pragma unroll
         for (int i = 0; i < LPI; ++i) {
             const int n = gd_weight_row<EPI>(a, u0, u_last, UPT, i * 4 + lane / 16);
-            w[i] = gd_load_streaming(w_buf, n >= 0 && kl < K ? (unsigned)(n * K + kl) * 2 : GD_NOWHERE);
+            w[i] = gd_load_streaming(w_buf, n >= 0 && kl < K ? (unsigned)(n * a.ldw + kl) * 2 : GD_NOWHERE);
         }
     };
 #pragma unroll
@@ -649,7 +656,7 @@ __global__ __launch_bounds__(GR_NW* LLMS_WAVE) void gemm_decode_rows_kernel(cons
                 return sum;
             };
             if (m >= M || u >= u_last) continue;
-            if (!PAIRS) gd_finish_row<TOut, EPI>(a, m, u, total_of(i), fin[e]);
+            if (!PAIRS) gd_finish_row<TOut, EPI>(a, m, u, total_of(i), fin[e], (size_t)(part * a.part_stride));
             else gd_finish_pair<TOut, EPI>(a, m, u, total_of(i), total_of(i + 8), fin[e]);
         }
     };
@@ -751,15 +758,19 @@ int llms_gemm_decode_fits(int M, int K) {
 // or neither: no rotation), 3 residual (residual[M, N] += X W^T in place, bfloat16; C unused).
 // norm_weight (bfloat16 [K]) given: the rows of X are replaced by RMSNorm(X) * norm_weight with `eps` on the way in.
 // workgroups: how many share the work out (the caller passes the number of compute units).
+// k_parts > 1 (17 to 64 rows, plain 32-bit sums): K is shared out as well, to k_parts sets of workgroups, and C is
+// [k_parts][M][ldc]: partial sums for a norm to add up.
 int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* X, int ldx, const void* W,
                      const void* bias, const void* norm_weight, float eps, int M, int N, int K, int inter,
                      int n_heads, int n_kv_heads, int head_dim, int block_size, const float* inv_freq,
                      const float* angles, const int* positions, const int* slots, void* k_pool, void* v_pool,
-                     void* residual, int ldr, int workgroups, hipStream_t stream) {
+                     void* residual, int ldr, int workgroups, int k_parts, hipStream_t stream) {
     LLMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_decode: needs 1 <= M <= 64 and positive sizes");
     LLMS_REQUIRE((long long)N * K < (1ll << 30) && (long long)M * ldx < (1ll << 30), "gemm_decode: operands of 2 GB or more");
     const int x_rows = M <= 8 ? 8 : 16, x_pitch = (K + GD_KC - 1) / GD_KC * (GD_KC * 2) + 16;
-    LLMS_REQUIRE(llms_gemm_decode_fits(M, K), "gemm_decode: the rows of X do not fit a compute unit (see llms_gemm_decode_fits)");
+    LLMS_REQUIRE(k_parts >= 1 && k_parts <= 16, "gemm_decode: k_parts must be 1..16");
+    const int k_each = k_parts == 1 ? K : ((K + GD_KC - 1) / GD_KC + k_parts - 1) / k_parts * GD_KC;  // columns of a part
+    LLMS_REQUIRE(llms_gemm_decode_fits(M, k_each), "gemm_decode: the rows of X do not fit a compute unit (see llms_gemm_decode_fits)");
     LLMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "gemm_decode: K and the row stride of X must be multiples of 8");
     LLMS_REQUIRE(M <= 32 || norm_weight == nullptr, "gemm_decode: more than 32 rows are taken as they are (no norm on the way in)");
     LLMS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)norm_weight % 16) == 0,
@@ -769,7 +780,7 @@ int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* 
     LLMS_REQUIRE(workgroups > 0 && workgroups <= 4096, "gemm_decode: bad number of workgroups");
     DecodeGemmArgs a = {(const bf16*)W, (const bf16*)X, (const bf16*)bias, (const bf16*)norm_weight, eps, C, ldc, ldx,
                         M, N, K, 0, 0, 0, 0, x_rows, x_pitch, inter, n_heads, n_kv_heads, head_dim, block_size, 0u, -1, inv_freq, angles, positions, slots,
-                        (bf16*)k_pool, (bf16*)v_pool, (bf16*)residual, ldr};
+                        (bf16*)k_pool, (bf16*)v_pool, (bf16*)residual, ldr, K, 1, K, 0, 0};
     if (epilogue == GD_PLAIN) {
         LLMS_REQUIRE(C != nullptr && ldc >= N, "gemm_decode: bad output");
         a.units = N;
@@ -793,11 +804,22 @@ int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* 
         a.half_inv = (unsigned)(((1ull << 32) + head_dim / 2 - 1) / (head_dim / 2));
         a.bs_shift = block_size > 0 && (block_size & (block_size - 1)) == 0 ? __builtin_ctz((unsigned)block_size) : -1;
     }
-    const unsigned grid = (unsigned)(workgroups < a.units ? workgroups : a.units);
-    a.units_each = a.units / (int)grid;
-    a.units_more = a.units % (int)grid;
+    if (k_parts > 1) {  // C is [k_parts][M][ldc] floats
+        LLMS_REQUIRE(M > 16 && epilogue == GD_PLAIN && out_dtype == 0 && bias == nullptr && norm_weight == nullptr,
+                     "gemm_decode: K is shared out only for 17 to 64 rows with plain 32-bit sums (no bias, no norm)");
+        a.k_parts = k_parts;
+        a.k_each = k_each;
+        LLMS_REQUIRE((long long)(k_parts - 1) * a.k_each < K, "gemm_decode: more parts than K has chunks of 128");
+        a.part_stride = (long long)M * ldc;
+    }
+    const int per_part = workgroups / k_parts > 0 ? workgroups / k_parts : 1;
+    const unsigned wgs = (unsigned)(per_part < a.units ? per_part : a.units);  // workgroups that share the units out
+    const unsigned grid = wgs * (unsigned)k_parts;
+    a.wgs_per_part = (int)wgs;
+    a.units_each = a.units / (int)wgs;
+    a.units_more = a.units % (int)wgs;
     const int most = a.units_each + (a.units_more ? 1 : 0);  // units of the largest share
-    const int chunks = (K + GD_KC - 1) / GD_KC;
+    const int chunks = (a.k_each + GD_KC - 1) / GD_KC;
     const unsigned lds = GD_LDS_TILES + GD_LDS_SQ + (unsigned)(x_rows * x_pitch);
     int rc;
     if (M > 16) {  // tiles of 16 rows (8 units with partners), 8 waves

@@ -420,6 +420,26 @@ def gemm_decode_fits(m: int, k: int) -> bool:
     return (8 if m <= 8 else 16) * (-(-k // 128) * 256 + 16) <= _GEMM_DECODE_LDS_FOR_ROWS
 
 
+GEMM_DECODE_ROWS_K = 2 * 8 * 128  # 17 to 64 rows: what 8 waves hold of a row in registers
+
+
+def gemm_decode_k_parts(m: int, k: int) -> int:
+    """Into how many parts ops.gemm_decode best shares K out when it leaves partial sums for 17 to 64 rows (0: it
+    cannot take them).  At least what makes a part fit the registers; beyond that about 1,408 columns a part, a compute
+    unit then pulls as little of X as of its weights (measured on 2048 x 2048, 2048 x 5632 and 4096 x 4096 at 24 to 64
+    rows: 2, 4 and 4 parts), and a count that divides K's chunks of 128 evenly where one is near."""
+    if not 16 < m <= GEMM_DECODE_MAX_ROWS or k <= 0:
+        return 0
+    chunks = -(-k // 128)
+    first = max(-(-k // GEMM_DECODE_ROWS_K), -(-k // 1408))
+    if first > 8:
+        return 0
+    for parts in range(first, min(8, first + 2) + 1):
+        if chunks % parts == 0:
+            return parts
+    return first if (first - 1) * (-(-chunks // first) * 128) < k else 0
+
+
 def gemm_decode_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether ops.gemm_decode takes x [M, K] against w [N, K]."""
     return x.dtype == torch.bfloat16 and gemm_decode_fits(x.shape[0], x.shape[1]) and gemm_bf16_supported(x, w)
@@ -427,7 +447,7 @@ def gemm_decode_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None, *,
                 norm: tuple[torch.Tensor, float] | None = None, swiglu: bool = False, rope: dict | None = None,
-                residual: torch.Tensor | None = None) -> torch.Tensor:
+                residual: torch.Tensor | None = None, k_parts: int = 1) -> torch.Tensor:
     """The product for up to 64 bfloat16 rows with one workgroup per compute unit, and what surrounds it fused in.
 
     norm = (weight [K], eps): the rows of x are replaced by RMSNorm(x) * weight on the way in (up to 32 rows).
@@ -438,7 +458,10 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
                are stored at the tokens' cache slots.  `angles` (rotary_angles(positions, inv_freq), float32
                [M, head_dim / 2, 2]) saves the kernel the sines and cosines; the result is the same to the bit.
     residual:  residual[M, N] += x w^T (+ bias) in place (32-bit sum of the rounded product and the row, rounded
-               once); `out` is not used and `residual` is returned."""
+               once); `out` is not used and `residual` is returned.
+    k_parts > 1 (17 to 64 rows, plain, no bias, no norm): K is shared out to that many sets of workgroups and `out` is
+               float32 [k_parts, M, N], the parts' sums, for a norm to add up (gemm_decode_k_parts says how many
+               parts a K needs)."""
     dev = _dev(out, x, w, bias, residual, norm[0] if norm else None)
     if x.dim() != 2 or x.stride(1) != 1:
         raise ValueError("x must be 2-d with unit inner stride")
@@ -447,9 +470,17 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
     n = w.shape[0]
     if not 0 < m <= GEMM_DECODE_MAX_ROWS:
         raise ValueError(f"gemm_decode takes 1..{GEMM_DECODE_MAX_ROWS} rows")
-    if not gemm_decode_fits(m, k):
+    if k_parts != 1:
+        if not 1 < k_parts <= 16 or m <= 16 or bias is not None or norm is not None or swiglu or rope is not None \
+                or residual is not None:
+            raise ValueError("K is shared out (k_parts 2..16) only for 17 to 64 rows with the plain epilogue, no bias, no norm")
+        if (k_parts - 1) * (-(-(-(-k // 128)) // k_parts) * 128) >= k:
+            raise ValueError(f"K = {k} has too few chunks of 128 for {k_parts} parts")
+        if out is None or out.dtype != torch.float32 or tuple(out.shape) != (k_parts, m, n) or not out.is_contiguous():
+            raise ValueError(f"out must be a contiguous float32 [{k_parts}, {m}, {n}] tensor")
+    if not gemm_decode_fits(m, -(-(-(-k // 128)) // k_parts) * 128 if k_parts > 1 else k):
         raise ValueError(f"gemm_decode keeps the rows of x in a compute unit: {m} rows of K = {k} do not fit (K up to "
-                         f"{GEMM_DECODE_MAX_K} with up to 8 rows, 2,944 with up to 16, 2,048 beyond)")
+                         f"{GEMM_DECODE_MAX_K} with up to 8 rows, 2,944 with up to 16, 2,048 beyond, per part)")
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ValueError("gemm_decode takes bfloat16 operands")
     if not gemm_bf16_supported(x, w):
@@ -498,18 +529,19 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
                 or residual.dtype != torch.bfloat16):
             raise ValueError(f"residual must be a bfloat16 [{m}, {n}] tensor with unit inner stride")
         epilogue = 3
-    if epilogue != 3:
+    if epilogue != 3 and k_parts == 1:
         if out is None or out.dim() != 2 or out.stride(1) != 1 or tuple(out.shape) != (m, cols):
             raise ValueError(f"out must be 2-d [{m}, {cols}] with unit inner stride")
         if out.dtype != torch.bfloat16 and not (epilogue == 0 and out.dtype == torch.float32):
             raise ValueError("gemm_decode stores bfloat16 (the plain epilogue also float32)")
     _check(load("gemm_decode").llms_gemm_decode(
         c_int(1 if epilogue == 3 else _code(out)), c_int(epilogue), _ptr(None if epilogue == 3 else out),
-        c_int(0 if epilogue == 3 else out.stride(0)), _ptr(x), c_int(x.stride(0)), _ptr(w), _ptr(bias),
+        c_int(0 if epilogue == 3 else out.stride(-2)), _ptr(x), c_int(x.stride(0)), _ptr(w), _ptr(bias),
         _ptr(norm_weight), c_float(eps), c_int(m), c_int(n), c_int(k), c_int(inter), c_int(r["n_heads"]),
         c_int(r["n_kv_heads"]), c_int(r["head_dim"]), c_int(r["block_size"]), _ptr(r["inv_freq"]), _ptr(r["angles"]), _ptr(r["positions"]),
         _ptr(r["slots"]), _ptr(r["k_pool"]), _ptr(r["v_pool"]), _ptr(residual),
-        c_int(residual.stride(0) if residual is not None else 0), c_int(compute_units(dev)), _stream(dev)), "gemm_decode")
+        c_int(residual.stride(0) if residual is not None else 0), c_int(compute_units(dev)), c_int(k_parts),
+        _stream(dev)), "gemm_decode")
     return residual if epilogue == 3 else out
 
 

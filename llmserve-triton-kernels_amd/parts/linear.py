@@ -9,8 +9,9 @@ bfloat16, few rows otherwise: the hand-written kernel that streams the weight on
   (ops.gemm_stream); it takes up to 64 rows, one workgroup per 16 rows and 16 weight rows, so
   beyond 16 rows the weights are re-read from L2 and it only pays for the smaller matrices.
   A product whose result goes to a norm may be left as 32-bit partial sums over shares of K, which
-  the norm kernel adds up (linear_partial_sums): that fills the chip for a short, wide weight, and
-  for 17 to 64 rows it is ops.gemm_slices, which keeps a slice of all rows in LDS.
+  the norm kernel adds up (linear_partial_sums): that fills the chip for a short, wide weight; for 17 to
+  64 rows it is ops.gemm_decode with K shared out to 2 to 8 sets of workgroups (ops.gemm_slices, which
+  keeps a slice of all rows in LDS, where that kernel is switched off).
 bfloat16, more rows: the library's matrix product (hipBLASLt through torch.mm), which is
   where the reference's engine uses a library too (nn.Linear, src/llmserve/model/llama.py:64-67);
   sums are 32-bit, the result bfloat16 or, for logits, float32.
@@ -106,6 +107,11 @@ def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor):
     m = x.shape[0]
     if not (SPLIT_K and x.dtype == torch.bfloat16 and ops.gemm_bf16_supported(x, weight)):
         return None
+    if STREAM_ROWS < m <= STREAM_MAX_ROWS and DECODE_KERNEL:
+        k_parts = ops.gemm_decode_k_parts(m, weight.shape[1])
+        if k_parts > 1:  # the rows in registers, K shared out to a few sets of workgroups
+            parts = torch.empty((k_parts, m, weight.shape[0]), dtype=torch.float32, device=x.device)
+            return PartialSums(ops.gemm_decode(parts, x, weight, k_parts=k_parts), x.dtype)
     if slices_pay(m, weight):
         parts = torch.empty((-(-weight.shape[1] // ops.SLICE_K), m, weight.shape[0]), dtype=torch.float32, device=x.device)
         return PartialSums(ops.gemm_slices(parts, x, weight), x.dtype)

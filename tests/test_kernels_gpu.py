@@ -365,6 +365,26 @@ def test_gemm_decode_plain(m, n, k):
     assert torch.equal(ops().gemm_decode(torch.empty(m, n, dtype=torch.bfloat16, device=DEV), wide[:, :k], w.to(DEV)), out)
 
 
+@pytest.mark.parametrize("m,n,k,parts", [(64, 2048, 5632, 3), (17, 333, 2048 + 8, 2), (33, 4096, 11008, 6), (40, 100, 520, 5),
+                                         (24, 2048, 5632, 3), (64, 48, 256, 2)])
+def test_gemm_decode_shares_k_out_for_many_rows(m, n, k, parts):
+    """17 to 64 rows against a weight whose K does not fit the registers: partial sums per part of K."""
+    x, w = rnd(m, k, seed=61).bfloat16(), rnd(n, k, seed=62, scale=0.2).bfloat16()
+    ref = x.double() @ w.double().t()
+    out = ops().gemm_decode(torch.full((parts, m, n), float("nan"), device=DEV), x.to(DEV), w.to(DEV), k_parts=parts)
+    assert (out.sum(0).cpu().double() - ref).abs().max() <= 1e-5 * float(ref.abs().max()) + 1e-5
+    each = -(-(-(-k // 128)) // parts) * 128  # the first part alone is the product over its columns
+    first = x[:, :each].double() @ w[:, :each].double().t()
+    assert (out[0].cpu().double() - first).abs().max() <= 1e-5 * float(first.abs().max()) + 1e-5
+    best = ops().gemm_decode_k_parts(m, k)  # the number of parts the parts of a model would ask for: it has to work too
+    assert 1 <= best <= 8
+    if best > 1:
+        again = ops().gemm_decode(torch.empty(best, m, n, device=DEV), x.to(DEV), w.to(DEV), k_parts=best)
+        assert (again.sum(0).cpu().double() - ref).abs().max() <= 1e-5 * float(ref.abs().max()) + 1e-5
+    with pytest.raises(ValueError, match="shared out"):
+        ops().gemm_decode(torch.empty(parts, 8, n, device=DEV), x[:8].to(DEV), w.to(DEV), k_parts=parts)
+
+
 def test_gemm_decode_refuses_what_it_cannot_take():
     x, w = rnd(65, 64).bfloat16().to(DEV), rnd(32, 64).bfloat16().to(DEV)
     with pytest.raises(ValueError, match="1..64"):
