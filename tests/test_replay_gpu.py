@@ -216,23 +216,13 @@ def test_replay_at_full_layer_sizes(wide_model_dir, dtype_name, mode, monkeypatc
         assert any(not waves and splits > 1 for waves, splits in shared_out), "no portion shared its keys out"
 
 
-@pytest.mark.parametrize("use_graphs", [True, False], ids=["graphs", "launches"])
-@pytest.mark.parametrize("live", [20, 48])
-@pytest.mark.parametrize("dtype_name", list(DTYPES))
-def test_many_live_requests_at_full_layer_sizes(wide_model_dir, dtype_name, live, use_graphs):
-    """17 to 64 rows at the widths of real models: the products for that many rows (a slice of all rows in LDS for
-    o_proj and down_proj, the library's product and the activation kernel for gate and up, the rotary epilogue over
-    several blocks of rows, the library's head), decode graphs for 32 and 64 requests.  Prompts come in portions
-    beside decoded tokens of others; then all requests decode side by side."""
-    model_dir, cfg = wide_model_dir
-    if cfg["hidden_size"] > 4096:
-        pytest.skip("the 1.1B and 7B widths cover the arrangement; the 70B width is replayed with four requests above")
+def many_live_trace(cfg, live):
+    """Portions of some prompts beside decoded tokens of requests whose prompt is in, until every request has at most
+    5 tokens to go; then all of them decode side by side."""
     import random
 
     rng = random.Random(live)
     seqs = {f"m{i}": traces.random_ids(cfg["vocab_size"], rng.randint(12, 70), 3000 + i) for i in range(live)}
-    # portions of some prompts beside decoded tokens of requests whose prompt is in, until every request has at
-    # most 5 tokens to go; then all of them decode side by side
     pos = {rid: 0 for rid in seqs}
     steps = []
 
@@ -260,9 +250,52 @@ def test_many_live_requests_at_full_layer_sizes(wide_model_dir, dtype_name, live
         step_of([bring(rid, 1) for rid, ids in seqs.items() if pos[rid] < len(ids)])
     assert any(len(rec["entries"]) == live and all(len(e["tokens"]) == 1 for e in rec["entries"]) for rec in steps)
     assert any(len(rec["entries"]) > 16 and any(len(e["tokens"]) > 1 for e in rec["entries"]) for rec in steps) or live <= 20
+    return seqs, steps
+
+
+@pytest.mark.parametrize("use_graphs", [True, False], ids=["graphs", "launches"])
+@pytest.mark.parametrize("live", [20, 48])
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_many_live_requests_at_full_layer_sizes(wide_model_dir, dtype_name, live, use_graphs):
+    """17 to 64 rows at the widths of real models: the products for that many rows (the rows in registers, with the
+    activation or the rotation and cache store behind them, K shared out where the sums go to a norm; the library's
+    product and the activation kernel where K is too long for that), decode graphs for 32 and 64 requests.  Prompts
+    come in portions beside decoded tokens of others; then all requests decode side by side."""
+    model_dir, cfg = wide_model_dir
+    if cfg["hidden_size"] > 4096:
+        pytest.skip("the 1.1B and 7B widths cover the arrangement; the 70B width is replayed with four requests above")
+    seqs, steps = many_live_trace(cfg, live)
     num_blocks = traces.tokens_needed(steps, round_to=16) // 16
     outputs = replay_in_process(model_dir, dtype_name, steps, 16, num_blocks, use_graphs=use_graphs, max_seqs=live)
     check_against_plain(model_dir, dtype_name, seqs, steps, outputs)
+
+
+@pytest.mark.parametrize("live", [4, 20, 48])
+def test_the_kernels_behind_the_switches_at_full_layer_sizes(wide_model_dir, live, monkeypatch):
+    """The same replays with the decode product that has one workgroup per compute unit switched off
+    (LLMSERVE_DECODE_GEMM=0: a workgroup per 16 weight rows, slices of K in LDS for 17 to 64 rows, norms as kernels of
+    their own) and the shares of a split decode attention added up by the merge kernel (LLMSERVE_ATTN_MERGE=kernel)."""
+    from llmserve.ops import library as ops
+    from llmserve.parts import linear
+
+    model_dir, cfg = wide_model_dir
+    if cfg["hidden_size"] > 4096:
+        pytest.skip("the 1.1B and 7B widths cover the arrangement")
+    monkeypatch.setattr(linear, "DECODE_KERNEL", False)
+    monkeypatch.setattr(ops, "MERGE_BY_KERNEL", True)
+    used = set()
+    for name in ("gemm_stream", "gemm_slices", "gemm_decode"):
+        original = getattr(ops, name)
+        monkeypatch.setattr(ops, name, (lambda name, original: lambda *a, **kw: (used.add(name), original(*a, **kw))[1])(name, original))
+    seqs, steps = many_live_trace(cfg, live) if live > 4 else (None, None)
+    if live <= 4:
+        seqs = {f"s{i}": traces.random_ids(cfg["vocab_size"], 40 + 9 * i, 4100 + i) for i in range(live)}
+        steps = traces.mixed(seqs, seed=5, live_max=4, tail=6)
+    num_blocks = traces.tokens_needed(steps, round_to=16) // 16
+    outputs = replay_in_process(model_dir, "bfloat16", steps, 16, num_blocks, max_seqs=max(live, 4))
+    check_against_plain(model_dir, "bfloat16", seqs, steps, outputs)
+    assert "gemm_stream" in used and "gemm_decode" not in used
+    assert live <= 16 or cfg["hidden_size"] > 2048 or "gemm_slices" in used  # (it takes weights of up to 24 MB)
 
 
 @pytest.mark.parametrize("seed", [1, 2, 3, 4])
