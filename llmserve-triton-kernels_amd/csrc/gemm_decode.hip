@@ -463,14 +463,17 @@ __global__ __launch_bounds__(GD_NW* LLMS_WAVE) void gemm_decode_kernel(const Dec
 // layout (64 rows are full load instructions there), and every chunk of weights it stages meets RB blocks of rows:
 // RB matrix instructions per fragment read from LDS.  X enters a compute unit once, as much as the unit's share of
 // a large weight; with one workgroup per block of 16 rows it would enter four times as many workgroups.
+// With 16 waves and one block of rows the same kernel takes 9 to 16 rows whose K is too long for LDS (up to 6,144: three
+// chunks of 16 rows are 48 of a wave's 128 registers).
 #define GR_NW 8
 
-template <typename TOut, int EPI, int XC, int RB, int NT, bool NORM>
-__global__ __launch_bounds__(GR_NW* LLMS_WAVE) void gemm_decode_rows_kernel(const DecodeGemmArgs a) {
+template <typename TOut, int EPI, int XC, int RB, int NT, bool NORM, int NW = GR_NW, int LPI = 4>
+__global__ __launch_bounds__(NW* LLMS_WAVE) void gemm_decode_rows_kernel(const DecodeGemmArgs a) {
     static_assert(!NORM || RB <= 2, "the norm's registers fit beside up to 32 rows of X");
-    constexpr int NW = GR_NW, LPI = 4;
+    static_assert(NW == GR_NW || (NW == 16 && RB == 1), "16 waves have registers for one block of rows");
     constexpr bool PAIRS = EPI == GD_SWIGLU || EPI == GD_ROPE_QKV;
-    constexpr int UPT = PAIRS ? 8 : 16;  // units per tile
+    static_assert(!PAIRS || LPI == 4, "units with partners fill rows 0..7 and 8..15");
+    constexpr int UPT = PAIRS ? 8 : 4 * LPI;  // units per tile (rows of the tile beyond them hold whatever lies in LDS)
     constexpr int ITEMS = NT * XC;
     constexpr int RING = ITEMS % 2 == 0 ? 2 : (ITEMS < 3 ? ITEMS : 3);  // (1, 2, 3, 4, 6 items: 1, 2, 3, 2, 2)
     static_assert(ITEMS % RING == 0, "the ring must go round a whole number of times per group");
@@ -696,8 +699,44 @@ static void gd_launch_rows_two_chunks(int tiles, unsigned grid, DecodeGemmArgs& 
 }
 #undef GR_GO
 
+// 9 to 16 rows whose K does not fit LDS: 16 waves, two or three chunks each.  LPI = 2: tiles of 8 weight rows, for a
+// share whose last tile of 16 would be half empty (two load instructions less per chunk, and with three chunks a group
+// of one tile whose ring of three fits the registers).
+template <typename TOut, int EPI, bool NORM, int LPI>
+static void gd_launch_rows_16_waves(int chunks, int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
+#define GR_GO16(XC, NT)                                                                                          \
+    do {                                                                                                         \
+        a.groups = (tiles + NT - 1) / NT;                                                                        \
+        gemm_decode_rows_kernel<TOut, EPI, XC, 1, NT, NORM, 16, LPI><<<grid, 16 * LLMS_WAVE, 0, stream>>>(a);    \
+    } while (0)
+    if (chunks <= 32) {
+        if (tiles == 1) GR_GO16(2, 1);
+        else GR_GO16(2, 2);
+    } else {
+        if constexpr (LPI == 2) {
+            if (tiles == 1) {
+                GR_GO16(3, 1);
+                return;
+            }
+        }
+        GR_GO16(3, 2);  // (a ring of three whole chunks beside three chunks of X would not fit the registers: two tiles
+                        // a group, of which the second may not exist, and a ring of two)
+    }
+#undef GR_GO16
+}
+
 template <typename TOut, int EPI>
-static int gd_launch_rows(int chunks, int rows, int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
+static int gd_launch_rows(int chunks, int rows, int tiles, bool low, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
+    if (rows <= 16) {
+        if (low) {
+            if constexpr (EPI == GD_PLAIN || EPI == GD_RESIDUAL) {
+                if (a.norm_weight) gd_launch_rows_16_waves<TOut, EPI, true, 2>(chunks, tiles, grid, a, stream);
+                else gd_launch_rows_16_waves<TOut, EPI, false, 2>(chunks, tiles, grid, a, stream);
+            }
+        } else if (a.norm_weight) gd_launch_rows_16_waves<TOut, EPI, true, 4>(chunks, tiles, grid, a, stream);
+        else gd_launch_rows_16_waves<TOut, EPI, false, 4>(chunks, tiles, grid, a, stream);
+        return LLMS_OK;
+    }
     if (a.norm_weight) {  // (up to 32 rows: checked by the caller)
         if (chunks <= GR_NW) gd_launch_rows_one_chunk<TOut, EPI, 2, true>(tiles, grid, a, stream);
         else gd_launch_rows_two_chunks<TOut, EPI, 2, true>(tiles, grid, a, stream);
@@ -744,12 +783,17 @@ static int gd_launch(int chunks, int tiles, unsigned grid, unsigned lds_bytes, D
 
 extern "C" {
 
-// Whether M rows of K elements fit: up to 16 rows stay in LDS beside the tiles (8 of them up to 8 rows, else 16);
-// 17 to 64 rows in the registers of 8 waves, two chunks of 128 each.
+// Whether up to 16 rows of K elements stay in LDS beside the tiles (8 of them up to 8 rows, else 16).
+static bool gd_rows_fit_lds(int M, int K) {
+    return (M <= 8 ? 8 : 16) * ((K + GD_KC - 1) / GD_KC * (GD_KC * 2) + 16) <= GD_LDS_X_MAX;
+}
+
+// Whether M rows of K elements fit: up to 16 rows in LDS, or where K is too long for that in the registers of 16
+// waves, three chunks of 128 each; 17 to 64 rows in the registers of 8 waves, two chunks each.
 int llms_gemm_decode_fits(int M, int K) {
     if (M <= 0 || M > 64 || K <= 0 || K > GD_MAX_K) return 0;
     if (M > 16) return K <= 2 * GR_NW * GD_KC;
-    return (M <= 8 ? 8 : 16) * ((K + GD_KC - 1) / GD_KC * (GD_KC * 2) + 16) <= GD_LDS_X_MAX;
+    return 1;
 }
 
 // epilogue: 0 plain (C [M,N] + bias; out_dtype 0 float32, 1 bfloat16), 1 gated (W = [gate; up] of `inter` rows each,
@@ -822,13 +866,16 @@ int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* 
     const int chunks = (a.k_each + GD_KC - 1) / GD_KC;
     const unsigned lds = GD_LDS_TILES + GD_LDS_SQ + (unsigned)(x_rows * x_pitch);
     int rc;
-    if (M > 16) {  // tiles of 16 rows (8 units with partners), 8 waves
-        const int tiles = epilogue == GD_SWIGLU || epilogue == GD_ROPE_QKV ? (most + 7) / 8 : (most + 15) / 16;
-        if (epilogue == GD_SWIGLU) rc = gd_launch_rows<bf16, GD_SWIGLU>(chunks, M, tiles, grid, a, stream);
-        else if (epilogue == GD_ROPE_QKV) rc = gd_launch_rows<bf16, GD_ROPE_QKV>(chunks, M, tiles, grid, a, stream);
-        else if (epilogue == GD_RESIDUAL) rc = gd_launch_rows<bf16, GD_RESIDUAL>(chunks, M, tiles, grid, a, stream);
-        else if (out_dtype == 0) rc = gd_launch_rows<float, GD_PLAIN>(chunks, M, tiles, grid, a, stream);
-        else rc = gd_launch_rows<bf16, GD_PLAIN>(chunks, M, tiles, grid, a, stream);
+    if (M > 16 || !gd_rows_fit_lds(M, K)) {  // the rows in registers: tiles of 16 weight rows (8 units with partners)
+        const bool pairs = epilogue == GD_SWIGLU || epilogue == GD_ROPE_QKV;
+        // up to 16 rows, units without partners: tiles of 8 weight rows where the last tile of 16 would be half empty
+        const bool low = M <= 16 && !pairs && ((most + 7) / 8) % 2 == 1;
+        const int tiles = pairs || low ? (most + 7) / 8 : (most + 15) / 16;
+        if (epilogue == GD_SWIGLU) rc = gd_launch_rows<bf16, GD_SWIGLU>(chunks, M, tiles, low, grid, a, stream);
+        else if (epilogue == GD_ROPE_QKV) rc = gd_launch_rows<bf16, GD_ROPE_QKV>(chunks, M, tiles, low, grid, a, stream);
+        else if (epilogue == GD_RESIDUAL) rc = gd_launch_rows<bf16, GD_RESIDUAL>(chunks, M, tiles, low, grid, a, stream);
+        else if (out_dtype == 0) rc = gd_launch_rows<float, GD_PLAIN>(chunks, M, tiles, low, grid, a, stream);
+        else rc = gd_launch_rows<bf16, GD_PLAIN>(chunks, M, tiles, low, grid, a, stream);
     } else if (epilogue == GD_SWIGLU) rc = gd_launch<bf16, GD_SWIGLU, 4>(chunks, (most + 7) / 8, grid, lds, a, stream);
     else if (epilogue == GD_ROPE_QKV) rc = gd_launch<bf16, GD_ROPE_QKV, 4>(chunks, (most + 7) / 8, grid, lds, a, stream);
     else {

@@ -407,17 +407,15 @@ def compute_units(dev: torch.device) -> int:
 GEMM_DECODE_MAX_ROWS = 64
 GEMM_DECODE_NORM_ROWS = 32  # up to here the kernel can norm its rows on the way in (beyond, their registers are full)
 GEMM_DECODE_MAX_K = 16 * 3 * 128  # 16 waves with up to three chunks of 128 each
-_GEMM_DECODE_LDS_FOR_ROWS = 160 * 1024 - 16 * 4096 - 1024  # what the waves' tiles leave of a compute unit's LDS
 
 
 def gemm_decode_fits(m: int, k: int) -> bool:
-    """Whether m rows of k elements fit ops.gemm_decode: up to 16 rows stay in LDS (8 of them up to 8 rows, else
-    16); 17 to 64 rows in the registers of 8 waves, two chunks of 128 each (k up to 2,048)."""
+    """Whether m rows of k elements fit ops.gemm_decode: up to 16 rows stay in LDS or, where K is too long for that, in
+    the registers of 16 waves (k up to 6,144 either way); 17 to 64 rows in the registers of 8 waves, two chunks of 128
+    each (k up to 2,048)."""
     if not (0 < m <= GEMM_DECODE_MAX_ROWS and 0 < k <= GEMM_DECODE_MAX_K):
         return False
-    if m > 16:
-        return k <= 2 * 8 * 128
-    return (8 if m <= 8 else 16) * (-(-k // 128) * 256 + 16) <= _GEMM_DECODE_LDS_FOR_ROWS
+    return m <= 16 or k <= 2 * 8 * 128
 
 
 GEMM_DECODE_ROWS_K = 2 * 8 * 128  # 17 to 64 rows: what 8 waves hold of a row in registers
@@ -480,7 +478,7 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
             raise ValueError(f"out must be a contiguous float32 [{k_parts}, {m}, {n}] tensor")
     if not gemm_decode_fits(m, -(-(-(-k // 128)) // k_parts) * 128 if k_parts > 1 else k):
         raise ValueError(f"gemm_decode keeps the rows of x in a compute unit: {m} rows of K = {k} do not fit (K up to "
-                         f"{GEMM_DECODE_MAX_K} with up to 8 rows, 2,944 with up to 16, 2,048 beyond, per part)")
+                         f"{GEMM_DECODE_MAX_K} with up to 16 rows, 2,048 beyond, per part)")
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ValueError("gemm_decode takes bfloat16 operands")
     if not gemm_bf16_supported(x, w):
