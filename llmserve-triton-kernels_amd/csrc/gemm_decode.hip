@@ -1,5 +1,8 @@
-// bfloat16 matrix product for up to 16 rows (decoding) with one workgroup per compute unit:
+// bfloat16 matrix product for up to 64 rows (decoding) with one workgroup per compute unit:
 //   C[M,N] = f(X)[M,K] * W[N,K]^T, 32-bit sums on the gfx950 matrix cores.
+// Two kernels: gemm_decode_kernel (up to 16 rows, which stay in LDS; described first) and gemm_decode_rows_kernel
+// (the rows in registers: 17 to 64 rows of up to 2,048 columns, 9 to 16 rows whose K is too long for LDS, and K
+// shared out to sets of workgroups that leave partial sums; described where it stands).
 //
 // A decode step is a chain of short launches; what each of them costs beyond the bytes of its weight is what it
 // does before its first load is out, the rows of X that every workgroup pulls in, and every launch that only
@@ -459,10 +462,12 @@ __global__ __launch_bounds__(GD_NW* LLMS_WAVE) void gemm_decode_kernel(const Dec
 }
 
 // 17 to 64 rows of X (RB blocks of 16): the same sharing out of weight rows and of K, with 8 waves that have
-// twice the registers.  A wave keeps its chunks of all rows of X in registers, loaded straight in the operand
-// layout (64 rows are full load instructions there), and every chunk of weights it stages meets RB blocks of rows:
-// RB matrix instructions per fragment read from LDS.  X enters a compute unit once, as much as the unit's share of
-// a large weight; with one workgroup per block of 16 rows it would enter four times as many workgroups.
+// twice the registers.  A wave keeps its chunks of all rows of X in registers (asked for as whole lines, then
+// turned into the operand layout through the wave's LDS tile), and every chunk of weights it stages meets RB blocks
+// of rows: RB matrix instructions per fragment read from LDS.  X enters a compute unit once, as much as the unit's
+// share of a large weight; with one workgroup per block of 16 rows it would enter four times as many workgroups.
+// Where the sums go to a norm (plain 32-bit output), K may be shared out as well: k_parts sets of workgroups, each
+// with all of N and a part of K, leave one array of partial sums each, and a compute unit pulls 1/k_parts of X.
 // With 16 waves and one block of rows the same kernel takes 9 to 16 rows whose K is too long for LDS (up to 6,144: three
 // chunks of 16 rows are 48 of a wave's 128 registers).
 #define GR_NW 8
