@@ -10,7 +10,8 @@ step (`chunked`: the same prompt in portions of 512 tokens, the scheduler cuttin
 `roofline` prices the decode step against HBM bandwidth (every weight it uses read once, plus
 the keys and values of the live requests); `points` holds decode at further batch sizes
 (1, 16, 24, 32, 64: the step grows with the blocks of 16 rows) and, at the default batch, behind
-contexts of 2,048 and 4,096 tokens; `serve` is a short continuous-batching run on the same model
+contexts of 2,048 and 4,096 tokens, and with temperature, top-k and top-p for every request
+instead of greedy (`decode_b8_sampled`); `serve` is a short continuous-batching run on the same model
 (requests with random prompt lengths arriving at once: tokens a second, time to first token,
 inter-token latency); `peak_mib` is the most device memory the process held; `measured_peaks` is
 what this box delivers to a plain device copy and to a large library matrix product, the
