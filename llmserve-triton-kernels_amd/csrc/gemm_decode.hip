@@ -474,7 +474,7 @@ __global__ __launch_bounds__(GD_NW* LLMS_WAVE) void gemm_decode_kernel(const Dec
 
 template <typename TOut, int EPI, int XC, int RB, int NT, bool NORM, int NW = GR_NW, int LPI = 4>
 __global__ __launch_bounds__(NW* LLMS_WAVE) void gemm_decode_rows_kernel(const DecodeGemmArgs a) {
-    static_assert(!NORM || RB <= 2, "the norm's registers fit beside up to 32 rows of X");
+    static_assert(!NORM || RB == 1, "the norm on the way in is for up to 16 rows");
     static_assert(NW == GR_NW || (NW == 16 && RB == 1), "16 waves have registers for one block of rows");
     constexpr bool PAIRS = EPI == GD_SWIGLU || EPI == GD_ROPE_QKV;
     static_assert(!PAIRS || LPI == 4, "units with partners fill rows 0..7 and 8..15");
@@ -686,7 +686,7 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void gemm_decode_rows_kernel(const D
         gemm_decode_rows_kernel<TOut, EPI, XC, RB, NT, NORM><<<grid, GR_NW * LLMS_WAVE, 0, stream>>>(a);   \
     } while (0)
 
-template <typename TOut, int EPI, int RB, bool NORM>
+template <typename TOut, int EPI, int RB, bool NORM = false>
 static void gd_launch_rows_one_chunk(int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
     const int groups = (tiles + 3) / 4, nt = (tiles + groups - 1) / groups;
     if (nt == 1) GR_GO(1, RB, 1);
@@ -695,7 +695,7 @@ static void gd_launch_rows_one_chunk(int tiles, unsigned grid, DecodeGemmArgs& a
     else GR_GO(1, RB, 4);
 }
 
-template <typename TOut, int EPI, int RB, bool NORM>
+template <typename TOut, int EPI, int RB, bool NORM = false>
 static void gd_launch_rows_two_chunks(int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
     if (tiles == 1) GR_GO(2, RB, 1);
     else if constexpr (RB == 4) GR_GO(2, RB, 2);  // (three tiles of 64 rows of two chunks would not fit the registers)
@@ -742,15 +742,12 @@ static int gd_launch_rows(int chunks, int rows, int tiles, bool low, unsigned gr
         else gd_launch_rows_16_waves<TOut, EPI, false, 4>(chunks, tiles, grid, a, stream);
         return LLMS_OK;
     }
-    if (a.norm_weight) {  // (up to 32 rows: checked by the caller)
-        if (chunks <= GR_NW) gd_launch_rows_one_chunk<TOut, EPI, 2, true>(tiles, grid, a, stream);
-        else gd_launch_rows_two_chunks<TOut, EPI, 2, true>(tiles, grid, a, stream);
-    } else if (chunks <= GR_NW) {
-        if (rows <= 32) gd_launch_rows_one_chunk<TOut, EPI, 2, false>(tiles, grid, a, stream);
-        else gd_launch_rows_one_chunk<TOut, EPI, 4, false>(tiles, grid, a, stream);
+    if (chunks <= GR_NW) {  // (no norm on the way in beyond 16 rows: checked by the caller)
+        if (rows <= 32) gd_launch_rows_one_chunk<TOut, EPI, 2>(tiles, grid, a, stream);
+        else gd_launch_rows_one_chunk<TOut, EPI, 4>(tiles, grid, a, stream);
     } else {
-        if (rows <= 32) gd_launch_rows_two_chunks<TOut, EPI, 2, false>(tiles, grid, a, stream);
-        else gd_launch_rows_two_chunks<TOut, EPI, 4, false>(tiles, grid, a, stream);
+        if (rows <= 32) gd_launch_rows_two_chunks<TOut, EPI, 2>(tiles, grid, a, stream);
+        else gd_launch_rows_two_chunks<TOut, EPI, 4>(tiles, grid, a, stream);
     }
     return LLMS_OK;
 }
@@ -821,7 +818,9 @@ int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* 
     const int k_each = k_parts == 1 ? K : ((K + GD_KC - 1) / GD_KC + k_parts - 1) / k_parts * GD_KC;  // columns of a part
     LLMS_REQUIRE(llms_gemm_decode_fits(M, k_each), "gemm_decode: the rows of X do not fit a compute unit (see llms_gemm_decode_fits)");
     LLMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "gemm_decode: K and the row stride of X must be multiples of 8");
-    LLMS_REQUIRE(M <= 32 || norm_weight == nullptr, "gemm_decode: more than 32 rows are taken as they are (no norm on the way in)");
+    // (norming 32 rows in every compute unit was built and measured: 4 microseconds of vector arithmetic in the
+    // prologue, more than the norm kernel it saves)
+    LLMS_REQUIRE(M <= 16 || norm_weight == nullptr, "gemm_decode: more than 16 rows are taken as they are (no norm on the way in)");
     LLMS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)norm_weight % 16) == 0,
                  "gemm_decode: X, W and the norm's weight must be 16-byte aligned");
     LLMS_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm_decode: epilogue must be 0..3");

@@ -405,7 +405,8 @@ def compute_units(dev: torch.device) -> int:
 
 
 GEMM_DECODE_MAX_ROWS = 64
-GEMM_DECODE_NORM_ROWS = 32  # up to here the kernel can norm its rows on the way in (beyond, their registers are full)
+GEMM_DECODE_NORM_ROWS = 16  # up to here the kernel norms its rows on the way in (with more rows that costs a compute
+# unit more vector arithmetic than a norm kernel of its own: measured at 32 rows, 4 microseconds)
 GEMM_DECODE_MAX_K = 16 * 3 * 128  # 16 waves with up to three chunks of 128 each
 
 
@@ -448,7 +449,7 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
                 residual: torch.Tensor | None = None, k_parts: int = 1) -> torch.Tensor:
     """The product for up to 64 bfloat16 rows with one workgroup per compute unit, and what surrounds it fused in.
 
-    norm = (weight [K], eps): the rows of x are replaced by RMSNorm(x) * weight on the way in (up to 32 rows).
+    norm = (weight [K], eps): the rows of x are replaced by RMSNorm(x) * weight on the way in (up to 16 rows).
     plain:     out[M, N] = x w^T (+ bias), bfloat16 or float32.
     swiglu:    w = [gate; up] ([2I, K]); out[M, I] = silu(gate) * up.
     rope = dict(n_heads, n_kv_heads, head_dim, inv_freq | None, positions, slots | None, k_pool, v_pool,

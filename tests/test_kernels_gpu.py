@@ -390,7 +390,7 @@ def test_gemm_decode_refuses_what_it_cannot_take():
     with pytest.raises(ValueError, match="1..64"):
         ops().gemm_decode(torch.empty(65, 32, dtype=torch.bfloat16, device=DEV), x, w)
     with pytest.raises(ValueError, match="taken as they are"):
-        ops().gemm_decode(torch.empty(33, 32, dtype=torch.bfloat16, device=DEV), x[:33], w, norm=(rnd(64).bfloat16().to(DEV), 1e-5))
+        ops().gemm_decode(torch.empty(17, 32, dtype=torch.bfloat16, device=DEV), x[:17], w, norm=(rnd(64).bfloat16().to(DEV), 1e-5))
     for rows, big in ((2, ops().GEMM_DECODE_MAX_K + 8), (9, ops().GEMM_DECODE_MAX_K + 8), (17, 2048 + 8)):
         with pytest.raises(ValueError, match="do not fit"):
             ops().gemm_decode(torch.empty(rows, 32, dtype=torch.bfloat16, device=DEV), rnd(rows, big).bfloat16().to(DEV),
@@ -402,9 +402,8 @@ def test_gemm_decode_refuses_what_it_cannot_take():
 
 
 @pytest.mark.parametrize("m,n,k,eps", [(1, 64, 64, 1e-5), (8, 2560, 2048, 1e-5), (16, 333, 96, 1e-6), (5, 100, 4096, 1e-5),
-                                       (3, 48, 5888 - 8, 1e-6), (13, 200, 2560, 1e-5), (17, 333, 96, 1e-6),
-                                       (32, 2560, 2048, 1e-5), (29, 11264, 2048, 1e-5), (24, 100, 1024 + 8, 1e-6),
-                                       (16, 2560, 4096, 1e-5), (9, 100, 5632, 1e-6)])
+                                       (3, 48, 5888 - 8, 1e-6), (13, 200, 2560, 1e-5), (16, 11264, 2048, 1e-5),
+                                       (16, 2560, 4096, 1e-5), (9, 100, 5632, 1e-6), (12, 333, 3072 + 8, 1e-6)])
 def test_gemm_decode_norms_its_rows_on_the_way_in(m, n, k, eps):
     """RMSNorm in the prologue: the same as the norm kernel followed by the product (the sum of squares is added up
     in another order, so the normed rows may differ by one rounding)."""
