@@ -47,6 +47,7 @@ class StepBatch:
     # what a part has worked out for this step and the same kind of part in later layers can use again (the sines
     # and cosines of the tokens' angles); emptied by the model when a step starts
     shared: dict = field(default_factory=dict)
+    all_rows_wanted: bool = False  # logit_rows is 0, 1, ..., num_tokens - 1 (known on the host: nothing to pick)
 
 
 class BatchUploader:
@@ -138,6 +139,7 @@ def build_batch(layout: StepLayout, tokens: list[list[int]], logit_rows: list[in
         num_tokens=n_tokens, num_seqs=n_seqs, token_ids=view(0, n_tokens), positions=view(1, n_tokens),
         token_seq=view(2, n_tokens), cu_seqlens=view(3, n_seqs + 1), context_lens=view(4, n_seqs),
         state_slots=view(5, n_seqs), logit_rows=view(6, len(logit_rows)), groups=groups,
+        all_rows_wanted=list(logit_rows) == list(range(n_tokens)),
         counts=list(counts), starts=list(starts), state_slot_list=list(layout.state_slots),
         num_decode=num_decode, max_count=max(counts), max_context=max(context),
         max_decode_context=max(context[:num_decode], default=0))
@@ -170,7 +172,8 @@ class StaticDecodeBatch:
         self.batch = StepBatch(
             num_tokens=c, num_seqs=c, token_ids=v(0), positions=v(1), token_seq=v(2), cu_seqlens=v(3),
             context_lens=v(4), state_slots=v(5), logit_rows=v(6), groups=groups, counts=[1] * c, starts=[0] * c,
-            state_slot_list=[0] * c, num_decode=c, max_count=1, max_context=1, max_decode_context=1)
+            state_slot_list=[0] * c, num_decode=c, max_count=1, max_context=1, max_decode_context=1,
+            all_rows_wanted=True)
         # what never changes: one token per request, every row's logits wanted
         h = self._host_view
         h(2)[:] = range(c)

@@ -7,8 +7,8 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .linear import linear
-from .registry import EMBEDDINGS, HEADS, Part
+from .linear import decode_product, linear
+from .registry import EMBEDDINGS, HEADS, DeferredNorm, Part
 from .spec import ParamInfo
 
 
@@ -38,7 +38,7 @@ class LMHead(Part):
     """Parameters: vocab, hidden, tied.  A tied head has no tensor of its own: the model
     hands it the embedding table."""
     graph_safe = True
-
+    accepts_deferred_norm = True  # (when every row's logits are wanted the model hands over the final norm's input)
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
@@ -53,5 +53,12 @@ class LMHead(Part):
     def load(self, tensors):
         self.weight = tensors["weight"].contiguous()
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, h) -> torch.Tensor:
+        if isinstance(h, DeferredNorm):
+            rows, norm = h.residual, h.fused()
+            if norm is not None and rows.shape[0] <= ops.GEMM_DECODE_NORM_ROWS and decode_product(rows, self.weight):
+                h.resolve(None)  # few rows: the product norms them on the way in, and the norm kernel is not launched
+                out = torch.empty((rows.shape[0], self.weight.shape[0]), dtype=torch.float32, device=rows.device)
+                return ops.gemm_decode(out, rows, self.weight, norm=norm)
+            h = h.materialize()
         return linear(h, self.weight, out_dtype=torch.float32)

@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from . import attention, block, embedding, rmsnorm, rope, swiglu  # noqa: F401  (register the built-in parts)
-from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, BuildContext, Part
+from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, BuildContext, DeferredNorm, Part
 from .spec import ModelSpec, ParamInfo
 
 
@@ -105,5 +105,7 @@ class Model:
         rows = batch.logit_rows
         if rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
+        if getattr(batch, "all_rows_wanted", False) and getattr(self.head, "accepts_deferred_norm", False):
+            return self.head.forward(DeferredNorm(self.final_norm, x, delta))  # (no rows to pick: the head may norm them itself)
         h = self.final_norm.norm_rows(x, delta, rows)
         return self.head.forward(h)
