@@ -834,6 +834,7 @@ int llms_gemm_decode(int out_dtype, int epilogue, void* C, int ldc, const void* 
         a.units = N;
     } else if (epilogue == GD_RESIDUAL) {
         LLMS_REQUIRE(residual != nullptr && ldr >= N, "gemm_decode: the residual epilogue needs the residual rows");
+        LLMS_REQUIRE((long long)M * ldr < (1ll << 30), "gemm_decode: residual rows of 2 GB or more");
         a.units = N;
     } else if (epilogue == GD_SWIGLU) {
         LLMS_REQUIRE(C != nullptr && inter > 0 && N == 2 * inter && bias == nullptr && ldc >= inter,
