@@ -698,7 +698,10 @@ static void gd_launch_rows_one_chunk(int tiles, unsigned grid, DecodeGemmArgs& a
 template <typename TOut, int EPI, int RB, bool NORM = false>
 static void gd_launch_rows_two_chunks(int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
     if (tiles == 1) GR_GO(2, RB, 1);
-    else if constexpr (RB == 4) GR_GO(2, RB, 2);  // (three tiles of 64 rows of two chunks would not fit the registers)
+    else if constexpr (RB == 4) {  // (three tiles of 64 rows of two chunks would not fit the registers)
+        if (tiles % 2) GR_GO(2, RB, 1);
+        else GR_GO(2, RB, 2);
+    }
     else if (tiles % 3 == 0 || tiles > 4) GR_GO(2, RB, 3);
     else GR_GO(2, RB, 2);
 }
