@@ -702,7 +702,8 @@ static void gd_launch_rows_two_chunks(int tiles, unsigned grid, DecodeGemmArgs& 
         if (tiles % 2) GR_GO(2, RB, 1);
         else GR_GO(2, RB, 2);
     }
-    else if (tiles % 3 == 0 || tiles > 4) GR_GO(2, RB, 3);
+    // three tiles a group, or two where that leaves fewer tiles that do not exist in the last group
+    else if ((tiles + 2) / 3 * 3 - tiles <= (tiles + 1) / 2 * 2 - tiles) GR_GO(2, RB, 3);
     else GR_GO(2, RB, 2);
 }
 #undef GR_GO
