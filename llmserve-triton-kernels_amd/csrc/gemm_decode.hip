@@ -706,6 +706,15 @@ static void gd_launch_rows_two_chunks(int tiles, unsigned grid, DecodeGemmArgs& 
     else if ((tiles + 2) / 3 * 3 - tiles <= (tiles + 1) / 2 * 2 - tiles) GR_GO(2, RB, 3);
     else GR_GO(2, RB, 2);
 }
+
+// 17 to 32 rows of a longer K (up to 4,096): three or four chunks of two blocks of rows are up to 128 of a wave's 256
+// registers.  Two tiles a group, one where there is only one.
+template <typename TOut, int EPI, int XC>
+static void gd_launch_rows_long_k(int tiles, unsigned grid, DecodeGemmArgs& a, hipStream_t stream) {
+    constexpr bool NORM = false;
+    if (tiles == 1) GR_GO(XC, 2, 1);
+    else GR_GO(XC, 2, 2);
+}
 #undef GR_GO
 
 // 9 to 16 rows whose K does not fit LDS: 16 waves, two or three chunks each.  LPI = 2: tiles of 8 weight rows, for a
@@ -744,6 +753,11 @@ static int gd_launch_rows(int chunks, int rows, int tiles, bool low, unsigned gr
             }
         } else if (a.norm_weight) gd_launch_rows_16_waves<TOut, EPI, true, 4>(chunks, tiles, grid, a, stream);
         else gd_launch_rows_16_waves<TOut, EPI, false, 4>(chunks, tiles, grid, a, stream);
+        return LLMS_OK;
+    }
+    if (chunks > 2 * GR_NW) {  // (17 to 32 rows: checked by the caller)
+        if (chunks <= 3 * GR_NW) gd_launch_rows_long_k<TOut, EPI, 3>(tiles, grid, a, stream);
+        else gd_launch_rows_long_k<TOut, EPI, 4>(tiles, grid, a, stream);
         return LLMS_OK;
     }
     if (chunks <= GR_NW) {  // (no norm on the way in beyond 16 rows: checked by the caller)
@@ -795,10 +809,11 @@ static bool gd_rows_fit_lds(int M, int K) {
 }
 
 // Whether M rows of K elements fit: up to 16 rows in LDS, or where K is too long for that in the registers of 16
-// waves, three chunks of 128 each; 17 to 64 rows in the registers of 8 waves, two chunks each.
+// waves, three chunks of 128 each; 17 to 64 rows in the registers of 8 waves, two chunks each (four up to 32 rows).
 int llms_gemm_decode_fits(int M, int K) {
     if (M <= 0 || M > 64 || K <= 0 || K > GD_MAX_K) return 0;
-    if (M > 16) return K <= 2 * GR_NW * GD_KC;
+    if (M > 32) return K <= 2 * GR_NW * GD_KC;
+    if (M > 16) return K <= 4 * GR_NW * GD_KC;
     return 1;
 }
 

@@ -412,11 +412,11 @@ GEMM_DECODE_MAX_K = 16 * 3 * 128  # 16 waves with up to three chunks of 128 each
 
 def gemm_decode_fits(m: int, k: int) -> bool:
     """Whether m rows of k elements fit ops.gemm_decode: up to 16 rows stay in LDS or, where K is too long for that, in
-    the registers of 16 waves (k up to 6,144 either way); 17 to 64 rows in the registers of 8 waves, two chunks of 128
-    each (k up to 2,048)."""
+    the registers of 16 waves (k up to 6,144 either way); 17 to 64 rows in the registers of 8 waves: four chunks of
+    128 each up to 32 rows (k up to 4,096), two beyond (k up to 2,048)."""
     if not (0 < m <= GEMM_DECODE_MAX_ROWS and 0 < k <= GEMM_DECODE_MAX_K):
         return False
-    return m <= 16 or k <= 2 * 8 * 128
+    return m <= 16 or k <= 2 * 8 * 128 or (m <= 32 and k <= 4 * 8 * 128)
 
 
 GEMM_DECODE_ROWS_K = 2 * 8 * 128  # 17 to 64 rows: what 8 waves hold of a row in registers
@@ -479,7 +479,7 @@ def gemm_decode(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias
             raise ValueError(f"out must be a contiguous float32 [{k_parts}, {m}, {n}] tensor")
     if not gemm_decode_fits(m, -(-(-(-k // 128)) // k_parts) * 128 if k_parts > 1 else k):
         raise ValueError(f"gemm_decode keeps the rows of x in a compute unit: {m} rows of K = {k} do not fit (K up to "
-                         f"{GEMM_DECODE_MAX_K} with up to 16 rows, 2,048 beyond, per part)")
+                         f"{GEMM_DECODE_MAX_K} with up to 16 rows, 4,096 with up to 32, 2,048 beyond, per part)")
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ValueError("gemm_decode takes bfloat16 operands")
     if not gemm_bf16_supported(x, w):

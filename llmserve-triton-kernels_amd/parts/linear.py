@@ -1,7 +1,7 @@
 """y = x W^T (+ b) for the parts: picks the matrix product by dtype and shape.
 
 float32: the 32-bit multiply-add kernel, always (no reduced-precision matrix mode).
-bfloat16, up to 16 rows of up to 6,144 columns, or 17 to 64 rows of up to 2,048 columns:
+bfloat16, up to 16 rows of up to 6,144 columns, 17 to 32 rows of up to 4,096, or 33 to 64 rows of up to 2,048:
   ops.gemm_decode, one workgroup per compute unit, with the activation or the rotation and cache store in
   its epilogue; up to 16 rows it also norms its rows on the way in and adds its result to the residual
   rows where the parts ask for that (decode_product, adds_residual_in_epilogue).

@@ -314,7 +314,7 @@ def test_gemm_stream_gated_epilogue(m, inter, k):
 def test_gemm_stream_rotary_epilogue(nh, nkv, d, bs, theta, bias, m):
     """q/k/v projection with the rotation and the cache store in the epilogue: the same bits as the
     projection followed by the rotation kernel."""
-    k, pages = (4096 if m in (9, 12) else 96), 12  # (9 to 16 rows of a long K are kept in registers, not in LDS)
+    k, pages = (4096 if m in (9, 12, 24) else 96), 12  # (a long K: the rows are kept in registers, not in LDS)
     n = (nh + 2 * nkv) * d
     x, w = rnd(m, k, seed=23).bfloat16().to(DEV), rnd(n, k, seed=24, scale=0.3 if k < 1000 else 0.05).bfloat16().to(DEV)
     b = rnd(n, seed=25).bfloat16().to(DEV) if bias else None
@@ -349,7 +349,8 @@ def test_gemm_stream_rotary_epilogue(nh, nkv, d, bs, theta, bias, m):
 @pytest.mark.parametrize("m,n,k", [(1, 16, 64), (3, 333, 96), (16, 2056, 2048), (7, 100, 5632), (9, 48, 176),
                                    (8, 32000, 2048), (5, 2048, 4096), (8, 24, 5888), (2, 5000, 8), (12, 40, 2944),
                                    (17, 333, 96), (64, 2056, 2048), (33, 32000, 2048), (40, 100, 1024), (48, 50, 176),
-                                   (25, 3000, 1032), (16, 2048, 5632), (9, 333, 3072 - 8), (12, 4100, 4096), (16, 40, 6144)])
+                                   (25, 3000, 1032), (16, 2048, 5632), (9, 333, 3072 - 8), (12, 4100, 4096), (16, 40, 6144),
+                                   (24, 4100, 4096), (32, 100, 3072 - 8), (17, 48, 2048 + 8)])
 def test_gemm_decode_plain(m, n, k):
     x, w, b = rnd(m, k, seed=11).bfloat16(), rnd(n, k, seed=12).bfloat16(), rnd(n, seed=13).bfloat16()
     ref = x.double() @ w.double().t() + b.double()
@@ -391,7 +392,7 @@ def test_gemm_decode_refuses_what_it_cannot_take():
         ops().gemm_decode(torch.empty(65, 32, dtype=torch.bfloat16, device=DEV), x, w)
     with pytest.raises(ValueError, match="taken as they are"):
         ops().gemm_decode(torch.empty(17, 32, dtype=torch.bfloat16, device=DEV), x[:17], w, norm=(rnd(64).bfloat16().to(DEV), 1e-5))
-    for rows, big in ((2, ops().GEMM_DECODE_MAX_K + 8), (9, ops().GEMM_DECODE_MAX_K + 8), (17, 2048 + 8)):
+    for rows, big in ((2, ops().GEMM_DECODE_MAX_K + 8), (9, ops().GEMM_DECODE_MAX_K + 8), (17, 4096 + 8), (33, 2048 + 8)):
         with pytest.raises(ValueError, match="do not fit"):
             ops().gemm_decode(torch.empty(rows, 32, dtype=torch.bfloat16, device=DEV), rnd(rows, big).bfloat16().to(DEV),
                               rnd(32, big).bfloat16().to(DEV))
@@ -425,7 +426,7 @@ def test_gemm_decode_norms_its_rows_on_the_way_in(m, n, k, eps):
 
 @pytest.mark.parametrize("m,inter,k", [(1, 176, 64), (5, 5632, 2048), (16, 256, 96), (8, 1000, 4096), (3, 22, 2048),
                                        (64, 5632, 2048), (17, 176, 64), (37, 1000, 1024), (32, 256, 2048),
-                                       (16, 11008, 4096), (10, 100, 6144 - 8)])
+                                       (16, 11008, 4096), (10, 100, 6144 - 8), (32, 11008, 4096), (20, 50, 2560)])
 def test_gemm_decode_gated_epilogue(m, inter, k):
     """silu(gate) * up in the epilogue: the same bits as the product followed by the activation kernel."""
     x = rnd(m, k, seed=16).bfloat16()
@@ -444,7 +445,7 @@ def test_gemm_decode_gated_epilogue(m, inter, k):
                                                       (5, 5, 128, 16, 1e4, True, 3), (6, 3, 80, 16, 1e6, False, 1),
                                                       (32, 4, 64, 16, 1e4, False, 64), (3, 1, 32, 8, 5e5, True, 33),
                                                       (8, 2, 128, 16, 1e4, True, 20), (32, 8, 128, 16, 1e4, False, 12),
-                                                      (3, 3, 64, 8, 1e4, True, 9)])
+                                                      (3, 3, 64, 8, 1e4, True, 9), (32, 32, 128, 16, 1e4, False, 24)])
 def test_gemm_decode_rotary_epilogue(nh, nkv, d, bs, theta, bias, m):
     """q/k/v projection with the rotation and the cache store in the epilogue: the same bits as the
     projection followed by the rotation kernel."""
@@ -487,7 +488,7 @@ def test_gemm_decode_rotary_epilogue(nh, nkv, d, bs, theta, bias, m):
 @pytest.mark.parametrize("m,n,k,bias", [(1, 64, 64, False), (8, 2048, 2048, False), (8, 2048, 5632, True), (16, 333, 176, True),
                                         (5, 4096, 4096, False), (11, 90, 2900 - 4, True), (64, 2048, 2048, False),
                                         (19, 333, 176, True), (40, 4000, 1024, True), (16, 2048, 5632, False),
-                                        (13, 4096, 4096, True), (9, 50, 3000, False)])
+                                        (13, 4096, 4096, True), (9, 50, 3000, False), (30, 4096, 4096, False)])
 def test_gemm_decode_residual_epilogue(m, n, k, bias):
     """residual += x w^T: the rounded product added to the row in 32-bit and rounded once, as the norm kernel adds a
     delta (same bits as product, then that kernel's residual output)."""
